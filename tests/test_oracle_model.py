@@ -1,0 +1,140 @@
+"""Pins the CPU oracle's model math against independent implementations.
+
+The independent implementation is `transformers.Lfm2ForCausalLM` (random init
+from a config, eager attention); the reference holds the same check at
+`tests/test_lfm25_26b_compat.py:79-104` (atol=rtol=1e-5 in fp32).  Invariants:
+cached decode == full recompute (`tests/test_lfm25_engine.py:109-126`), padded
+chunk prefill == per-prompt prefill incl. a dirty reused cache
+(`tests/test_lfm25_cuda.py:283-313`).
+"""
+import pytest
+import torch
+
+from climbing_gym_amd.synthetic import TINY, random_state_dict
+from oracle.lfm2_oracle import (OracleConfig, OracleEngine, apply_rotary, graph_capacity,
+                                plan_prefill_chunks, rms_norm)
+
+SMALL = dict(hidden=64, mlp_hidden=128, layer_types=("conv", "full_attention", "conv", "full_attention"),
+             q_heads=8, kv_heads=4, vocab=257)
+
+
+def _cfg(shape, max_pos=256, theta=1e6):
+    return OracleConfig(vocab_size=shape["vocab"], hidden_size=shape["hidden"], mlp_hidden_size=shape["mlp_hidden"],
+                        num_hidden_layers=len(shape["layer_types"]), num_attention_heads=shape["q_heads"],
+                        num_key_value_heads=shape["kv_heads"], max_position_embeddings=max_pos,
+                        rope_theta=theta, layer_types=tuple(shape["layer_types"]))
+
+
+def _hf_model(shape, sd, theta=1e6):
+    from transformers import Lfm2Config, Lfm2ForCausalLM
+    hf = Lfm2Config(vocab_size=shape["vocab"], hidden_size=shape["hidden"], intermediate_size=shape["mlp_hidden"],
+                    num_hidden_layers=len(shape["layer_types"]), num_attention_heads=shape["q_heads"],
+                    num_key_value_heads=shape["kv_heads"], max_position_embeddings=256, norm_eps=1e-5,
+                    conv_L_cache=3, conv_bias=False, block_auto_adjust_ff_dim=False,
+                    layer_types=list(shape["layer_types"]), tie_word_embeddings=True,
+                    rope_parameters={"rope_type": "default", "rope_theta": theta})
+    hf._attn_implementation = "eager"
+    model = Lfm2ForCausalLM(hf).eval()
+    state = dict(sd)
+    state["lm_head.weight"] = sd["model.embed_tokens.weight"]
+    missing, unexpected = model.load_state_dict(state, strict=False)
+    assert not unexpected, unexpected
+    assert all("rotary" in m or "lm_head" in m for m in missing), missing
+    return model
+
+
+@pytest.mark.parametrize("shape", [SMALL, TINY])
+@torch.inference_mode()
+def test_prefill_and_cached_decode_match_transformers(shape):
+    sd = random_state_dict(**shape, seed=0)
+    eng = OracleEngine(_cfg(shape), sd, torch.float32, max_model_len=256)
+    hf = _hf_model(shape, sd)
+    prompts = [[1, 11, 12, 13, 14, 15, 16], [1, 21, 22], [5]]
+    cache, logits = eng.prefill(prompts, cap=16)
+    for i, p in enumerate(prompts):
+        want = hf(torch.tensor([p]), use_cache=False).logits[0, -1]
+        torch.testing.assert_close(logits[i], want, atol=1e-5, rtol=1e-5)
+    assert cache.seq_lens.tolist() == [7, 3, 1]
+    # three cached decode steps against full recompute by the independent model
+    seqs = [list(p) for p in prompts]
+    for step in range(3):
+        toks = torch.tensor([40 + step, 50 + step, 60 + step])
+        out = eng.append_tokens(cache, torch.arange(3), toks)
+        for i in range(3):
+            seqs[i].append(int(toks[i]))
+            want = hf(torch.tensor([seqs[i]]), use_cache=False).logits[0, -1]
+            torch.testing.assert_close(out[i], want, atol=2e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("budget", (4, 24, 4096))
+@torch.inference_mode()
+def test_padded_chunk_prefill_equals_per_prompt_with_dirty_cache(budget):
+    sd = random_state_dict(**SMALL, seed=1)
+    eng = OracleEngine(_cfg(SMALL), sd, torch.float32, max_model_len=256)
+    prompts = [[1], [1, 2], [1, 3, 4, 5, 6], [1, 7, 8], [1, 9, 10, 11]]
+    ref_cache, ref_logits = eng.prefill(prompts, cap=32)
+    dirty = eng.empty_cache(len(prompts), 32)
+    dirty.k.fill_(0.5), dirty.v.fill_(-0.5), dirty.conv.fill_(1.0)
+    cache, logits = eng.prefill(prompts, cache=dirty, max_prefill_tokens=budget)
+    torch.testing.assert_close(logits, ref_logits, atol=1e-5, rtol=1e-4)
+    torch.testing.assert_close(cache.conv, ref_cache.conv, atol=1e-6, rtol=1e-4)
+    assert cache.seq_lens.tolist() == ref_cache.seq_lens.tolist()
+    slots = torch.arange(len(prompts))
+    for step in range(3):
+        a = eng.append_tokens(cache, slots, slots + 40 + step)
+        b = eng.append_tokens(ref_cache, slots, slots + 40 + step)
+        torch.testing.assert_close(a, b, atol=1e-5, rtol=1e-4)
+
+
+@torch.inference_mode()
+def test_decode_on_slot_subset_leaves_other_slots_alone():
+    sd = random_state_dict(**SMALL, seed=2)
+    eng = OracleEngine(_cfg(SMALL), sd, torch.float32, max_model_len=64)
+    cache, _ = eng.prefill([[1, 2, 3], [4, 5], [6, 7, 8, 9]], cap=16)
+    before = (cache.k[:, 1].clone(), cache.conv[:, 1].clone())
+    eng.append_tokens(cache, torch.tensor([2, 0]), torch.tensor([30, 31]))
+    assert cache.seq_lens.tolist() == [4, 2, 5]
+    assert torch.equal(cache.k[:, 1], before[0]) and torch.equal(cache.conv[:, 1], before[1])
+
+
+def test_rms_norm_matches_transformers_module():
+    from transformers.models.lfm2.modeling_lfm2 import Lfm2RMSNorm
+    torch.manual_seed(3)
+    for dt in (torch.float32, torch.bfloat16):
+        x = torch.randn(5, 7, 64, dtype=dt)
+        mod = Lfm2RMSNorm(64, eps=1e-5)
+        with torch.no_grad():
+            mod.weight.copy_(torch.randn(64))
+        mod = mod.to(dt)
+        torch.testing.assert_close(rms_norm(x, mod.weight.data, 1e-5), mod(x), atol=0, rtol=0)
+
+
+def test_rotary_bf16_is_bitwise_transformers():
+    # same construction as the reference's tests/test_lfm25_cuda.py:95-109
+    from transformers.models.lfm2.modeling_lfm2 import apply_rotary_pos_emb
+    torch.manual_seed(18)
+    q = torch.randn(3, 1, 32, 64, dtype=torch.bfloat16)
+    k = torch.randn(3, 1, 8, 64, dtype=torch.bfloat16)
+    freq = torch.tensor([27, 1331, 8000])[:, None, None] / (1e7 ** (torch.arange(0, 64, 2) / 64))
+    cos, sin = freq.cos().bfloat16(), freq.sin().bfloat16()
+    eq, ek = apply_rotary_pos_emb(q, k, cos.repeat(1, 1, 2), sin.repeat(1, 1, 2), unsqueeze_dim=2)
+    assert torch.equal(apply_rotary(q, cos[:, :, None], sin[:, :, None]), eq)
+    assert torch.equal(apply_rotary(k, cos[:, :, None], sin[:, :, None]), ek)
+
+
+def test_chunk_planner_known_answers():
+    # lengths of tests/test_lfm25_cuda.py:291 under its three budgets
+    lens = [1, 2, 5, 3, 4]
+    assert plan_prefill_chunks(lens, 4) == [(0, 2, 2), (2, 3, 5), (3, 4, 3), (4, 5, 4)]
+    assert plan_prefill_chunks(lens, 24) == [(0, 4, 5), (4, 5, 4)]
+    assert plan_prefill_chunks(lens, 4096) == [(0, 5, 5)]
+    # a single prompt longer than the budget is still taken alone
+    assert plan_prefill_chunks([9, 1], 4) == [(0, 1, 9), (1, 2, 1)]
+
+
+def test_capacity_rounding_known_answers():
+    # tests/test_lfm25_cuda.py:367-380: 64 rows, prompt<=10 + 20 new -> 32; +12 tokens -> 64
+    assert graph_capacity(10 + 20, 64, 256) == 32
+    assert graph_capacity(22 + 20, 64, 256) == 64
+    assert graph_capacity(30, 3, 256) == 128
+    assert graph_capacity(250, 3, 256) == 256
