@@ -1,0 +1,116 @@
+"""ctypes binding of liblfm2_hip.so (the C ABI declared in include/lfm2_hip.h).
+
+There is no CPU fallback: if the library is missing or a call fails, an exception is raised.
+Tensors are passed as raw device pointers; launches go to torch's current HIP stream so they are
+ordered with torch's own work and are recorded by `torch.cuda.graph` captures.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIBRARY_PATH = os.path.join(_HERE, "liblfm2_hip.so")
+
+DTYPE_CODE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
+
+# p = pointer, l = int64, i = int, f = float.  Order matches include/lfm2_hip.h.
+_SIGNATURES = {
+    "lfm2_embedding": "ppplllip",
+    "lfm2_rms_norm": "ppppp" "llfip",
+    "lfm2_rms_norm_fp8": "pppppp" "llfip",
+    "lfm2_swiglu": "ppllip",
+    "lfm2_swiglu_fp8": "pppllip",
+    "lfm2_quantize_rows": "pppllip",
+    "lfm2_conv_update": "pppppp" "lllip",
+    "lfm2_prepare_qkv": "ppppppppp" "liiilfip",
+    "lfm2_conv_prefill": "ppppppp" "llllip",
+    "lfm2_fp8_gemm": "pppppp" "llliiip",
+    "lfm2_bf16_gemm": "pppp" "llliip",
+    "lfm2_store_kv_fp8": "ppppppppp" "lliilllllllllip",
+    "lfm2_append_kv": "ppppppp" "liilllip",
+    "lfm2_store_kv_packed": "ppppppppp" "liillliip",
+    "lfm2_decode_attention": "pppppppppp" "lip" "liiillllfiip",
+    "lfm2_prefill_attention": "ppppp" "lliiifip",
+    "lfm2_build_token_map": "ppp" "llp",
+    "lfm2_gather_inputs": "ppppppp" "lp",
+    "lfm2_scatter_logits": "pppp" "llip",
+    "lfm2_advance_positions": "pppp" "lp",
+    "lfm2_sample": "ppppppp" "llfllip",
+    "lfm2_sample_filtered": "pppppp" "llfifllip",
+    "lfm2_head_logprobs": "ppppp" "lliip",
+    "lfm2_record_sample": "ppppppppppppppp" "llllp",
+    "lfm2_record_head": "pppppp" "illp",
+}
+_INT64_RESULT = {
+    "lfm2_fp8_gemm_workspace": "lll",
+    "lfm2_bf16_gemm_workspace": "lll",
+    "lfm2_decode_attention_workspace": "liil",
+}
+_CTYPE = {"p": ctypes.c_void_p, "l": ctypes.c_int64, "i": ctypes.c_int, "f": ctypes.c_float}
+
+_lib = None
+
+
+def exported_symbols():
+    """Every entry point include/lfm2_hip.h declares."""
+    return sorted([*_SIGNATURES, *_INT64_RESULT, "lfm2_last_error", "lfm2_abi_version"])
+
+
+def load():
+    """Load the shared library once; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIBRARY_PATH):
+        raise RuntimeError(
+            f"{LIBRARY_PATH} is missing: build it with `python -m climbing_gym_amd.build` (hipcc, gfx950). "
+            "This package has no CPU or PyTorch fallback for its kernels.")
+    lib = ctypes.CDLL(LIBRARY_PATH)
+    for name, sig in _SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.argtypes = [_CTYPE[c] for c in sig]
+        fn.restype = ctypes.c_int
+    for name, sig in _INT64_RESULT.items():
+        fn = getattr(lib, name)
+        fn.argtypes = [_CTYPE[c] for c in sig]
+        fn.restype = ctypes.c_int64
+    lib.lfm2_last_error.restype = ctypes.c_char_p
+    lib.lfm2_abi_version.restype = ctypes.c_int
+    _lib = lib
+    return lib
+
+
+def _arg(value):
+    if value is None:
+        return None
+    if isinstance(value, torch.Tensor):
+        return value.data_ptr()
+    return value
+
+
+def stream_handle() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def call(name: str, *args):
+    """Invoke an int-returning entry point on the current stream (appended as the last argument)."""
+    lib = load()
+    status = getattr(lib, name)(*[_arg(a) for a in args], stream_handle())
+    if status != 0:
+        message = lib.lfm2_last_error().decode()
+        if status == -1:
+            raise ValueError(f"{name}: {message}")
+        raise RuntimeError(f"{name} failed ({status}): {message}")
+
+
+def query(name: str, *args) -> int:
+    return int(getattr(load(), name)(*args))
+
+
+def require_device(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise ValueError("HIP kernels require tensors on the GPU")

@@ -1,0 +1,463 @@
+// Row-wise fused kernels of the LFM2 decode step: embedding gather, residual+RMSNorm (with an
+// optional per-token e4m3 epilogue), SwiGLU (same), row quantisation, the gated short-conv
+// rolling-state update, QK-norm + RoPE + QKV split, and the packed-prefill short conv.
+//
+// All of them are HBM/launch bound: one 256-thread workgroup owns one row (or one row x 2048
+// column slab), reads it once with 16-byte loads, keeps it in registers across the two
+// reductions (sum of squares, abs-max) and writes each output once.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "lfm2_common.h"
+
+// ------------------------------------------------------------------------------------ errors
+static thread_local char g_error[512] = "";
+void lfm2_set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+extern "C" const char* lfm2_last_error(void) { return g_error; }
+extern "C" int lfm2_abi_version(void) { return 1; }
+
+#define DISPATCH_DTYPE(dtype, ...)                                         \
+  switch (dtype) {                                                         \
+    case LFM2_DTYPE_BF16: { typedef __bf16 T; __VA_ARGS__; } break;        \
+    case LFM2_DTYPE_F16: { typedef _Float16 T; __VA_ARGS__; } break;       \
+    case LFM2_DTYPE_F32: { typedef float T; __VA_ARGS__; } break;          \
+    default: LFM2_FAIL(LFM2_ERR_ARGUMENT, "unknown dtype %d", dtype);      \
+  }
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / 64;
+
+template <typename T> struct Vec {
+  static constexpr int N = 16 / sizeof(T);
+  typedef T type __attribute__((ext_vector_type(16 / sizeof(T))));
+};
+
+template <typename T> __device__ __forceinline__ void load_vec(const T* p, float* out) {
+  typename Vec<T>::type v = *reinterpret_cast<const typename Vec<T>::type*>(p);
+#pragma unroll
+  for (int i = 0; i < Vec<T>::N; ++i) out[i] = Elem<T>::load(v[i]);
+}
+template <typename T> __device__ __forceinline__ void store_vec(T* p, const float* in) {
+  typename Vec<T>::type v;
+#pragma unroll
+  for (int i = 0; i < Vec<T>::N; ++i) v[i] = Elem<T>::store(in[i]);
+  *reinterpret_cast<typename Vec<T>::type*>(p) = v;
+}
+// N consecutive e4m3 codes (N = 4 or 8).
+template <int N> __device__ __forceinline__ void store_e4m3(uint8_t* p, const float* v, float scale) {
+  int w0 = pack_e4m3x4(v[0] / scale, v[1] / scale, v[2] / scale, v[3] / scale);
+  if (N == 4) {
+    *reinterpret_cast<int*>(p) = w0;
+  } else {
+    int w1 = pack_e4m3x4(v[4] / scale, v[5] / scale, v[6] / scale, v[7] / scale);
+    i32x2 w = {w0, w1};
+    *reinterpret_cast<i32x2*>(p) = w;
+  }
+}
+
+// ------------------------------------------------------------------------------------ embedding
+template <typename T>
+__global__ void __launch_bounds__(kThreads) embedding_kernel(T* out, const T* table, const int64_t* tokens,
+                                                            int64_t H, int64_t V) {
+  const int64_t row = blockIdx.x;
+  int64_t tok = tokens[row];
+  tok = tok < 0 ? 0 : (tok >= V ? V - 1 : tok);
+  const T* src = table + tok * H;
+  T* dst = out + row * H;
+  constexpr int N = Vec<T>::N;
+  if (H % N == 0) {
+    for (int64_t i = threadIdx.x * N; i < H; i += kThreads * N)
+      *reinterpret_cast<typename Vec<T>::type*>(dst + i) = *reinterpret_cast<const typename Vec<T>::type*>(src + i);
+  } else {
+    for (int64_t i = threadIdx.x; i < H; i += kThreads) dst[i] = src[i];
+  }
+}
+
+extern "C" int lfm2_embedding(void* out, const void* table, const int64_t* tokens, int64_t M, int64_t H,
+                              int64_t V, int dtype, void* stream) {
+  LFM2_REQUIRE(M > 0 && H > 0 && V > 0, "embedding: empty shape");
+  DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(embedding_kernel<T>, dim3(M), dim3(kThreads), 0, (hipStream_t)stream,
+                                           (T*)out, (const T*)table, tokens, H, V));
+  LFM2_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------------------ RMSNorm (+e4m3)
+// NV = 16-byte vectors per thread held in registers; NV == 0 selects the scalar path that
+// recomputes values from global memory in each pass (any H).
+template <typename T, int NV, bool ADD, bool FP8>
+__global__ void __launch_bounds__(kThreads)
+rms_norm_kernel(T* out, uint8_t* q, float* scales, T* summed, const T* x, const T* w, const T* res, int64_t H,
+                float eps) {
+  __shared__ float red[kWaves];
+  const int64_t row = blockIdx.x;
+  constexpr int N = Vec<T>::N;
+  x += row * H;
+  if (ADD) { res += row * H; summed += row * H; }
+  if (FP8) q += row * H; else out += row * H;
+
+  if constexpr (NV > 0) {
+    float v[NV][N];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int64_t i = (int64_t)(j * kThreads + threadIdx.x) * N;
+      if (i < H) {
+        load_vec<T>(x + i, v[j]);
+        if (ADD) {
+          float r[N];
+          load_vec<T>(res + i, r);
+#pragma unroll
+          for (int e = 0; e < N; ++e) v[j][e] = round_to<T>(v[j][e] + r[e]);
+          store_vec<T>(summed + i, v[j]);
+        }
+#pragma unroll
+        for (int e = 0; e < N; ++e) ss += v[j][e] * v[j][e];
+      }
+    }
+    ss = block_sum<kWaves>(ss, red);
+    const float rstd = 1.0f / sqrtf(ss / (float)H + eps);
+    float amax = 0.f;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int64_t i = (int64_t)(j * kThreads + threadIdx.x) * N;
+      if (i < H) {
+        float g[N];
+        load_vec<T>(w + i, g);
+#pragma unroll
+        for (int e = 0; e < N; ++e) {
+          v[j][e] = round_to<T>(v[j][e] * rstd) * g[e];
+          if (FP8) { v[j][e] = round_to<T>(v[j][e]); amax = fmaxf(amax, fabsf(v[j][e])); }
+        }
+        if (!FP8) store_vec<T>(out + i, v[j]);
+      }
+    }
+    if (FP8) {
+      amax = block_max<kWaves>(amax, red);
+      const float scale = fmaxf(amax / LFM2_E4M3_MAX, 1.0e-12f);
+      if (threadIdx.x == 0) scales[row] = scale;
+#pragma unroll
+      for (int j = 0; j < NV; ++j) {
+        const int64_t i = (int64_t)(j * kThreads + threadIdx.x) * N;
+        if (i < H) store_e4m3<N>(q + i, v[j], scale);
+      }
+    }
+  } else {
+    auto value = [&](int64_t i) {
+      float a = Elem<T>::load(x[i]);
+      if (ADD) a = round_to<T>(a + Elem<T>::load(res[i]));
+      return a;
+    };
+    float ss = 0.f;
+    for (int64_t i = threadIdx.x; i < H; i += kThreads) {
+      const float a = value(i);
+      if (ADD) summed[i] = Elem<T>::store(a);
+      ss += a * a;
+    }
+    ss = block_sum<kWaves>(ss, red);
+    const float rstd = 1.0f / sqrtf(ss / (float)H + eps);
+    auto normed = [&](int64_t i) {
+      float n = round_to<T>(value(i) * rstd) * Elem<T>::load(w[i]);
+      return FP8 ? round_to<T>(n) : n;
+    };
+    if (!FP8) {
+      for (int64_t i = threadIdx.x; i < H; i += kThreads) out[i] = Elem<T>::store(normed(i));
+    } else {
+      float amax = 0.f;
+      for (int64_t i = threadIdx.x; i < H; i += kThreads) amax = fmaxf(amax, fabsf(normed(i)));
+      amax = block_max<kWaves>(amax, red);
+      const float scale = fmaxf(amax / LFM2_E4M3_MAX, 1.0e-12f);
+      if (threadIdx.x == 0) scales[row] = scale;
+      for (int64_t i = threadIdx.x; i < H; i += kThreads) q[i] = to_e4m3(normed(i) / scale);
+    }
+  }
+}
+
+// Smallest register tile that covers a row of `width` elements, 0 when it must take the scalar path.
+template <typename T> static int pick_nv(int64_t width) {
+  constexpr int N = 16 / sizeof(T);
+  if (width % N != 0) return 0;
+  for (int nv = 1; nv <= 16; nv *= 2)
+    if ((int64_t)nv * kThreads * N >= width) return nv;
+  return 0;
+}
+
+#define LAUNCH_NV(nv, KERNEL_EXPR_1, KERNEL_EXPR_2, KERNEL_EXPR_4, KERNEL_EXPR_8, KERNEL_EXPR_16, KERNEL_EXPR_0) \
+  switch (nv) {                                                                                                  \
+    case 1: KERNEL_EXPR_1; break;                                                                                \
+    case 2: KERNEL_EXPR_2; break;                                                                                \
+    case 4: KERNEL_EXPR_4; break;                                                                                \
+    case 8: KERNEL_EXPR_8; break;                                                                                \
+    case 16: KERNEL_EXPR_16; break;                                                                              \
+    default: KERNEL_EXPR_0; break;                                                                               \
+  }
+
+template <typename T, bool ADD, bool FP8>
+static void launch_rms(void* out, uint8_t* q, float* scales, void* summed, const void* x, const void* w,
+                       const void* res, int64_t M, int64_t H, float eps, hipStream_t s) {
+  const int nv = pick_nv<T>(H);
+#define RMS_(NVV)                                                                                            \
+  hipLaunchKernelGGL((rms_norm_kernel<T, NVV, ADD, FP8>), dim3(M), dim3(kThreads), 0, s, (T*)out, q, scales, \
+                     (T*)summed, (const T*)x, (const T*)w, (const T*)res, H, eps)
+  LAUNCH_NV(nv, RMS_(1), RMS_(2), RMS_(4), RMS_(8), RMS_(16), RMS_(0));
+#undef RMS_
+}
+
+extern "C" int lfm2_rms_norm(void* out, void* summed, const void* x, const void* weight, const void* residual,
+                             int64_t M, int64_t H, float eps, int dtype, void* stream) {
+  LFM2_REQUIRE(M > 0 && H > 0, "rms_norm: empty shape");
+  LFM2_REQUIRE(residual == nullptr || summed != nullptr, "rms_norm: residual given without a summed output");
+  hipStream_t s = (hipStream_t)stream;
+  DISPATCH_DTYPE(dtype, if (residual) launch_rms<T, true, false>(out, nullptr, nullptr, summed, x, weight, residual, M, H, eps, s);
+                 else launch_rms<T, false, false>(out, nullptr, nullptr, nullptr, x, weight, nullptr, M, H, eps, s));
+  LFM2_LAUNCH_CHECK();
+}
+
+extern "C" int lfm2_rms_norm_fp8(uint8_t* q, float* scales, void* summed, const void* x, const void* weight,
+                                 const void* residual, int64_t M, int64_t H, float eps, int dtype, void* stream) {
+  LFM2_REQUIRE(M > 0 && H > 0, "rms_norm_fp8: empty shape");
+  LFM2_REQUIRE(residual == nullptr || summed != nullptr, "rms_norm_fp8: residual given without a summed output");
+  hipStream_t s = (hipStream_t)stream;
+  DISPATCH_DTYPE(dtype, if (residual) launch_rms<T, true, true>(nullptr, q, scales, summed, x, weight, residual, M, H, eps, s);
+                 else launch_rms<T, false, true>(nullptr, q, scales, nullptr, x, weight, nullptr, M, H, eps, s));
+  LFM2_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------------------ SwiGLU
+__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
+
+template <typename T>
+__global__ void __launch_bounds__(kThreads) swiglu_kernel(T* out, const T* x, int64_t I) {
+  const int64_t row = blockIdx.y;
+  constexpr int N = Vec<T>::N;
+  const T* gate = x + row * 2 * I;
+  const T* up = gate + I;
+  out += row * I;
+  if (I % N == 0) {
+    const int64_t i = ((int64_t)blockIdx.x * kThreads + threadIdx.x) * N;
+    if (i < I) {
+      float g[N], u[N];
+      load_vec<T>(gate + i, g);
+      load_vec<T>(up + i, u);
+#pragma unroll
+      for (int e = 0; e < N; ++e) g[e] = round_to<T>(silu_f(g[e])) * u[e];
+      store_vec<T>(out + i, g);
+    }
+  } else {
+    for (int e = 0; e < N; ++e) {
+      const int64_t i = ((int64_t)blockIdx.x * kThreads + threadIdx.x) * N + e;
+      if (i < I) out[i] = Elem<T>::store(round_to<T>(silu_f(Elem<T>::load(gate[i]))) * Elem<T>::load(up[i]));
+    }
+  }
+}
+
+extern "C" int lfm2_swiglu(void* out, const void* x, int64_t M, int64_t I, int dtype, void* stream) {
+  LFM2_REQUIRE(M > 0 && I > 0, "swiglu: empty shape");
+  LFM2_REQUIRE(M <= 65535, "swiglu: more than 65535 rows");
+  DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(swiglu_kernel<T>, dim3(ceil_div(I, kThreads * Vec<T>::N), M), dim3(kThreads),
+                                           0, (hipStream_t)stream, (T*)out, (const T*)x, I));
+  LFM2_LAUNCH_CHECK();
+}
+
+// SWIGLU = false gives plain row quantisation of x[M,K].
+template <typename T, int NV, bool SWIGLU>
+__global__ void __launch_bounds__(kThreads) quantize_kernel(uint8_t* q, float* scales, const T* x, int64_t K) {
+  __shared__ float red[kWaves];
+  const int64_t row = blockIdx.x;
+  constexpr int N = Vec<T>::N;
+  const T* a = x + row * (SWIGLU ? 2 * K : K);
+  const T* b = a + K;
+  q += row * K;
+  float amax = 0.f;
+  if constexpr (NV > 0) {
+    float v[NV][N];
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int64_t i = (int64_t)(j * kThreads + threadIdx.x) * N;
+      if (i < K) {
+        load_vec<T>(a + i, v[j]);
+        if (SWIGLU) {
+          float u[N];
+          load_vec<T>(b + i, u);
+#pragma unroll
+          for (int e = 0; e < N; ++e) v[j][e] = round_to<T>(round_to<T>(silu_f(v[j][e])) * u[e]);
+        }
+#pragma unroll
+        for (int e = 0; e < N; ++e) amax = fmaxf(amax, fabsf(v[j][e]));
+      }
+    }
+    amax = block_max<kWaves>(amax, red);
+    const float scale = fmaxf(amax / LFM2_E4M3_MAX, 1.0e-12f);
+    if (threadIdx.x == 0) scales[row] = scale;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int64_t i = (int64_t)(j * kThreads + threadIdx.x) * N;
+      if (i < K) store_e4m3<N>(q + i, v[j], scale);
+    }
+  } else {
+    auto value = [&](int64_t i) {
+      float g = Elem<T>::load(a[i]);
+      return SWIGLU ? round_to<T>(round_to<T>(silu_f(g)) * Elem<T>::load(b[i])) : g;
+    };
+    for (int64_t i = threadIdx.x; i < K; i += kThreads) amax = fmaxf(amax, fabsf(value(i)));
+    amax = block_max<kWaves>(amax, red);
+    const float scale = fmaxf(amax / LFM2_E4M3_MAX, 1.0e-12f);
+    if (threadIdx.x == 0) scales[row] = scale;
+    for (int64_t i = threadIdx.x; i < K; i += kThreads) q[i] = to_e4m3(value(i) / scale);
+  }
+}
+
+template <typename T, bool SWIGLU>
+static void launch_quantize(uint8_t* q, float* scales, const void* x, int64_t M, int64_t K, hipStream_t s) {
+  const int nv = pick_nv<T>(K);
+#define Q_(NVV) \
+  hipLaunchKernelGGL((quantize_kernel<T, NVV, SWIGLU>), dim3(M), dim3(kThreads), 0, s, q, scales, (const T*)x, K)
+  LAUNCH_NV(nv, Q_(1), Q_(2), Q_(4), Q_(8), Q_(16), Q_(0));
+#undef Q_
+}
+
+extern "C" int lfm2_swiglu_fp8(uint8_t* q, float* scales, const void* x, int64_t M, int64_t I, int dtype, void* stream) {
+  LFM2_REQUIRE(M > 0 && I > 0, "swiglu_fp8: empty shape");
+  DISPATCH_DTYPE(dtype, launch_quantize<T, true>(q, scales, x, M, I, (hipStream_t)stream));
+  LFM2_LAUNCH_CHECK();
+}
+
+extern "C" int lfm2_quantize_rows(uint8_t* q, float* scales, const void* x, int64_t M, int64_t K, int dtype, void* stream) {
+  LFM2_REQUIRE(M > 0 && K > 0, "quantize_rows: empty shape");
+  DISPATCH_DTYPE(dtype, launch_quantize<T, false>(q, scales, x, M, K, (hipStream_t)stream));
+  LFM2_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------------------ short-conv update
+template <typename T>
+__global__ void __launch_bounds__(kThreads)
+conv_update_kernel(T* out, const T* bcx, const T* w, T* state, const uint8_t* active, const int32_t* slot_ids, int64_t H) {
+  const int64_t row = blockIdx.y;
+  const int64_t col = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (col >= H) return;
+  int64_t slot = row;
+  if (slot_ids) { const int32_t s = slot_ids[row]; slot = s < 0 ? 0 : s; }
+  const bool on = active ? active[row] != 0 : true;
+  const T* in = bcx + row * 3 * H;
+  const float b = Elem<T>::load(in[col]), c = Elem<T>::load(in[H + col]), x = Elem<T>::load(in[2 * H + col]);
+  const float bx = round_to<T>(b * x);
+  T* st = state + (slot * H + col) * 3;
+  const T t1 = st[1], t2 = st[2];
+  const float s0 = Elem<T>::load(t1), s1 = Elem<T>::load(t2);
+  const float w0 = Elem<T>::load(w[col * 3]), w1 = Elem<T>::load(w[col * 3 + 1]), w2 = Elem<T>::load(w[col * 3 + 2]);
+  const float p0 = round_to<T>(s0 * w0), p1 = round_to<T>(s1 * w1), p2 = round_to<T>(bx * w2);
+  const float conv = round_to<T>((p0 + p1) + p2);
+  if (on) { st[0] = t1; st[1] = t2; st[2] = Elem<T>::store(bx); }
+  out[row * H + col] = Elem<T>::store(c * conv);
+}
+
+extern "C" int lfm2_conv_update(void* out, const void* bcx, const void* weight, void* state, const uint8_t* active,
+                                const int32_t* slot_ids, int64_t M, int64_t H, int64_t slots, int dtype, void* stream) {
+  LFM2_REQUIRE(M > 0 && H > 0 && slots > 0, "conv_update: empty shape");
+  LFM2_REQUIRE(slot_ids != nullptr || M <= slots, "conv_update: %ld rows but only %ld state slots", (long)M, (long)slots);
+  LFM2_REQUIRE(M <= 65535, "conv_update: more than 65535 rows");
+  DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(conv_update_kernel<T>, dim3(ceil_div(H, kThreads), M), dim3(kThreads), 0,
+                                           (hipStream_t)stream, (T*)out, (const T*)bcx, (const T*)weight, (T*)state,
+                                           active, slot_ids, H));
+  LFM2_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------------------ packed-prefill short conv
+// One thread per (token, channel).  Taps that would reach before the start of the token's own
+// sequence read zero, so sequences packed back to back do not leak into each other.
+template <typename T>
+__global__ void __launch_bounds__(kThreads)
+conv_prefill_kernel(T* out, T* state, const T* bcx, const T* w, const int32_t* cu, const int32_t* seq_of_token,
+                    const int32_t* slots, int64_t H) {
+  const int64_t t = blockIdx.y;
+  const int64_t col = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (col >= H) return;
+  const int seq = seq_of_token[t];
+  const int64_t begin = cu[seq], end = cu[seq + 1];
+  auto bx_at = [&](int64_t tok) -> float {
+    if (tok < begin) return 0.f;
+    const T* in = bcx + tok * 3 * H;
+    return round_to<T>(Elem<T>::load(in[col]) * Elem<T>::load(in[2 * H + col]));
+  };
+  const float x0 = bx_at(t - 2), x1 = bx_at(t - 1), x2 = bx_at(t);
+  const float w0 = Elem<T>::load(w[col * 3]), w1 = Elem<T>::load(w[col * 3 + 1]), w2 = Elem<T>::load(w[col * 3 + 2]);
+  const float conv = round_to<T>(fmaf(x2, w2, fmaf(x1, w1, x0 * w0)));
+  const float c = Elem<T>::load(bcx[t * 3 * H + H + col]);
+  out[t * H + col] = Elem<T>::store(c * conv);
+  if (t == end - 1) {
+    T* st = state + ((int64_t)slots[seq] * H + col) * 3;
+    st[0] = Elem<T>::store(x0); st[1] = Elem<T>::store(x1); st[2] = Elem<T>::store(x2);
+  }
+}
+
+extern "C" int lfm2_conv_prefill(void* out, void* state, const void* bcx, const void* weight, const int32_t* cu_seqlens,
+                                 const int32_t* seq_of_token, const int32_t* slots, int64_t T_, int64_t nseq, int64_t H,
+                                 int64_t nslots, int dtype, void* stream) {
+  LFM2_REQUIRE(T_ > 0 && nseq > 0 && H > 0 && nslots > 0, "conv_prefill: empty shape");
+  LFM2_REQUIRE(T_ <= 65535, "conv_prefill: more than 65535 packed tokens in one call");
+  DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(conv_prefill_kernel<T>, dim3(ceil_div(H, kThreads), T_), dim3(kThreads), 0,
+                                           (hipStream_t)stream, (T*)out, (T*)state, (const T*)bcx, (const T*)weight,
+                                           cu_seqlens, seq_of_token, slots, H));
+  LFM2_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------------------ QK-norm + RoPE + split
+// One workgroup per row; each wave walks over heads.  A lane owns D/64 (or fewer) elements of a
+// head and reaches its rotate-half partner through LDS.
+template <typename T>
+__global__ void __launch_bounds__(kThreads)
+prepare_qkv_kernel(T* q, T* k, T* v, const T* x, const T* qw, const T* kw, const float* cosT, const float* sinT,
+                   const int32_t* positions, int QH, int KH, int D, int64_t max_positions, float eps) {
+  __shared__ float buf[kWaves][256];
+  const int64_t row = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t width = (int64_t)(QH + 2 * KH) * D;
+  const T* in = x + row * width;
+  int64_t pos = positions[row];
+  pos = pos < 0 ? 0 : (pos >= max_positions ? max_positions - 1 : pos);
+  const int half = D / 2;
+  for (int head = wave; head < QH + KH; head += kWaves) {
+    const T* src = in + (int64_t)head * D;
+    const T* wgt = head < QH ? qw : kw;
+    float ss = 0.f;
+    for (int d = lane; d < D; d += 64) { const float a = Elem<T>::load(src[d]); ss += a * a; }
+    ss = wave_sum(ss);
+    const float rstd = 1.0f / sqrtf(ss / (float)D + eps);
+    for (int d = lane; d < D; d += 64) {
+      float n = round_to<T>(Elem<T>::load(src[d]) * rstd);
+      buf[wave][d] = round_to<T>(n * Elem<T>::load(wgt[d]));
+    }
+    __builtin_amdgcn_wave_barrier();
+    T* dst = head < QH ? q + (row * QH + head) * D : k + (row * KH + (head - QH)) * D;
+    for (int d = lane; d < D; d += 64) {
+      const float c = round_to<T>(cosT[pos * half + d % half]);
+      const float s = round_to<T>(sinT[pos * half + d % half]);
+      const float left = round_to<T>(buf[wave][d] * c);
+      const float right = round_to<T>(buf[wave][(d + half) % D] * s);
+      dst[d] = Elem<T>::store(d < half ? left - right : left + right);
+    }
+    __builtin_amdgcn_wave_barrier();
+    if (head >= QH) {
+      const int kh = head - QH;
+      const T* vs = in + (int64_t)(QH + KH + kh) * D;
+      T* vd = v + (row * KH + kh) * D;
+      for (int d = lane; d < D; d += 64) vd[d] = vs[d];
+    }
+  }
+}
+
+extern "C" int lfm2_prepare_qkv(void* q, void* k, void* v, const void* x, const void* q_weight, const void* k_weight,
+                                const float* cos, const float* sin, const int32_t* positions, int64_t M, int QH, int KH,
+                                int D, int64_t max_positions, float eps, int dtype, void* stream) {
+  LFM2_REQUIRE(M > 0 && QH > 0 && KH > 0, "prepare_qkv: empty shape");
+  LFM2_REQUIRE(D > 0 && D <= 256 && D % 2 == 0, "prepare_qkv: head_dim %d not in (0,256] or odd", D);
+  LFM2_REQUIRE(max_positions > 0, "prepare_qkv: empty rotary table");
+  DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(prepare_qkv_kernel<T>, dim3(M), dim3(kThreads), 0, (hipStream_t)stream, (T*)q,
+                                           (T*)k, (T*)v, (const T*)x, (const T*)q_weight, (const T*)k_weight, cos, sin,
+                                           positions, QH, KH, D, max_positions, eps));
+  LFM2_LAUNCH_CHECK();
+}

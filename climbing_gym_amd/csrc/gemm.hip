@@ -1,0 +1,319 @@
+// "NT" GEMMs of the LFM2 linear layers on MFMA: out[M,N] = A[M,K] . W[N,K]^T.
+//
+//   fp8  : A, W are OCP e4m3 bytes, v_mfma_f32_16x16x32_fp8_fp8, epilogue * a_scale[m] * w_scale[n]
+//   bf16 : v_mfma_f32_16x16x32_bf16, plain epilogue
+//
+// Both operands are K-contiguous, so the kernel works on 16-byte chunks of K for either type:
+// a workgroup stages a BM x 128 B tile of A and a BN x 128 B tile of W per step through LDS
+// (double buffered, one barrier per step, next tile prefetched into registers during the MFMAs).
+// Chunks are XOR-swizzled by row so the 16-lane column reads of the MFMA operand layout spread
+// over all banks.  A lane of lane-group g = lane/16 takes chunks g and g+4 of its row for both
+// operands, so the contraction order inside a 128 B step is permuted identically on both sides
+// and needs no shuffles.  W is the MFMA "A" operand, so a lane ends with four consecutive output
+// columns of one row and stores 8 bytes at a time.
+//
+// Workgroup ids are remapped so that the M-tiles sharing one W tile run back to back on the same
+// XCD (ids are dealt round-robin over the 8 XCDs, each with its own L2): W streams from HBM once.
+#include "lfm2_common.h"
+
+namespace {
+
+constexpr int kStepBytes = 128;          // K bytes staged per step
+constexpr int kChunksPerRow = kStepBytes / 16;
+
+__device__ __forceinline__ int lds_slot(int row, int chunk) { return row * kChunksPerRow + (chunk ^ (row & 7)); }
+
+template <int EB> struct Mfma;
+template <> struct Mfma<1> {  // e4m3: one 16 B chunk feeds two K=32 instructions
+  static __device__ __forceinline__ f32x4 run(const i32x4& w, const i32x4& a, f32x4 acc) {
+    long w0 = ((long)(unsigned)w[1] << 32) | (unsigned)w[0], w1 = ((long)(unsigned)w[3] << 32) | (unsigned)w[2];
+    long a0 = ((long)(unsigned)a[1] << 32) | (unsigned)a[0], a1 = ((long)(unsigned)a[3] << 32) | (unsigned)a[2];
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w0, a0, acc, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w1, a1, acc, 0, 0, 0);
+  }
+};
+template <> struct Mfma<2> {  // bf16: one chunk is one K=32 operand
+  static __device__ __forceinline__ f32x4 run(const i32x4& w, const i32x4& a, f32x4 acc) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, w), __builtin_bit_cast(bf16x8, a), acc, 0, 0, 0);
+  }
+};
+
+__device__ __forceinline__ void store_out(void* out, int out_dtype, int64_t idx, float v) {
+  if (out_dtype == LFM2_DTYPE_BF16) ((__bf16*)out)[idx] = (__bf16)v;
+  else if (out_dtype == LFM2_DTYPE_F16) ((_Float16*)out)[idx] = (_Float16)v;
+  else ((float*)out)[idx] = v;
+}
+
+template <int EB, int BM, int BN, int WM, int WN>
+__global__ void __launch_bounds__(WM * WN * 64)
+gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_t* __restrict__ A,
+               const uint8_t* __restrict__ W, const float* __restrict__ a_scales, const float* __restrict__ w_scales,
+               int M, int N, int64_t Kb, int steps_per_split, int out_dtype) {
+  constexpr int NT = WM * WN * 64;
+  constexpr int TM = BM / WM, TN = BN / WN, MI = TM / 16, NI = TN / 16;
+  constexpr int A_CHUNKS = BM * kChunksPerRow, W_CHUNKS = BN * kChunksPerRow;
+  constexpr int A_PER = (A_CHUNKS + NT - 1) / NT, W_PER = (W_CHUNKS + NT - 1) / NT;
+  __shared__ i32x4 lds[2][A_CHUNKS + W_CHUNKS];
+
+  // XCD-aware tile order: consecutive logical ids (same XCD, adjacent in time) share an N tile.
+  const int mt = (M + BM - 1) / BM, nt = (N + BN - 1) / BN, tiles = mt * nt;
+  const int per_xcd = gridDim.x / 8;
+  const int lid = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (lid >= tiles) return;
+  const int m_base = (lid % mt) * BM, n_base = (lid / mt) * BN;
+
+  const int64_t total_steps = (Kb + kStepBytes - 1) / kStepBytes;
+  const int64_t step0 = (int64_t)blockIdx.y * steps_per_split;
+  int64_t nsteps = total_steps - step0;
+  if (nsteps > steps_per_split) nsteps = steps_per_split;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave % WM, wn = wave / WM;
+  const int lrow = lane & 15, lgrp = lane >> 4;
+
+  i32x4 ra[A_PER], rw[W_PER];
+  auto fetch = [&](int64_t step) {
+    const int64_t kb = (step0 + step) * kStepBytes;
+#pragma unroll
+    for (int i = 0; i < A_PER; ++i) {
+      const int idx = tid + i * NT;
+      const int row = idx / kChunksPerRow, c = idx % kChunksPerRow;
+      i32x4 v = {0, 0, 0, 0};
+      if ((A_CHUNKS % NT == 0 || idx < A_CHUNKS) && kb + c * 16 < Kb) {
+        int gr = m_base + row;
+        gr = gr < M ? gr : M - 1;
+        v = *reinterpret_cast<const i32x4*>(A + (int64_t)gr * Kb + kb + c * 16);
+      }
+      ra[i] = v;
+    }
+#pragma unroll
+    for (int i = 0; i < W_PER; ++i) {
+      const int idx = tid + i * NT;
+      const int row = idx / kChunksPerRow, c = idx % kChunksPerRow;
+      i32x4 v = {0, 0, 0, 0};
+      if ((W_CHUNKS % NT == 0 || idx < W_CHUNKS) && kb + c * 16 < Kb) {
+        int gr = n_base + row;
+        gr = gr < N ? gr : N - 1;
+        v = *reinterpret_cast<const i32x4*>(W + (int64_t)gr * Kb + kb + c * 16);
+      }
+      rw[i] = v;
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < A_PER; ++i) {
+      const int idx = tid + i * NT;
+      if (A_CHUNKS % NT == 0 || idx < A_CHUNKS) lds[buf][lds_slot(idx / kChunksPerRow, idx % kChunksPerRow)] = ra[i];
+    }
+#pragma unroll
+    for (int i = 0; i < W_PER; ++i) {
+      const int idx = tid + i * NT;
+      if (W_CHUNKS % NT == 0 || idx < W_CHUNKS)
+        lds[buf][A_CHUNKS + lds_slot(idx / kChunksPerRow, idx % kChunksPerRow)] = rw[i];
+    }
+  };
+
+  f32x4 acc[MI][NI];
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < NI; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  if (nsteps > 0) {
+    fetch(0);
+    stash(0);
+  }
+  __syncthreads();
+  for (int64_t s = 0; s < nsteps; ++s) {
+    const int buf = (int)(s & 1);
+    if (s + 1 < nsteps) fetch(s + 1);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int c = lgrp + 4 * h;
+      i32x4 fa[MI], fw[NI];
+#pragma unroll
+      for (int i = 0; i < MI; ++i) fa[i] = lds[buf][lds_slot(wm * TM + i * 16 + lrow, c)];
+#pragma unroll
+      for (int j = 0; j < NI; ++j) fw[j] = lds[buf][A_CHUNKS + lds_slot(wn * TN + j * 16 + lrow, c)];
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) acc[i][j] = Mfma<EB>::run(fw[j], fa[i], acc[i][j]);
+    }
+    if (s + 1 < nsteps) stash(buf ^ 1);
+    __syncthreads();
+  }
+
+  // Epilogue: lane holds out[m = .. + lrow][n = .. + 4*lgrp + r], r = 0..3.
+  const bool split = partial != nullptr;
+#pragma unroll
+  for (int i = 0; i < MI; ++i) {
+    const int m = m_base + wm * TM + i * 16 + lrow;
+    if (m >= M) continue;
+    const float sa = (!split && a_scales) ? a_scales[m] : 1.0f;
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const int n = n_base + wn * TN + j * 16 + 4 * lgrp;
+      if (n >= N) continue;
+      f32x4 v = acc[i][j];
+      if (split) {
+        float* dst = partial + ((int64_t)blockIdx.y * M + m) * N + n;
+        if (n + 3 < N && (N & 3) == 0) *reinterpret_cast<f32x4*>(dst) = v;
+        else for (int r = 0; r < 4 && n + r < N; ++r) dst[r] = v[r];
+        continue;
+      }
+      if (a_scales)
+        for (int r = 0; r < 4; ++r) v[r] = (v[r] * sa) * (n + r < N ? w_scales[n + r] : 0.f);
+      const int64_t idx = (int64_t)m * N + n;
+      if (out_dtype == LFM2_DTYPE_BF16 && n + 3 < N && (N & 3) == 0) {
+        bf16x4 o = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
+        *reinterpret_cast<bf16x4*>((__bf16*)out + idx) = o;
+      } else {
+        for (int r = 0; r < 4 && n + r < N; ++r) store_out(out, out_dtype, idx + r, v[r]);
+      }
+    }
+  }
+}
+
+// Sum split-K partials in split order, then scale (lfm25_fp8.py:94-105 order: row scale, column scale).
+__global__ void __launch_bounds__(256)
+reduce_split_kernel(void* out, const float* partial, const float* a_scales, const float* w_scales, int64_t M, int64_t N,
+                    int splits, int out_dtype) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= M * N) return;
+  float t = 0.f;
+  for (int s = 0; s < splits; ++s) t += partial[(int64_t)s * M * N + idx];
+  if (a_scales) t = (t * a_scales[idx / N]) * w_scales[idx % N];
+  store_out(out, out_dtype, idx, t);
+}
+
+// Any-shape fallback (K not a multiple of 16 bytes): one thread per output element.
+template <int EB>
+__global__ void __launch_bounds__(256)
+gemm_naive_kernel(void* out, const uint8_t* A, const uint8_t* W, const float* a_scales, const float* w_scales, int64_t M,
+                  int64_t N, int64_t K, int out_dtype) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= M * N) return;
+  const int64_t m = idx / N, n = idx % N;
+  float t = 0.f;
+  if (EB == 1) {
+    const uint8_t *a = A + m * K, *w = W + n * K;
+    for (int64_t k = 0; k < K; ++k) {
+      f32x2 x = __builtin_amdgcn_cvt_pk_f32_fp8((int)a[k], false), y = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[k], false);
+      t = fmaf(x[0], y[0], t);
+    }
+  } else {
+    const __bf16 *a = (const __bf16*)A + m * K, *w = (const __bf16*)W + n * K;
+    for (int64_t k = 0; k < K; ++k) t = fmaf((float)a[k], (float)w[k], t);
+  }
+  if (a_scales) t = (t * a_scales[m]) * w_scales[n];
+  store_out(out, out_dtype, idx, t);
+}
+
+struct TileInfo { int bm, bn; };
+constexpr int kNumTiles = 6;
+constexpr TileInfo kTiles[kNumTiles] = {{16, 64}, {32, 64}, {64, 64}, {128, 64}, {128, 128}, {64, 128}};
+
+struct Plan { int tile, splits; };
+
+// Default tile/split choice: the largest tile that still gives every CU work, then split K until
+// the chip (256 CUs) is covered, keeping at least four 128-byte steps per split.
+Plan default_plan(int64_t M, int64_t N, int64_t Kb) {
+  int tile;
+  if (M <= 16) tile = 0;
+  else if (M <= 32) tile = 1;
+  else if (M <= 64) tile = 2;
+  else {
+    const int64_t big = ((M + 127) / 128) * ((N + 127) / 128);
+    const int64_t mid = ((M + 127) / 128) * ((N + 63) / 64);
+    tile = big >= 512 ? 4 : (mid >= 384 ? 3 : 2);
+  }
+  const int64_t tiles = ((M + kTiles[tile].bm - 1) / kTiles[tile].bm) * ((N + kTiles[tile].bn - 1) / kTiles[tile].bn);
+  const int64_t steps = (Kb + kStepBytes - 1) / kStepBytes;
+  int splits = 1;
+  while (tiles * splits < 256 && splits < 16 && steps / (splits * 2) >= 4) splits *= 2;
+  return {tile, splits};
+}
+
+template <int EB, int BM, int BN, int WM, int WN>
+void launch_tile(void* out, float* partial, const uint8_t* A, const uint8_t* W, const float* as, const float* ws, int M,
+                 int N, int64_t Kb, int splits, int out_dtype, hipStream_t s) {
+  const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  const int64_t steps = (Kb + kStepBytes - 1) / kStepBytes;
+  const int per = (int)((steps + splits - 1) / splits);
+  hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN>), dim3((tiles + 7) / 8 * 8, splits), dim3(WM * WN * 64), 0, s, out,
+                     splits > 1 ? partial : nullptr, A, W, as, ws, M, N, Kb, per, out_dtype);
+}
+
+template <int EB>
+int gemm_entry(const char* name, void* out, const void* a, const float* as, const void* w, const float* ws,
+               float* workspace, int64_t M, int64_t N, int64_t K, int out_dtype, int tile, int split_k, void* stream) {
+  LFM2_REQUIRE(M > 0 && N > 0 && K > 0, "%s: empty shape", name);
+  LFM2_REQUIRE(M < (1 << 30) && N < (1 << 30), "%s: M or N too large", name);
+  LFM2_REQUIRE(out_dtype >= LFM2_DTYPE_BF16 && out_dtype <= LFM2_DTYPE_F32, "%s: bad output dtype", name);
+  hipStream_t s = (hipStream_t)stream;
+  const uint8_t *A = (const uint8_t*)a, *W = (const uint8_t*)w;
+  const int64_t Kb = K * EB;
+  if (Kb % 16 != 0 || ((uintptr_t)a | (uintptr_t)w) % 16 != 0) {
+    hipLaunchKernelGGL(gemm_naive_kernel<EB>, dim3(ceil_div(M * N, 256)), dim3(256), 0, s, out, A, W, as, ws, M, N, K, out_dtype);
+    LFM2_LAUNCH_CHECK();
+  }
+  Plan plan = default_plan(M, N, Kb);
+  if (tile >= 0) {
+    LFM2_REQUIRE(tile < kNumTiles, "%s: tile index %d out of range", name, tile);
+    plan.tile = tile;
+  }
+  if (split_k > 0) plan.splits = split_k;
+  const int64_t steps = (Kb + kStepBytes - 1) / kStepBytes;
+  if (plan.splits > steps) plan.splits = (int)steps;
+  // every split must own at least one step
+  while (plan.splits > 1 && (steps + plan.splits - 1) / plan.splits * (plan.splits - 1) >= steps) --plan.splits;
+  LFM2_REQUIRE(plan.splits == 1 || workspace != nullptr, "%s: split-K needs a workspace", name);
+#define TILE_(ID, BM, BN, WM, WN) \
+  case ID: launch_tile<EB, BM, BN, WM, WN>(out, workspace, A, W, as, ws, (int)M, (int)N, Kb, plan.splits, out_dtype, s); break
+  switch (plan.tile) {
+    TILE_(0, 16, 64, 1, 4);
+    TILE_(1, 32, 64, 2, 2);
+    TILE_(2, 64, 64, 2, 2);
+    TILE_(3, 128, 64, 2, 2);
+    TILE_(4, 128, 128, 2, 2);
+    TILE_(5, 64, 128, 2, 2);
+  }
+#undef TILE_
+  if (plan.splits > 1)
+    hipLaunchKernelGGL(reduce_split_kernel, dim3(ceil_div(M * N, 256)), dim3(256), 0, s, out, workspace, as, ws, M, N,
+                       plan.splits, out_dtype);
+  LFM2_LAUNCH_CHECK();
+}
+
+int64_t workspace_floats(int64_t M, int64_t N, int64_t Kb) {
+  if (Kb % 16 != 0) return 0;
+  // Upper bound over every split choice the entry point accepts (<= 16 splits).
+  return 16 * M * N;
+}
+
+}  // namespace
+
+extern "C" int lfm2_fp8_gemm(void* out, const uint8_t* a_q, const float* a_scales, const uint8_t* w_q,
+                             const float* w_scales, float* workspace, int64_t M, int64_t N, int64_t K, int out_dtype,
+                             int tile, int split_k, void* stream) {
+  LFM2_REQUIRE(a_scales && w_scales, "fp8_gemm: scales are required");
+  LFM2_REQUIRE(split_k <= 16, "fp8_gemm: split_k above 16");
+  return gemm_entry<1>("fp8_gemm", out, a_q, a_scales, w_q, w_scales, workspace, M, N, K, out_dtype, tile, split_k, stream);
+}
+
+extern "C" int64_t lfm2_fp8_gemm_workspace(int64_t M, int64_t N, int64_t K) {
+  const Plan p = default_plan(M, N, K);
+  return (K % 16 == 0 && p.splits > 1) ? (int64_t)p.splits * M * N : 0;
+}
+
+extern "C" int lfm2_bf16_gemm(void* out, const void* x, const void* w, float* workspace, int64_t M, int64_t N, int64_t K,
+                              int tile, int split_k, void* stream) {
+  LFM2_REQUIRE(split_k <= 16, "bf16_gemm: split_k above 16");
+  return gemm_entry<2>("bf16_gemm", out, x, nullptr, w, nullptr, workspace, M, N, K, LFM2_DTYPE_BF16, tile, split_k, stream);
+}
+
+extern "C" int64_t lfm2_bf16_gemm_workspace(int64_t M, int64_t N, int64_t K) {
+  const Plan p = default_plan(M, N, K * 2);
+  return ((K * 2) % 16 == 0 && p.splits > 1) ? (int64_t)p.splits * M * N : 0;
+}

@@ -1,0 +1,113 @@
+// Shared device helpers for the LFM2 gfx950 kernels (wave64, CDNA4).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/lfm2_hip.h"
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+#define LFM2_E4M3_MAX 448.0f
+#define LFM2_LOG2E 1.4426950408889634f
+
+// ---- error reporting shared by every translation unit -------------------------------
+void lfm2_set_error(const char* fmt, ...);
+#define LFM2_FAIL(code, ...)       \
+  do {                             \
+    lfm2_set_error(__VA_ARGS__);   \
+    return (code);                 \
+  } while (0)
+#define LFM2_REQUIRE(cond, ...) \
+  do {                          \
+    if (!(cond)) LFM2_FAIL(LFM2_ERR_ARGUMENT, __VA_ARGS__); \
+  } while (0)
+#define LFM2_LAUNCH_CHECK()                                                    \
+  do {                                                                         \
+    hipError_t e_ = hipGetLastError();                                         \
+    if (e_ != hipSuccess) LFM2_FAIL(LFM2_ERR_LAUNCH, "%s", hipGetErrorString(e_)); \
+    return LFM2_OK;                                                            \
+  } while (0)
+
+// ---- dtype traits -----------------------------------------------------------------
+template <typename T> struct Elem;
+template <> struct Elem<__bf16> {
+  static __device__ __forceinline__ float load(__bf16 v) { return (float)v; }
+  static __device__ __forceinline__ __bf16 store(float v) { return (__bf16)v; }
+};
+template <> struct Elem<_Float16> {
+  static __device__ __forceinline__ float load(_Float16 v) { return (float)v; }
+  static __device__ __forceinline__ _Float16 store(float v) { return (_Float16)v; }
+};
+template <> struct Elem<float> {
+  static __device__ __forceinline__ float load(float v) { return v; }
+  static __device__ __forceinline__ float store(float v) { return v; }
+};
+// Round an fp32 value to the model dtype and return it as fp32 again.
+template <typename T> __device__ __forceinline__ float round_to(float v) { return Elem<T>::load(Elem<T>::store(v)); }
+
+// ---- wave / block reductions (64-lane wavefronts) ----------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+// Block-wide reductions through a small LDS array; every thread gets the result.
+template <int WAVES> __device__ __forceinline__ float block_sum(float v, float* scratch) {
+  v = wave_sum(v);
+  if (WAVES == 1) return v;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float t = 0.f;
+#pragma unroll
+  for (int i = 0; i < WAVES; ++i) t += scratch[i];
+  return t;
+}
+template <int WAVES> __device__ __forceinline__ float block_max(float v, float* scratch) {
+  v = wave_max(v);
+  if (WAVES == 1) return v;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float t = scratch[0];
+#pragma unroll
+  for (int i = 1; i < WAVES; ++i) t = fmaxf(t, scratch[i]);
+  return t;
+}
+
+// ---- e4m3 (OCP, finite-only) conversions --------------------------------------------
+// Saturating round-to-nearest-even of four fp32 values into one dword of e4m3 codes.
+__device__ __forceinline__ int pack_e4m3x4(float a, float b, float c, float d) {
+  a = fminf(fmaxf(a, -LFM2_E4M3_MAX), LFM2_E4M3_MAX);
+  b = fminf(fmaxf(b, -LFM2_E4M3_MAX), LFM2_E4M3_MAX);
+  c = fminf(fmaxf(c, -LFM2_E4M3_MAX), LFM2_E4M3_MAX);
+  d = fminf(fmaxf(d, -LFM2_E4M3_MAX), LFM2_E4M3_MAX);
+  int r = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+  return __builtin_amdgcn_cvt_pk_fp8_f32(c, d, r, true);
+}
+__device__ __forceinline__ uint8_t to_e4m3(float a) {
+  a = fminf(fmaxf(a, -LFM2_E4M3_MAX), LFM2_E4M3_MAX);
+  return (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(a, a, 0, false) & 0xff);
+}
+// Four e4m3 codes in a dword -> four floats.
+__device__ __forceinline__ void unpack_e4m3x4(int w, float* out) {
+  f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
+  f32x2 hi = __builtin_amdgcn_cvt_pk_f32_fp8(w, true);
+  out[0] = lo[0]; out[1] = lo[1]; out[2] = hi[0]; out[3] = hi[1];
+}
+
+static inline int ceil_div(long a, long b) { return (int)((a + b - 1) / b); }

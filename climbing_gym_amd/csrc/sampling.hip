@@ -1,0 +1,516 @@
+// On-GPU sampling and scheduler bookkeeping: greedy / Gumbel-max categorical sampling with raw
+// log-probabilities, temperature + top-k + nucleus sampling, the per-row record step of a
+// generation session (stop automaton, finish codes, RNG positions) and the slot gather/scatter
+// used by compact decode batches.  Nothing here synchronises with the host.
+#include "lfm2_common.h"
+
+namespace {
+
+#define DISPATCH_DTYPE(dtype, name, ...)                                               \
+  switch (dtype) {                                                                     \
+    case LFM2_DTYPE_BF16: { typedef __bf16 T; __VA_ARGS__; } break;                    \
+    case LFM2_DTYPE_F16: { typedef _Float16 T; __VA_ARGS__; } break;                   \
+    case LFM2_DTYPE_F32: { typedef float T; __VA_ARGS__; } break;                      \
+    default: LFM2_FAIL(LFM2_ERR_ARGUMENT, "%s: unknown dtype %d", name, dtype);        \
+  }
+
+constexpr uint64_t kGolden = 0x9E3779B97F4A7C15ull;
+constexpr uint64_t kMask63 = 0x7FFFFFFFFFFFFFFFull;
+constexpr int kTile = 4096;
+
+// Philox4x32-10 (Salmon et al. 2011): 128-bit counter, 64-bit key -> four 32-bit words.
+__device__ __forceinline__ void philox(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1,
+                                       uint32_t* out) {
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    const uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+    const uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+    c0 = hi1 ^ c1 ^ k0; c1 = lo1; c2 = hi0 ^ c3 ^ k1; c3 = lo0;
+    k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+  }
+  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+// Standard Gumbel noise from a 32-bit word: u in [0,1) floored at 1e-30 (lfm25_sampling.py:21-27).
+__device__ __forceinline__ float gumbel(uint32_t bits) {
+  const float u = fmaxf((float)(bits >> 8) * (1.0f / 16777216.0f), 1.0e-30f);
+  return -logf(-logf(u));
+}
+__device__ __forceinline__ uint64_t row_key(int64_t seed, int64_t step) {
+  return ((uint64_t)seed + (uint64_t)step * kGolden) & kMask63;
+}
+
+// ------------------------------------------------------------------------------------ full-support sampler
+// Pass 1: one workgroup per (row, 4096-column tile): best Gumbel score with its first index, and
+// the tile's (max, sum exp) of the raw logits.  scratch[(row*parts+part)*4 + {score,index,max,sum}].
+template <typename T>
+__global__ void __launch_bounds__(256)
+sample_partial_kernel(const T* logits, float* scratch, const int64_t* seeds, const int64_t* steps,
+                      const float* temperatures, int64_t seed, int64_t step, float temperature, int64_t V, int parts) {
+  __shared__ float s_score[4], s_max[4], s_sum[4];
+  __shared__ int s_index[4];
+  const int64_t row = blockIdx.y;
+  const int part = blockIdx.x;
+  const bool per_row = seeds != nullptr;
+  const float temp = per_row ? temperatures[row] : temperature;
+  const uint64_t key = per_row ? row_key(seeds[row], steps[row]) : row_key(seed, step);
+  const T* src = logits + row * V;
+  float best = -INFINITY, tmax = -INFINITY;
+  int best_i = 0x7fffffff;
+  float vals[16];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t col0 = (int64_t)part * kTile + (i * 256 + threadIdx.x) * 4;
+    uint32_t rnd[4] = {0, 0, 0, 0};
+    if (temp > 0.f && col0 < V) {
+      // per-row streams count columns; the shared stream counts flattened (row, column) like the reference
+      const uint64_t ctr = per_row ? (uint64_t)(col0 >> 2) : (uint64_t)((row * V + col0) >> 2);
+      philox((uint32_t)ctr, (uint32_t)(ctr >> 32), per_row ? 0u : (uint32_t)((row * V + col0) & 3), 0u, (uint32_t)key,
+             (uint32_t)(key >> 32), rnd);
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int64_t col = col0 + e;
+      const float x = col < V ? Elem<T>::load(src[col]) : -INFINITY;
+      vals[i * 4 + e] = x;
+      tmax = fmaxf(tmax, x);
+      float score = x;
+      if (temp > 0.f) score = x / fmaxf(temp, 1.0e-30f) + gumbel(rnd[e]);
+      if (col < V && (score > best || best_i == 0x7fffffff)) { best = score; best_i = (int)col; }
+    }
+  }
+  // wave then block arg-max (ties -> lowest column) and max
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ob = __shfl_xor(best, o, 64);
+    const int oi = __shfl_xor(best_i, o, 64);
+    if (oi != 0x7fffffff && (best_i == 0x7fffffff || ob > best || (ob == best && oi < best_i))) { best = ob; best_i = oi; }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, o, 64));
+  }
+  if (lane == 0) { s_score[wave] = best; s_index[wave] = best_i; s_max[wave] = tmax; }
+  __syncthreads();
+  float bmax = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
+  const float shift = bmax == -INFINITY ? 0.f : bmax;
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) sum += expf(vals[i] - shift);
+  sum = wave_sum(sum);
+  if (lane == 0) s_sum[wave] = sum;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float b = s_score[0];
+    int bi = s_index[0];
+    for (int w = 1; w < 4; ++w)
+      if (s_index[w] != 0x7fffffff && (bi == 0x7fffffff || s_score[w] > b || (s_score[w] == b && s_index[w] < bi))) { b = s_score[w]; bi = s_index[w]; }
+    float* dst = scratch + (row * parts + part) * 4;
+    dst[0] = b; dst[1] = __int_as_float(bi); dst[2] = bmax; dst[3] = (s_sum[0] + s_sum[1]) + (s_sum[2] + s_sum[3]);
+  }
+}
+
+// Pass 2: merge the tiles of a row.
+template <typename T>
+__global__ void __launch_bounds__(64)
+sample_finish_kernel(const T* logits, const float* scratch, int64_t* tokens, float* logprobs, int64_t V, int parts) {
+  const int64_t row = blockIdx.x;
+  const float* src = scratch + row * parts * 4;
+  float best = -INFINITY, mx = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int p = threadIdx.x; p < parts; p += 64) {
+    const float s = src[p * 4];
+    const int i = __float_as_int(src[p * 4 + 1]);
+    if (i != 0x7fffffff && (bi == 0x7fffffff || s > best || (s == best && i < bi))) { best = s; bi = i; }
+    mx = fmaxf(mx, src[p * 4 + 2]);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ob = __shfl_xor(best, o, 64);
+    const int oi = __shfl_xor(bi, o, 64);
+    if (oi != 0x7fffffff && (bi == 0x7fffffff || ob > best || (ob == best && oi < bi))) { best = ob; bi = oi; }
+    mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+  }
+  float total = 0.f;
+  for (int p = threadIdx.x; p < parts; p += 64) total += src[p * 4 + 3] * expf(src[p * 4 + 2] - mx);
+  total = wave_sum(total);
+  if (threadIdx.x == 0) {
+    if (bi == 0x7fffffff) bi = 0;
+    tokens[row] = bi;
+    if (logprobs) logprobs[row] = Elem<T>::load(logits[row * V + bi]) - (mx + logf(total));
+  }
+}
+
+// ------------------------------------------------------------------------------------ filtered sampler
+// Order-preserving map float -> uint32 (larger float = larger key).
+__device__ __forceinline__ uint32_t order_key(float x) {
+  const uint32_t b = __float_as_uint(x);
+  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+constexpr int kFT = 1024;  // threads of the filtered sampler
+
+// One workgroup per row.  All decisions use integer histograms (counts, and 2^40 fixed-point
+// softmax mass), so results do not depend on the order in which lanes reach the atomics.
+template <typename T>
+__global__ void __launch_bounds__(kFT)
+sample_filtered_kernel(const T* logits, int64_t* tokens, float* logprobs, int32_t* kept_count, const int64_t* seeds,
+                       const int64_t* steps, int64_t seed, int64_t step, float temperature, int top_k, float top_p, int64_t V) {
+  __shared__ uint32_t h_cnt[256];
+  __shared__ unsigned long long h_mass[256];
+  __shared__ float s_f[kFT / 64];
+  __shared__ int s_i[kFT / 64];
+  __shared__ uint32_t s_digit, s_remaining, s_cnt_above;
+  __shared__ unsigned long long s_mass_above, s_total;
+  __shared__ int s_scan[kFT];
+  __shared__ int s_cut, s_cross;
+  const int64_t row = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const T* src = logits + row * V;
+  const uint64_t key64 = seeds ? row_key(seeds[row], steps[row]) : row_key(seed, step);
+
+  // raw max / normaliser (for the returned log-probability) -- identical for scaled logits' argmax
+  float mx = -INFINITY;
+  for (int64_t i = tid; i < V; i += kFT) mx = fmaxf(mx, Elem<T>::load(src[i]));
+  mx = wave_max(mx);
+  if (lane == 0) s_f[wave] = mx;
+  __syncthreads();
+  mx = s_f[0];
+  for (int w = 1; w < kFT / 64; ++w) mx = fmaxf(mx, s_f[w]);
+  __syncthreads();
+  float raw_sum = 0.f;
+  for (int64_t i = tid; i < V; i += kFT) raw_sum += expf(Elem<T>::load(src[i]) - mx);
+  raw_sum = wave_sum(raw_sum);
+  if (lane == 0) s_f[wave] = raw_sum;
+  __syncthreads();
+  raw_sum = 0.f;
+  for (int w = 0; w < kFT / 64; ++w) raw_sum += s_f[w];
+  const float xmax = mx / temperature;
+  auto scaled = [&](int64_t i) { return Elem<T>::load(src[i]) / temperature; };
+  auto mass_of = [&](float x) -> unsigned long long { return (unsigned long long)(exp2f((x - xmax) * LFM2_LOG2E) * 1099511627776.0f); };
+
+  // ---- top-k: key of the k-th largest scaled logit
+  uint32_t key_k = 0;
+  if (top_k > 0 && top_k < V) {
+    uint32_t prefix = 0, mask = 0;
+    if (tid == 0) s_remaining = (uint32_t)top_k;
+    for (int pass = 0; pass < 4; ++pass) {
+      const int shift = 24 - 8 * pass;
+      for (int i = tid; i < 256; i += kFT) h_cnt[i] = 0;
+      __syncthreads();
+      for (int64_t i = tid; i < V; i += kFT) {
+        const uint32_t k = order_key(scaled(i));
+        if ((k & mask) == prefix) atomicAdd(&h_cnt[(k >> shift) & 255], 1u);
+      }
+      __syncthreads();
+      if (tid == 0) {
+        uint32_t rem = s_remaining;
+        int d = 255;
+        for (; d > 0; --d) {
+          if (h_cnt[d] >= rem) break;
+          rem -= h_cnt[d];
+        }
+        s_digit = (uint32_t)d; s_remaining = rem;
+      }
+      __syncthreads();
+      prefix |= s_digit << shift;
+      mask |= 0xFFu << shift;
+      __syncthreads();
+    }
+    key_k = prefix;
+  }
+
+  // ---- nucleus: walk keys downward until the inclusive cumulative mass exceeds top_p * Z
+  uint32_t kp = key_k;
+  int ties_kept = 0x7fffffff;
+  uint32_t cnt_above = 0;
+  if (top_p < 1.0f) {
+    unsigned long long z = 0;
+    for (int64_t i = tid; i < V; i += kFT) {
+      const float x = scaled(i);
+      if (order_key(x) >= key_k) z += mass_of(x);
+    }
+    if (tid == 0) s_total = 0;
+    __syncthreads();
+    atomicAdd(&s_total, z);
+    __syncthreads();
+    const unsigned long long limit = (unsigned long long)((double)top_p * (double)s_total);
+    uint32_t prefix = 0, mask = 0;
+    if (tid == 0) { s_mass_above = 0; s_cnt_above = 0; s_cross = 0; }
+    for (int pass = 0; pass < 4; ++pass) {
+      const int shift = 24 - 8 * pass;
+      for (int i = tid; i < 256; i += kFT) { h_cnt[i] = 0; h_mass[i] = 0; }
+      __syncthreads();
+      for (int64_t i = tid; i < V; i += kFT) {
+        const float x = scaled(i);
+        const uint32_t k = order_key(x);
+        if (k >= key_k && (k & mask) == prefix) {
+          atomicAdd(&h_cnt[(k >> shift) & 255], 1u);
+          atomicAdd(&h_mass[(k >> shift) & 255], mass_of(x));
+        }
+      }
+      __syncthreads();
+      if (tid == 0) {
+        unsigned long long above = s_mass_above;
+        uint32_t ca = s_cnt_above;
+        int d = 255, crossed = 0;
+        for (; d >= 0; --d) {
+          if (h_cnt[d] == 0) continue;
+          if (above + h_mass[d] > limit) { crossed = 1; break; }
+          above += h_mass[d]; ca += h_cnt[d];
+        }
+        s_cross = crossed; s_digit = (uint32_t)(d < 0 ? 0 : d); s_mass_above = above; s_cnt_above = ca;
+        s_remaining = crossed ? h_cnt[d] : 0;
+      }
+      __syncthreads();
+      if (!s_cross) break;
+      prefix |= s_digit << shift;
+      mask |= 0xFFu << shift;
+      __syncthreads();
+    }
+    if (s_cross) {
+      kp = prefix;
+      cnt_above = s_cnt_above;
+      const unsigned long long w = mass_of(__uint_as_float((kp & 0x80000000u) ? (kp & 0x7fffffffu) : ~kp));
+      unsigned long long fit = w ? (limit - s_mass_above) / w : 0;
+      if (fit >= s_remaining) fit = s_remaining;
+      ties_kept = (int)fit;
+      if (cnt_above == 0 && ties_kept == 0) ties_kept = 1;  // rank 0 always survives
+    }
+    __syncthreads();
+  }
+
+  // ---- when only some of the ties at kp survive, keep the lowest-index ones: find the cut column
+  int cut = 0x7fffffff;
+  if (ties_kept != 0x7fffffff) {
+    const int64_t strip = (V + kFT - 1) / kFT;
+    const int64_t lo = tid * strip, hi = lo + strip < V ? lo + strip : V;
+    int c = 0;
+    for (int64_t i = lo; i < hi; ++i) c += order_key(scaled(i)) == kp;
+    s_scan[tid] = c;
+    __syncthreads();
+    if (tid == 0) {
+      int run = 0;
+      s_cut = -1;
+      for (int t = 0; t < kFT; ++t) { const int v = s_scan[t]; s_scan[t] = run; run += v; }
+    }
+    __syncthreads();
+    const int before = s_scan[tid];
+    if (ties_kept > before && ties_kept <= before + c) {
+      int seen = before;
+      for (int64_t i = lo; i < hi; ++i)
+        if (order_key(scaled(i)) == kp && ++seen == ties_kept) { s_cut = (int)i; break; }
+    }
+    __syncthreads();
+    cut = s_cut;
+    if (kept_count && tid == 0) kept_count[row] = (int)cnt_above + ties_kept;
+  } else if (kept_count) {
+    int c = 0;
+    for (int64_t i = tid; i < V; i += kFT) c += order_key(scaled(i)) >= kp;
+    if (tid == 0) s_cut = 0;
+    __syncthreads();
+    atomicAdd(&s_cut, c);
+    __syncthreads();
+    if (tid == 0) kept_count[row] = s_cut;
+  }
+
+  // ---- Gumbel-max over the survivors
+  float best = -INFINITY;
+  int best_i = 0x7fffffff;
+  for (int64_t i = tid; i < V; i += kFT) {
+    const float x = scaled(i);
+    const uint32_t k = order_key(x);
+    if (!(k > kp || (k == kp && i <= cut))) continue;
+    uint32_t rnd[4];
+    philox((uint32_t)(i >> 2), (uint32_t)((uint64_t)i >> 34), 0x5eed5eedu, 0u, (uint32_t)key64, (uint32_t)(key64 >> 32), rnd);
+    const float score = x + gumbel(rnd[i & 3]);
+    if (best_i == 0x7fffffff || score > best) { best = score; best_i = (int)i; }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ob = __shfl_xor(best, o, 64);
+    const int oi = __shfl_xor(best_i, o, 64);
+    if (oi != 0x7fffffff && (best_i == 0x7fffffff || ob > best || (ob == best && oi < best_i))) { best = ob; best_i = oi; }
+  }
+  __syncthreads();
+  if (lane == 0) { s_f[wave] = best; s_i[wave] = best_i; }
+  __syncthreads();
+  if (tid == 0) {
+    float b = s_f[0];
+    int bi = s_i[0];
+    for (int w = 1; w < kFT / 64; ++w)
+      if (s_i[w] != 0x7fffffff && (bi == 0x7fffffff || s_f[w] > b || (s_f[w] == b && s_i[w] < bi))) { b = s_f[w]; bi = s_i[w]; }
+    if (bi == 0x7fffffff) bi = 0;
+    tokens[row] = bi;
+    if (logprobs) logprobs[row] = Elem<T>::load(src[bi]) - (mx + logf(raw_sum));
+  }
+}
+
+// ------------------------------------------------------------------------------------ small row kernels
+template <typename T>
+__global__ void head_logprobs_kernel(float* out, const T* logits, const int64_t* selected, const float* logprobs,
+                                     const T* values, int64_t V, int K) {
+  const int64_t row = blockIdx.x;
+  const float log_z = Elem<T>::load(logits[row * V + selected[row]]) - logprobs[row];
+  for (int c = threadIdx.x; c < K; c += blockDim.x) out[row * K + c] = Elem<T>::load(values[row * K + c]) - log_z;
+}
+
+__global__ void record_sample_kernel(const int64_t* sampled, const float* logp, int64_t* tokens, float* logprobs,
+                                     int32_t* lengths, const int32_t* limits, int8_t* reasons, uint8_t* alive,
+                                     uint8_t* pending, int64_t* input, int64_t* stop_states, const int64_t* stop_offsets,
+                                     const int32_t* stop_table, const uint8_t* ignore_eos, int64_t* rng_positions,
+                                     int64_t eos, int64_t V, int64_t cap, int64_t B) {
+  const int64_t row = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (row >= B || !alive[row]) return;
+  const int64_t token = sampled[row];
+  const int32_t length = lengths[row];
+  tokens[row * cap + length] = token;
+  logprobs[row * cap + length] = logp[row];
+  const int32_t value = stop_table[stop_offsets[row] + stop_states[row] * V + token];
+  stop_states[row] = value & 65535;
+  int8_t reason = 0;
+  if (token == eos && !ignore_eos[row]) reason = 1;
+  else if (value >= 65536) reason = 2;
+  else if (length + 1 >= limits[row]) reason = 3;
+  lengths[row] = length + 1;
+  rng_positions[row] += 1;
+  reasons[row] = reason;
+  alive[row] = reason == 0;
+  pending[row] = reason == 0;
+  input[row] = token;
+}
+
+__global__ void record_head_kernel(const int64_t* ids, const float* probs, int32_t* out_ids, float* out_probs,
+                                   const int32_t* lengths, const uint8_t* alive, int K, int64_t cap) {
+  const int64_t row = blockIdx.x;
+  if (!alive[row]) return;
+  const int64_t base = (row * cap + lengths[row]) * K;
+  for (int c = threadIdx.x; c < K; c += blockDim.x) {
+    out_ids[base + c] = (int32_t)ids[row * K + c];
+    out_probs[base + c] = probs[row * K + c];
+  }
+}
+
+__global__ void gather_inputs_kernel(int64_t* tokens, int32_t* positions, uint8_t* mask, const int64_t* input,
+                                     const int32_t* lengths, const uint8_t* active, const int32_t* slots, int64_t B) {
+  const int64_t row = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (row >= B) return;
+  const int32_t slot = slots[row];
+  const bool valid = slot >= 0;
+  tokens[row] = valid ? input[slot] : 0;
+  positions[row] = valid ? lengths[slot] : 0;
+  mask[row] = valid ? active[slot] : 0;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+scatter_logits_kernel(T* saved, const T* logits, const int32_t* slots, const uint8_t* active, int64_t V) {
+  const int64_t row = blockIdx.y;
+  if (!active[row]) return;
+  const int64_t slot = slots ? slots[row] : row;
+  if (slot < 0) return;
+  constexpr int N = 16 / sizeof(T);
+  typedef T vec __attribute__((ext_vector_type(N)));
+  const int64_t col = ((int64_t)blockIdx.x * 256 + threadIdx.x) * N;
+  if (V % N == 0) {
+    if (col < V) *reinterpret_cast<vec*>(saved + slot * V + col) = *reinterpret_cast<const vec*>(logits + row * V + col);
+  } else {
+    for (int e = 0; e < N; ++e)
+      if (col + e < V) saved[slot * V + col + e] = logits[row * V + col + e];
+  }
+}
+
+__global__ void advance_positions_kernel(int32_t* lengths, const int32_t* positions, const int32_t* slots,
+                                         const uint8_t* active, int64_t B) {
+  const int64_t row = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (row >= B) return;
+  const int32_t slot = slots ? slots[row] : (int32_t)row;
+  if (slot >= 0 && (active == nullptr || active[row])) lengths[slot] = positions[row] + 1;
+}
+
+}  // namespace
+
+extern "C" int lfm2_sample(int64_t* tokens, float* logprobs, const void* logits, float* scratch, const int64_t* seeds,
+                           const int64_t* steps, const float* temperatures, int64_t seed, int64_t step, float temperature,
+                           int64_t B, int64_t V, int dtype, void* stream) {
+  LFM2_REQUIRE(B > 0 && V > 0, "sample: empty logits");
+  LFM2_REQUIRE(B <= 65535, "sample: more than 65535 rows");
+  LFM2_REQUIRE(temperature >= 0.f, "sample: negative temperature");
+  LFM2_REQUIRE((seeds == nullptr) == (steps == nullptr) && (seeds == nullptr) == (temperatures == nullptr),
+               "sample: seeds, steps and temperatures go together");
+  const int parts = ceil_div(V, kTile);
+  hipStream_t s = (hipStream_t)stream;
+  DISPATCH_DTYPE(dtype, "sample",
+                 hipLaunchKernelGGL(sample_partial_kernel<T>, dim3(parts, B), dim3(256), 0, s, (const T*)logits, scratch, seeds,
+                                    steps, temperatures, seed, step, temperature, V, parts);
+                 hipLaunchKernelGGL(sample_finish_kernel<T>, dim3(B), dim3(64), 0, s, (const T*)logits, scratch, tokens,
+                                    logprobs, V, parts));
+  LFM2_LAUNCH_CHECK();
+}
+
+extern "C" int lfm2_sample_filtered(int64_t* tokens, float* logprobs, int32_t* kept_count, const void* logits,
+                                    const int64_t* seeds, const int64_t* steps, int64_t seed, int64_t step,
+                                    float temperature, int top_k, float top_p, int64_t B, int64_t V, int dtype,
+                                    void* stream) {
+  LFM2_REQUIRE(B > 0 && V > 0, "sample_filtered: empty logits");
+  LFM2_REQUIRE(temperature > 0.f, "sample_filtered: temperature must be positive");
+  LFM2_REQUIRE(top_k >= 0 && top_p > 0.f && top_p <= 1.f, "sample_filtered: top_k >= 0 and top_p in (0,1] required");
+  LFM2_REQUIRE(V < (1ll << 31), "sample_filtered: vocabulary too large");
+  LFM2_REQUIRE((seeds == nullptr) == (steps == nullptr), "sample_filtered: seeds and steps go together");
+  DISPATCH_DTYPE(dtype, "sample_filtered",
+                 hipLaunchKernelGGL(sample_filtered_kernel<T>, dim3(B), dim3(kFT), 0, (hipStream_t)stream, (const T*)logits,
+                                    tokens, logprobs, kept_count, seeds, steps, seed, step, temperature, top_k, top_p, V));
+  LFM2_LAUNCH_CHECK();
+}
+
+extern "C" int lfm2_head_logprobs(float* out, const void* logits, const int64_t* selected, const float* logprobs,
+                                  const void* values, int64_t B, int64_t V, int K, int dtype, void* stream) {
+  LFM2_REQUIRE(B > 0 && V > 0 && K > 0 && K <= 128, "head_logprobs: bad shape");
+  DISPATCH_DTYPE(dtype, "head_logprobs",
+                 hipLaunchKernelGGL(head_logprobs_kernel<T>, dim3(B), dim3(128), 0, (hipStream_t)stream, out, (const T*)logits,
+                                    selected, logprobs, (const T*)values, V, K));
+  LFM2_LAUNCH_CHECK();
+}
+
+extern "C" int lfm2_record_sample(const int64_t* sampled, const float* logp, int64_t* tokens, float* logprobs,
+                                  int32_t* lengths, const int32_t* limits, int8_t* reasons, uint8_t* alive,
+                                  uint8_t* pending, int64_t* input, int64_t* stop_states, const int64_t* stop_offsets,
+                                  const int32_t* stop_table, const uint8_t* ignore_eos, int64_t* rng_positions,
+                                  int64_t eos, int64_t V, int64_t cap, int64_t B, void* stream) {
+  LFM2_REQUIRE(B > 0 && V > 0 && cap > 0, "record_sample: bad shape");
+  hipLaunchKernelGGL(record_sample_kernel, dim3(ceil_div(B, 128)), dim3(128), 0, (hipStream_t)stream, sampled, logp, tokens,
+                     logprobs, lengths, limits, reasons, alive, pending, input, stop_states, stop_offsets, stop_table,
+                     ignore_eos, rng_positions, eos, V, cap, B);
+  LFM2_LAUNCH_CHECK();
+}
+
+extern "C" int lfm2_record_head(const int64_t* ids, const float* probs, int32_t* out_ids, float* out_probs,
+                                const int32_t* lengths, const uint8_t* alive, int K, int64_t cap, int64_t B, void* stream) {
+  LFM2_REQUIRE(B > 0 && K > 0 && cap > 0, "record_head: bad shape");
+  hipLaunchKernelGGL(record_head_kernel, dim3(B), dim3(128), 0, (hipStream_t)stream, ids, probs, out_ids, out_probs, lengths,
+                     alive, K, cap);
+  LFM2_LAUNCH_CHECK();
+}
+
+extern "C" int lfm2_gather_inputs(int64_t* tokens, int32_t* positions, uint8_t* mask, const int64_t* input,
+                                  const int32_t* lengths, const uint8_t* active, const int32_t* slots, int64_t B,
+                                  void* stream) {
+  LFM2_REQUIRE(B > 0, "gather_inputs: empty batch");
+  hipLaunchKernelGGL(gather_inputs_kernel, dim3(ceil_div(B, 128)), dim3(128), 0, (hipStream_t)stream, tokens, positions, mask,
+                     input, lengths, active, slots, B);
+  LFM2_LAUNCH_CHECK();
+}
+
+extern "C" int lfm2_scatter_logits(void* saved, const void* logits, const int32_t* slots, const uint8_t* active, int64_t B,
+                                   int64_t V, int dtype, void* stream) {
+  LFM2_REQUIRE(B > 0 && V > 0 && active, "scatter_logits: bad arguments");
+  LFM2_REQUIRE(B <= 65535, "scatter_logits: more than 65535 rows");
+  DISPATCH_DTYPE(dtype, "scatter_logits",
+                 hipLaunchKernelGGL(scatter_logits_kernel<T>, dim3(ceil_div(V, 256 * (16 / sizeof(T))), B), dim3(256), 0,
+                                    (hipStream_t)stream, (T*)saved, (const T*)logits, slots, active, V));
+  LFM2_LAUNCH_CHECK();
+}
+
+extern "C" int lfm2_advance_positions(int32_t* lengths, const int32_t* positions, const int32_t* slots,
+                                      const uint8_t* active, int64_t B, void* stream) {
+  LFM2_REQUIRE(B > 0, "advance_positions: empty batch");
+  hipLaunchKernelGGL(advance_positions_kernel, dim3(ceil_div(B, 128)), dim3(128), 0, (hipStream_t)stream, lengths, positions,
+                     slots, active, B);
+  LFM2_LAUNCH_CHECK();
+}

@@ -1,0 +1,365 @@
+"""Operator layer of the LFM2 decode/prefill step on MI355X.
+
+Each function keeps the name, argument meaning and error behaviour of the reference function it
+stands in for (cited per function, paths under the reference's src/climbing_gym/inference/), and
+launches the hand-written gfx950 kernel behind the C ABI.  Outputs are fresh tensors from torch's
+caching allocator unless stated, everything is ordered on the current stream and can be captured
+into a HIP graph.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from . import _lib
+from ._lib import DTYPE_CODE, call, query
+
+FP8 = torch.float8_e4m3fn
+
+
+def _code(dtype: torch.dtype) -> int:
+    try:
+        return DTYPE_CODE[dtype]
+    except KeyError:
+        raise ValueError(f"unsupported dtype {dtype}") from None
+
+
+def _rows(x: torch.Tensor) -> int:
+    return x.numel() // x.size(-1)
+
+
+def _check(*tensors):
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise ValueError("HIP kernels require GPU tensors")
+        if not t.is_contiguous():
+            raise ValueError("HIP kernels require contiguous tensors")
+
+
+# ----------------------------------------------------------------------------------- embedding / norms
+def embedding(tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    """F.embedding of lfm25_cuda.py:134 for int64 token ids."""
+    _check(tokens, table)
+    flat = tokens.reshape(-1).to(torch.long)
+    out = torch.empty((flat.numel(), table.size(1)), device=table.device, dtype=table.dtype)
+    call("lfm2_embedding", out, table, flat, flat.numel(), table.size(1), table.size(0), _code(table.dtype))
+    return out.view(*tokens.shape, table.size(1))
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: torch.Tensor | None = None):
+    """lfm25_cuda_kernels.py:47-55: returns (norm(x+residual)*w, x+residual); `summed is x` without residual."""
+    _check(x, weight, residual)
+    out = torch.empty_like(x)
+    summed = torch.empty_like(x) if residual is not None else x
+    call("lfm2_rms_norm", out, summed if residual is not None else None, x, weight, residual,
+         _rows(x), x.size(-1), float(eps), _code(x.dtype))
+    return out, summed
+
+
+def rms_norm_fp8(x, weight, eps, residual=None):
+    """lfm25_fp8.py:57-64: (e4m3 rows, per-row scales, x+residual)."""
+    _check(x, weight, residual)
+    q = torch.empty(x.shape, device=x.device, dtype=FP8)
+    scales = torch.empty(_rows(x), device=x.device, dtype=torch.float32)
+    summed = torch.empty_like(x) if residual is not None else x
+    call("lfm2_rms_norm_fp8", q, scales, summed if residual is not None else None, x, weight, residual,
+         _rows(x), x.size(-1), float(eps), _code(x.dtype))
+    return q, scales, summed
+
+
+def swiglu(x: torch.Tensor) -> torch.Tensor:
+    """lfm25_cuda_kernels.py:68-72: silu(gate) * up on [M, 2I] with the gate half first."""
+    _check(x)
+    width = x.size(-1) // 2
+    out = torch.empty((x.size(0), width), device=x.device, dtype=x.dtype)
+    call("lfm2_swiglu", out, x, x.size(0), width, _code(x.dtype))
+    return out
+
+
+def swiglu_fp8(x: torch.Tensor):
+    """lfm25_fp8.py:67-73."""
+    _check(x)
+    width = x.size(1) // 2
+    q = torch.empty((x.size(0), width), device=x.device, dtype=FP8)
+    scales = torch.empty(x.size(0), device=x.device, dtype=torch.float32)
+    call("lfm2_swiglu_fp8", q, scales, x, x.size(0), width, _code(x.dtype))
+    return q, scales
+
+
+def quantize_rows(x: torch.Tensor, *, out: tuple[torch.Tensor, torch.Tensor] | None = None):
+    """lfm25_fp8.py:108-117, including its argument errors."""
+    if x.ndim != 2 or not x.is_cuda or not x.is_contiguous() or x.dtype not in (torch.bfloat16, torch.float16):
+        raise ValueError("FP8 quantization requires a contiguous 2D CUDA BF16/FP16 tensor")
+    if min(x.shape) <= 0 or x.size(1) > 32768:
+        raise ValueError("FP8 row width must be in [1, 32768]")
+    if out is None:
+        out = (torch.empty(x.shape, device=x.device, dtype=FP8),
+               torch.empty(x.size(0), device=x.device, dtype=torch.float32))
+    call("lfm2_quantize_rows", out[0], out[1], x, x.size(0), x.size(1), _code(x.dtype))
+    return out
+
+
+def conv_update(bcx, weight, state, active=None, slot_ids=None):
+    """lfm25_cuda_kernels.py:103-110: one gated short-conv step; `state` [slots,H,3] is updated in place."""
+    _check(bcx, weight, state, active, slot_ids)
+    width = weight.size(0)
+    out = torch.empty((bcx.size(0), width), device=bcx.device, dtype=bcx.dtype)
+    call("lfm2_conv_update", out, bcx, weight, state, active, slot_ids, bcx.size(0), width, state.size(0),
+         _code(bcx.dtype))
+    return out
+
+
+def prepare_qkv(x, q_weight, k_weight, cos, sin, positions, q_heads: int, kv_heads: int, head_dim: int, eps: float):
+    """lfm25_cuda_kernels.py:143-151: QK RMSNorm + rotate-half RoPE + split; q/k/v come back as [M,1,heads,D]."""
+    _check(x, q_weight, k_weight, cos, sin, positions)
+    if positions.dtype != torch.int32:
+        raise ValueError("positions must be int32")
+    m = x.size(0)
+    q = torch.empty((m, 1, q_heads, head_dim), device=x.device, dtype=x.dtype)
+    k = torch.empty((m, 1, kv_heads, head_dim), device=x.device, dtype=x.dtype)
+    v = torch.empty_like(k)
+    call("lfm2_prepare_qkv", q, k, v, x, q_weight, k_weight, cos, sin, positions, m, q_heads, kv_heads, head_dim,
+         cos.size(0), float(eps), _code(x.dtype))
+    return q, k, v
+
+
+def conv_prefill(bcx, weight, state, cu_seqlens, seq_of_token, slots):
+    """Packed-batch form of lfm25_engine.py:1478-1511: causal depthwise conv over each sequence of a varlen
+    batch, gate, and the last three b*x of every sequence into `state[slots[seq]]`."""
+    _check(bcx, weight, state, cu_seqlens, seq_of_token, slots)
+    width = weight.size(0)
+    out = torch.empty((bcx.size(0), width), device=bcx.device, dtype=bcx.dtype)
+    call("lfm2_conv_prefill", out, state, bcx, weight, cu_seqlens, seq_of_token, slots, bcx.size(0),
+         cu_seqlens.numel() - 1, width, state.size(0), _code(bcx.dtype))
+    return out
+
+
+# ----------------------------------------------------------------------------------- GEMMs
+def linear(x: torch.Tensor, weight: torch.Tensor, *, tile: int = -1, split_k: int = 0) -> torch.Tensor:
+    """lfm25_cuda_kernels.py:19-29: y = x W^T.  bf16 runs the MFMA kernel of this package; other dtypes
+    (only used by tests of the fp32 plumbing) go to the vendor GEMM."""
+    if x.dtype != torch.bfloat16:
+        return torch.nn.functional.linear(x, weight)
+    _check(x, weight)
+    m, k = _rows(x), x.size(-1)
+    n = weight.size(0)
+    if weight.size(1) != k:
+        raise ValueError("activation and weight widths differ")
+    out = torch.empty((*x.shape[:-1], n), device=x.device, dtype=x.dtype)
+    need = query("lfm2_bf16_gemm_workspace", m, n, k) if split_k == 0 else max(split_k, 1) * m * n
+    ws = torch.empty(need, device=x.device, dtype=torch.float32) if need and split_k != 1 else None
+    call("lfm2_bf16_gemm", out, x, weight, ws, m, n, k, tile, split_k)
+    return out
+
+
+@dataclass
+class PackedFP8Weight:
+    """lfm25_fp8.py:120-168: per-output-channel e4m3 copy of a weight.  `refresh()` re-quantises into the
+    same buffers so captured graphs keep seeing current weights."""
+    original: torch.Tensor
+    values: torch.Tensor
+    scales: torch.Tensor
+
+    @classmethod
+    def from_weight(cls, weight: torch.Tensor):
+        values, scales = quantize_rows(weight)
+        return cls(weight, values, scales)
+
+    def refresh(self):
+        quantize_rows(self.original, out=(self.values, self.scales))
+
+    def linear(self, x: torch.Tensor, *, config=None):
+        values, scales = quantize_rows(x)
+        return self.linear_quantized(values, scales, dtype=x.dtype, config=config)
+
+    def linear_quantized(self, x, scales, *, dtype=torch.bfloat16, config=None):
+        """config = (tile index, split_k) overrides the default tile choice."""
+        batch, width = x.shape
+        rows = self.values.size(0)
+        if width != self.values.size(1):
+            raise ValueError("FP8 activation and weight widths differ")
+        tile, split_k = (-1, 0) if config is None else (int(config[0]), int(config[1]) if len(config) > 1 else 0)
+        out = torch.empty((batch, rows), device=x.device, dtype=dtype)
+        need = query("lfm2_fp8_gemm_workspace", batch, rows, width) if split_k == 0 else max(split_k, 1) * batch * rows
+        ws = torch.empty(need, device=x.device, dtype=torch.float32) if need and split_k != 1 else None
+        call("lfm2_fp8_gemm", out, x, scales, self.values, self.scales, ws, batch, rows, width, _code(dtype), tile, split_k)
+        return out
+
+
+# ----------------------------------------------------------------------------------- KV cache + attention
+def _cache_strides(cache: torch.Tensor):
+    if cache.ndim != 4 or cache.stride(3) != 1:
+        raise ValueError("cache views must be [slots, positions, heads, dim] with a contiguous last dimension")
+    return cache.stride(0), cache.stride(1), cache.stride(2)
+
+
+def store_kv(k, v, k_cache, v_cache, k_scales, v_scales, *, positions=None, active=None, slot_ids=None):
+    """lfm25_fp8_kv.py:58-69: write [batch, tokens, KV heads, dim] as e4m3 rows with fp32 scales into (possibly
+    strided) cache views; append mode when `positions` is given."""
+    batch, tokens, heads, dim = k.shape
+    if k.stride(3) != 1 or v.stride(3) != 1:
+        raise ValueError("k and v need a contiguous head dimension")
+    c0, c1, c2 = _cache_strides(k_cache)
+    call("lfm2_store_kv_fp8", k, v, k_cache, v_cache, k_scales, v_scales, positions, active, slot_ids, batch, tokens,
+         heads, dim, *k.stride()[:3], *v.stride()[:3], c0, c1, c2, _code(k.dtype))
+
+
+def append_bf16_kv(k, v, k_cache, v_cache, positions, slots, active):
+    """lfm25_batching.py:66-69 (also the in-kernel append of flash_attn_with_kvcache); slots/active may be None."""
+    _check(k, v)
+    c0, c1, c2 = _cache_strides(k_cache)
+    call("lfm2_append_kv", k, v, k_cache, v_cache, positions, slots, active, k.size(0), k.size(-2), k.size(-1),
+         c0, c1, c2, _code(k.dtype))
+
+
+def store_kv_packed(k, v, k_cache, v_cache, k_scales, v_scales, cu_seqlens, seq_of_token, slots):
+    """Cache write of a varlen prefill batch (LFM25HybridCache.store_prefill, lfm25_engine.py:387-398):
+    k, v are [tokens, KV heads, dim] packed by cu_seqlens; sequence i goes to cache slot slots[i]."""
+    _check(k, v)
+    c0, c1, c2 = _cache_strides(k_cache)
+    call("lfm2_store_kv_packed", k, v, k_cache, v_cache, k_scales, v_scales, cu_seqlens, seq_of_token, slots,
+         k.size(0), k.size(1), k.size(2), c0, c1, c2, int(k_scales is not None), _code(k.dtype))
+
+
+def attend(q, k_cache, v_cache, k_scales, v_scales, positions, *, active=None, scale=None, config=None,
+           slot_ids=None, window=0, block_table=None, page=16):
+    """lfm25_fp8_kv.py:138-167 (e4m3 history + scales) and flash_attn_with_kvcache of lfm25_cuda.py:156-165
+    (`k_scales is None`: history in the model dtype).  Attends over positions [0, positions[b]]; inactive rows
+    return zeros.  With `block_table` the caches are page pools [pages, page, KV heads, dim]."""
+    if window:
+        raise ValueError("sliding windows belong to LFM3 and are not part of this path")
+    batch, _, query_heads, dim = q.shape
+    _check(q, positions)
+    heads = k_cache.size(2)
+    c0, c1, c2 = _cache_strides(k_cache)
+    capacity = k_cache.size(1) if block_table is None else block_table.size(1) * page
+    out = torch.empty_like(q)
+    ws = torch.empty(query("lfm2_decode_attention_workspace", batch, query_heads, dim, capacity),
+                     device=q.device, dtype=torch.float32)
+    call("lfm2_decode_attention", out, q, k_cache, v_cache, k_scales, v_scales, positions, active, slot_ids,
+         block_table, 0 if block_table is None else block_table.size(1), page, ws, batch, query_heads, heads, dim,
+         capacity, c0, c1, c2, float(scale if scale is not None else dim ** -0.5), int(k_scales is not None),
+         _code(q.dtype))
+    return out
+
+
+def decode(q, k, v, k_cache, v_cache, k_scales, v_scales, positions, *, active=None, scale=None, slot_ids=None, window=0):
+    """lfm25_fp8_kv.py:170-172: append the new token, then attend."""
+    store_kv(k, v, k_cache, v_cache, k_scales, v_scales, positions=positions, active=active, slot_ids=slot_ids)
+    return attend(q, k_cache, v_cache, k_scales, v_scales, positions, active=active, scale=scale, slot_ids=slot_ids,
+                  window=window)
+
+
+def prefill_attention(q, k, v, cu_seqlens, max_seqlen: int, scale: float | None = None):
+    """Varlen causal GQA attention (flash_attn_func of lfm25_engine.py:1415-1417 on a packed batch):
+    q [tokens, QH, D], k/v [tokens, KH, D], cu_seqlens int32."""
+    _check(q, k, v, cu_seqlens)
+    out = torch.empty_like(q)
+    call("lfm2_prefill_attention", out, q, k, v, cu_seqlens, cu_seqlens.numel() - 1, int(max_seqlen), q.size(1),
+         k.size(1), q.size(2), float(scale if scale is not None else q.size(2) ** -0.5), _code(q.dtype))
+    return out
+
+
+# ----------------------------------------------------------------------------------- batch metadata
+def build_token_map(cu_seqlens: torch.Tensor, total: int):
+    """Device-side expansion of cu_seqlens into (sequence index, position) per packed token."""
+    seq = torch.empty(total, device=cu_seqlens.device, dtype=torch.int32)
+    pos = torch.empty_like(seq)
+    call("lfm2_build_token_map", seq, pos, cu_seqlens, cu_seqlens.numel() - 1, total)
+    return seq, pos
+
+
+def gather_inputs(tokens, positions, mask, input_tokens, lengths, active, slots):
+    """lfm25_batching.py:11-22 (writes into the three preallocated row buffers)."""
+    call("lfm2_gather_inputs", tokens, positions, mask, input_tokens, lengths, active, slots, slots.numel())
+
+
+def scatter_logits(saved, logits, slots, active):
+    """lfm25_batching.py:25-32; `slots=None` is `where(active[:,None], logits, saved)` of lfm25_cuda.py:243."""
+    call("lfm2_scatter_logits", saved, logits, slots, active, logits.size(0), logits.size(1), _code(logits.dtype))
+
+
+def advance_positions(lengths, positions, slots, active):
+    """lfm25_batching.py:44-46; `slots=None` advances row i itself (lfm25_cuda.py:185-186)."""
+    call("lfm2_advance_positions", lengths, positions, slots, active, positions.numel())
+
+
+# ----------------------------------------------------------------------------------- sampling
+def _sample_scratch(batch: int, vocab: int, device):
+    return torch.empty(batch * ((vocab + 4095) // 4096) * 4, device=device, dtype=torch.float32)
+
+
+def sample_logits(logits: torch.Tensor, *, temperature: float, seed: int, step: int, return_logprobs: bool):
+    """lfm25_sampling.py:61-92: greedy (first maximum) or Gumbel-max over the full support; log-probabilities
+    are the raw log-softmax of the chosen token.  Deterministic in (seed, step)."""
+    if logits.ndim != 2 or not logits.is_cuda or logits.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        raise ValueError("sampling requires a 2D CUDA BF16/FP16/FP32 logits tensor")
+    logits = logits.contiguous()
+    batch, vocab = logits.shape
+    if batch == 0 or vocab == 0 or temperature < 0:
+        raise ValueError("sampling requires nonempty logits and nonnegative temperature")
+    tokens = torch.empty(batch, device=logits.device, dtype=torch.long)
+    logprobs = torch.empty(batch, device=logits.device, dtype=torch.float32) if return_logprobs else None
+    call("lfm2_sample", tokens, logprobs, logits, _sample_scratch(batch, vocab, logits.device), None, None, None,
+         int(seed) & 0x7FFFFFFFFFFFFFFF, int(step), float(temperature), batch, vocab, _code(logits.dtype))
+    return tokens, logprobs
+
+
+class RowSampler:
+    """lfm25_sampling.py:95-123: per-row seeds/steps/temperatures; returns buffers that are reused."""
+
+    def __init__(self, logits):
+        self.batch, self.vocab = logits.shape
+        self.scratch = _sample_scratch(self.batch, self.vocab, logits.device)
+        self.tokens = torch.empty(self.batch, device=logits.device, dtype=torch.long)
+        self.logprobs = torch.empty(self.batch, device=logits.device, dtype=torch.float32)
+
+    def sample(self, logits, seeds, steps, temperatures):
+        call("lfm2_sample", self.tokens, self.logprobs, logits, self.scratch, seeds, steps, temperatures, 0, 0, 1.0,
+             self.batch, self.vocab, _code(logits.dtype))
+        return self.tokens, self.logprobs
+
+
+def sample_filtered(logits, *, temperature: float, top_k: int, top_p: float, seed: int = 0, step: int = 0,
+                    seeds=None, steps=None, return_kept: bool = False, out=None):
+    """Device form of `_sample` + `_apply_top_k_top_p` (lfm25_engine.py:1574-1609, 1759-1774) for temperature > 0:
+    returns (tokens, raw log-probabilities[, survivors per row])."""
+    if logits.ndim != 2 or not logits.is_cuda:
+        raise ValueError("sampling requires a 2D GPU logits tensor")
+    logits = logits.contiguous()
+    batch, vocab = logits.shape
+    tokens, logprobs = out if out is not None else (
+        torch.empty(batch, device=logits.device, dtype=torch.long),
+        torch.empty(batch, device=logits.device, dtype=torch.float32))
+    kept = torch.empty(batch, device=logits.device, dtype=torch.int32) if return_kept else None
+    call("lfm2_sample_filtered", tokens, logprobs, kept, logits, seeds, steps, int(seed) & 0x7FFFFFFFFFFFFFFF,
+         int(step), float(temperature), int(top_k), float(top_p), batch, vocab, _code(logits.dtype))
+    return (tokens, logprobs, kept) if return_kept else (tokens, logprobs)
+
+
+def behavior_topk(logits, selected, logprobs, k):
+    """lfm25_sampling.py:137-149: top-k ids with log-probabilities that reuse the sampler's normaliser."""
+    if not 0 < k <= min(logits.size(1), 128):
+        raise ValueError('Behavior head exceeds the vocabulary or supported size')
+    values, ids = torch.topk(logits, k, dim=-1, sorted=True)
+    probs = torch.empty(values.shape, dtype=torch.float32, device=logits.device)
+    call("lfm2_head_logprobs", probs, logits, selected, logprobs, values.contiguous(), logits.size(0), logits.size(1),
+         k, _code(logits.dtype))
+    return ids, probs
+
+
+def record_sample(sampled, logp, tokens, logprobs, lengths, limits, reasons, alive, pending, input_tokens,
+                  stop_states, stop_offsets, stop_table, ignore_eos, rng_positions, eos: int, vocab: int, cap: int):
+    """lfm25_session.py:34-56."""
+    call("lfm2_record_sample", sampled, logp, tokens, logprobs, lengths, limits, reasons, alive, pending, input_tokens,
+         stop_states, stop_offsets, stop_table, ignore_eos, rng_positions, int(eos), int(vocab), int(cap),
+         sampled.numel())
+
+
+def record_head(ids, probs, out_ids, out_probs, lengths, alive, k: int, cap: int):
+    """lfm25_session.py:22-31."""
+    call("lfm2_record_head", ids.contiguous(), probs.contiguous(), out_ids, out_probs, lengths, alive, int(k),
+         int(cap), lengths.numel())

@@ -1,0 +1,192 @@
+/* C ABI of the gfx950 kernels behind the LFM2 continuous-batching decode/prefill step.
+ *
+ * The reference (lms21a/climbing-gym) has no FFI for this path: its seam is the set of
+ * module-level Python functions that launch Triton kernels or call FlashAttention.  Each
+ * entry point below replaces one of those functions; the comment names it as
+ * file:line under src/climbing_gym/inference/ of the reference.
+ *
+ * Conventions
+ *   - every pointer is a device pointer unless stated; tensors are row-major contiguous
+ *     unless strides are passed;
+ *   - `stream` is a hipStream_t; launches are stream-ordered, never synchronise, never
+ *     allocate, and can be recorded into a hipGraph;
+ *   - `dtype` is one of LFM2_DTYPE_*; fp8 means OCP e4m3 (finite only, max 448);
+ *   - return value: LFM2_OK, or a negative code with text in lfm2_last_error().
+ */
+#ifndef LFM2_HIP_H
+#define LFM2_HIP_H
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { LFM2_OK = 0, LFM2_ERR_ARGUMENT = -1, LFM2_ERR_LAUNCH = -2, LFM2_ERR_UNSUPPORTED = -3 };
+enum { LFM2_DTYPE_BF16 = 0, LFM2_DTYPE_F16 = 1, LFM2_DTYPE_F32 = 2 };
+
+const char* lfm2_last_error(void);
+int lfm2_abi_version(void);
+
+/* ---------------------------------------------------------------- embedding / norms / MLP glue */
+
+/* F.embedding(tokens, table) of lfm25_cuda.py:134.  tokens int64[M], table [V,H] -> out [M,H]. */
+int lfm2_embedding(void* out, const void* table, const int64_t* tokens, int64_t M, int64_t H, int64_t V,
+                   int dtype, void* stream);
+
+/* rms_norm of lfm25_cuda_kernels.py:32-55.  residual may be NULL (then summed is ignored).
+ * out = round(x' * rsqrt(mean(x'^2)+eps)) * w with x' = round(x + residual); summed = x'. */
+int lfm2_rms_norm(void* out, void* summed, const void* x, const void* weight, const void* residual,
+                  int64_t M, int64_t H, float eps, int dtype, void* stream);
+
+/* rms_norm_fp8 of lfm25_fp8.py:27-41,57-64: same, then per-row e4m3 with scale=max(amax/448,1e-12).
+ * q uint8[M,H], scales float[M]. */
+int lfm2_rms_norm_fp8(uint8_t* q, float* scales, void* summed, const void* x, const void* weight,
+                      const void* residual, int64_t M, int64_t H, float eps, int dtype, void* stream);
+
+/* swiglu of lfm25_cuda_kernels.py:58-72.  x [M,2I] (gate first) -> out [M,I]. */
+int lfm2_swiglu(void* out, const void* x, int64_t M, int64_t I, int dtype, void* stream);
+
+/* swiglu_fp8 of lfm25_fp8.py:45-54,67-73. */
+int lfm2_swiglu_fp8(uint8_t* q, float* scales, const void* x, int64_t M, int64_t I, int dtype, void* stream);
+
+/* quantize_rows of lfm25_fp8.py:17-23,108-117.  x [M,K] -> q uint8[M,K], scales float[M]. */
+int lfm2_quantize_rows(uint8_t* q, float* scales, const void* x, int64_t M, int64_t K, int dtype, void* stream);
+
+/* conv_update of lfm25_cuda_kernels.py:75-110.  bcx [M,3H] in (B,C,x) thirds, weight [H,3],
+ * state [slots,H,3] updated in place for active rows; active uint8[M] or NULL; slot_ids int32[M]
+ * or NULL (negative ids read slot 0 and must be inactive). */
+int lfm2_conv_update(void* out, const void* bcx, const void* weight, void* state, const uint8_t* active,
+                     const int32_t* slot_ids, int64_t M, int64_t H, int64_t slots, int dtype, void* stream);
+
+/* prepare_qkv of lfm25_cuda_kernels.py:113-151.  x [M,(QH+2KH)*D]; cos/sin float[P,D/2];
+ * positions int32[M] -> q [M,QH,D], k [M,KH,D], v [M,KH,D]. */
+int lfm2_prepare_qkv(void* q, void* k, void* v, const void* x, const void* q_weight, const void* k_weight,
+                     const float* cos, const float* sin, const int32_t* positions, int64_t M, int QH, int KH,
+                     int D, int64_t max_positions, float eps, int dtype, void* stream);
+
+/* Packed-prefill short conv (F.conv1d path of lfm25_engine.py:1478-1511 on a varlen batch).
+ * bcx [T,3H]; seq_of_token/pos_of_token int32[T]; seq_start int32[nseq+1] (cu_seqlens);
+ * out [T,H]; state rows state[slots[seq]] receive the last three b*x of each sequence
+ * (zero filled for shorter ones). */
+int lfm2_conv_prefill(void* out, void* state, const void* bcx, const void* weight, const int32_t* cu_seqlens,
+                      const int32_t* seq_of_token, const int32_t* slots, int64_t T, int64_t nseq, int64_t H,
+                      int64_t nslots, int dtype, void* stream);
+
+/* ---------------------------------------------------------------- GEMMs */
+
+/* PackedFP8Weight.linear_quantized of lfm25_fp8.py:77-105,141-168:
+ * out[M,N] = (a_q[M,K] . w_q[N,K]^T) * a_scales[m] * w_scales[n], e4m3 x e4m3 -> fp32 MFMA.
+ * workspace: float[split_k*M*N] when split_k > 1 (NULL otherwise); split_k <= 0 picks a default.
+ * tile < 0 picks a default tile shape, otherwise an index into the table in gemm.hip. */
+int lfm2_fp8_gemm(void* out, const uint8_t* a_q, const float* a_scales, const uint8_t* w_q,
+                  const float* w_scales, float* workspace, int64_t M, int64_t N, int64_t K, int out_dtype,
+                  int tile, int split_k, void* stream);
+/* Workspace floats lfm2_fp8_gemm needs for a shape under its default choice (0 = none). */
+int64_t lfm2_fp8_gemm_workspace(int64_t M, int64_t N, int64_t K);
+
+/* linear of lfm25_cuda_kernels.py:19-29 (F.linear / GEMV): out[M,N] = x[M,K] . w[N,K]^T, bf16 in,
+ * fp32 MFMA accumulate, bf16 out. */
+int lfm2_bf16_gemm(void* out, const void* x, const void* w, float* workspace, int64_t M, int64_t N, int64_t K,
+                   int tile, int split_k, void* stream);
+int64_t lfm2_bf16_gemm_workspace(int64_t M, int64_t N, int64_t K);
+
+/* ---------------------------------------------------------------- KV cache and attention */
+
+/* store_kv of lfm25_fp8_kv.py:28-69.  k,v [B,T,KH,D] with element strides (ks0,ks1,ks2) / (vs0,..);
+ * caches e4m3 addressed slot*c0 + pos*c1 + head*c2 + d, scales float at the same offset / D.
+ * positions int32[B] or NULL (then pos = token index), active uint8[B] or NULL, slot_ids or NULL. */
+int lfm2_store_kv_fp8(const void* k, const void* v, uint8_t* k_cache, uint8_t* v_cache, float* k_scales,
+                      float* v_scales, const int32_t* positions, const uint8_t* active, const int32_t* slot_ids,
+                      int64_t B, int64_t T, int KH, int D, int64_t ks0, int64_t ks1, int64_t ks2, int64_t vs0,
+                      int64_t vs1, int64_t vs2, int64_t c0, int64_t c1, int64_t c2, int dtype, void* stream);
+
+/* append_bf16_kv of lfm25_batching.py:49-69 (also the in-kernel append of flash_attn_with_kvcache,
+ * lfm25_cuda.py:161-165).  k,v [B,KH,D] contiguous; cache element strides (c0,c1,c2). */
+int lfm2_append_kv(const void* k, const void* v, void* k_cache, void* v_cache, const int32_t* positions,
+                   const int32_t* slot_ids, const uint8_t* active, int64_t B, int KH, int D, int64_t c0,
+                   int64_t c1, int64_t c2, int dtype, void* stream);
+
+/* Packed-prefill cache write (LFM25HybridCache.store_prefill, lfm25_engine.py:387-398) for a varlen
+ * batch: token t goes to slot slots[seq_of_token[t]] at position t - cu_seqlens[seq].
+ * kv_fp8 != 0 writes e4m3 + scales like lfm2_store_kv_fp8, otherwise copies in the model dtype. */
+int lfm2_store_kv_packed(const void* k, const void* v, void* k_cache, void* v_cache, float* k_scales,
+                         float* v_scales, const int32_t* cu_seqlens, const int32_t* seq_of_token,
+                         const int32_t* slots, int64_t T, int KH, int D, int64_t c0, int64_t c1, int64_t c2,
+                         int kv_fp8, int dtype, void* stream);
+
+/* attend of lfm25_fp8_kv.py:72-167 (e4m3 history) and flash_attn_with_kvcache of
+ * lfm25_cuda.py:156-165 (history in the model dtype, kv_fp8 = 0).
+ * q [B,QH,D]; history rows [0, positions[b]] of slot slot_ids[b] (or b); out [B,QH,D];
+ * inactive rows produce zeros.  block_table int32[B,max_blocks] or NULL: when given, token t of
+ * row b lives in page block_table[b*max_blocks + t/page] at in-page index t%page and c0 is the
+ * page stride (slot-mapped paged layout).  workspace: lfm2_decode_attention_workspace() floats. */
+int lfm2_decode_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
+                          const float* k_scales, const float* v_scales, const int32_t* positions,
+                          const uint8_t* active, const int32_t* slot_ids, const int32_t* block_table,
+                          int64_t max_blocks, int page, float* workspace, int64_t B, int QH, int KH, int D,
+                          int64_t capacity, int64_t c0, int64_t c1, int64_t c2, float scale, int kv_fp8,
+                          int dtype, void* stream);
+int64_t lfm2_decode_attention_workspace(int64_t B, int QH, int D, int64_t capacity);
+
+/* flash_attn_func(causal=True) of lfm25_engine.py:1415-1417 in varlen form: q [T,QH,D], k,v [T,KH,D]
+ * packed by cu_seqlens int32[nseq+1]; out [T,QH,D]. */
+int lfm2_prefill_attention(void* out, const void* q, const void* k, const void* v, const int32_t* cu_seqlens,
+                           int64_t nseq, int64_t max_seqlen, int QH, int KH, int D, float scale, int dtype,
+                           void* stream);
+
+/* ---------------------------------------------------------------- batch metadata */
+
+/* Expand cu_seqlens int32[nseq+1] into seq_of_token/pos_of_token int32[T] on the device
+ * (replaces the host-side arange/indexing of lfm25_engine.py:659-662). */
+int lfm2_build_token_map(int32_t* seq_of_token, int32_t* pos_of_token, const int32_t* cu_seqlens, int64_t nseq,
+                         int64_t T, void* stream);
+
+/* _gather_inputs of lfm25_batching.py:11-22. */
+int lfm2_gather_inputs(int64_t* tokens, int32_t* positions, uint8_t* mask, const int64_t* input,
+                       const int32_t* lengths, const uint8_t* active, const int32_t* slots, int64_t B,
+                       void* stream);
+/* _scatter_logits of lfm25_batching.py:25-32: saved[slots[row]] = logits[row] for active rows.
+ * slots may be NULL (identity), which gives where(active, logits, saved) of lfm25_cuda.py:243. */
+int lfm2_scatter_logits(void* saved, const void* logits, const int32_t* slots, const uint8_t* active, int64_t B,
+                        int64_t V, int dtype, void* stream);
+/* _advance_positions of lfm25_batching.py:35-46; slots NULL = identity (seq_lens.add_(active),
+ * lfm25_cuda.py:185-186). */
+int lfm2_advance_positions(int32_t* lengths, const int32_t* positions, const int32_t* slots,
+                           const uint8_t* active, int64_t B, void* stream);
+
+/* ---------------------------------------------------------------- sampling and bookkeeping */
+
+/* sample_logits / RowSampler.sample of lfm25_sampling.py:9-123: greedy (temperature 0: first
+ * maximum) or Gumbel-max over the full support; logprobs are raw log-softmax of the pick.
+ * Per-row arrays (seeds int64, steps int64, temperatures float) may be NULL, then the scalar
+ * seed/step/temperature apply.  scratch: float[B*parts*4] with parts = ceil(V/4096). */
+int lfm2_sample(int64_t* tokens, float* logprobs, const void* logits, float* scratch, const int64_t* seeds,
+                const int64_t* steps, const float* temperatures, int64_t seed, int64_t step, float temperature,
+                int64_t B, int64_t V, int dtype, void* stream);
+
+/* _sample + _apply_top_k_top_p of lfm25_engine.py:1574-1609,1759-1774 on the device: temperature,
+ * top-k (ties with the k-th value kept), nucleus (rank 0 never dropped), then a Gumbel-max draw
+ * from what is left.  kept_count int32[B] (may be NULL) reports the survivors. */
+int lfm2_sample_filtered(int64_t* tokens, float* logprobs, int32_t* kept_count, const void* logits,
+                         const int64_t* seeds, const int64_t* steps, int64_t seed, int64_t step,
+                         float temperature, int top_k, float top_p, int64_t B, int64_t V, int dtype,
+                         void* stream);
+
+/* _head_logprobs of lfm25_sampling.py:126-149: out[b,j] = values[b,j] - logZ(b). */
+int lfm2_head_logprobs(float* out, const void* logits, const int64_t* selected, const float* logprobs,
+                       const void* values, int64_t B, int64_t V, int K, int dtype, void* stream);
+
+/* _record_sample of lfm25_session.py:34-56. */
+int lfm2_record_sample(const int64_t* sampled, const float* logp, int64_t* tokens, float* logprobs,
+                       int32_t* lengths, const int32_t* limits, int8_t* reasons, uint8_t* alive,
+                       uint8_t* pending, int64_t* input, int64_t* stop_states, const int64_t* stop_offsets,
+                       const int32_t* stop_table, const uint8_t* ignore_eos, int64_t* rng_positions,
+                       int64_t eos, int64_t V, int64_t cap, int64_t B, void* stream);
+/* _record_head of lfm25_session.py:22-31. */
+int lfm2_record_head(const int64_t* ids, const float* probs, int32_t* out_ids, float* out_probs,
+                     const int32_t* lengths, const uint8_t* alive, int K, int64_t cap, int64_t B, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,509 @@
+"""GPU parity tests: every HIP kernel, called through the C ABI, against the CPU oracle on the same
+seeded inputs.  The cases follow the reference's own kernel tests (tests/test_lfm25_cuda.py:19-63,
+316-347, tests/test_lfm25_fp8.py:14-56, tests/test_lfm25_fp8_kv.py:27-88).
+
+Bars: integer/index outputs exact; e4m3 codes and model-dtype roundings bit-exact except where a
+differently ordered fp32 reduction moves a value across a rounding boundary (bounded below as a
+fraction of elements and by one unit in the last place); fp32 within the stated tolerances.
+"""
+import math
+
+import pytest
+import torch
+
+from oracle import lfm2_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from climbing_gym_amd import ops as module
+    return module
+
+
+TOL = {torch.float32: (2e-5, 1e-5), torch.bfloat16: (0.04, 0.01), torch.float16: (0.004, 0.01)}
+
+
+def _close_mostly_exact(actual, expected, dtype, max_fraction=2e-3):
+    """Within the reference's kernel-test tolerances (tests/test_lfm25_cuda.py:31-32) everywhere and, for
+    the 16-bit dtypes, bit-exact except for rare flips caused by the order of an fp32 reduction."""
+    a, e = actual.float().cpu(), expected.float().cpu()
+    atol, rtol = TOL[dtype]
+    torch.testing.assert_close(a, e, atol=atol, rtol=rtol)
+    if dtype != torch.float32:
+        frac = (a != e).float().mean().item()
+        assert frac <= max_fraction, f"{frac:.2e} of elements differ from the oracle"
+
+
+@pytest.mark.parametrize("dtype", (torch.float32, torch.bfloat16, torch.float16))
+@torch.inference_mode()
+def test_fused_decode_kernels_match_oracle(ops, dtype):
+    torch.manual_seed(17)
+    batch, width = 3, 2048
+    x, residual = torch.randn(batch, width, dtype=dtype), torch.randn(batch, width, dtype=dtype)
+    weight = torch.randn(width, dtype=dtype)
+    out, summed = ops.rms_norm(x.to(DEV), weight.to(DEV), 1e-5, residual.to(DEV))
+    eo, es = O.k_rms_norm(x, weight, 1e-5, residual)
+    assert torch.equal(summed.cpu(), es)
+    _close_mostly_exact(out, eo, dtype)
+    out2, same = ops.rms_norm(x.to(DEV), weight.to(DEV), 1e-5)
+    assert same.data_ptr() != out2.data_ptr()
+    _close_mostly_exact(out2, O.k_rms_norm(x, weight, 1e-5)[0], dtype)
+
+    projected = torch.randn(batch, 2 * 10752, dtype=dtype)
+    _close_mostly_exact(ops.swiglu(projected.to(DEV)), O.k_swiglu(projected), dtype, 5e-3)
+
+    bcx = torch.randn(batch, width * 3, dtype=dtype)
+    state = torch.randn(batch, width, 3, dtype=dtype)
+    conv_w = torch.randn(width, 3, dtype=dtype)
+    dstate = state.to(DEV)
+    got = ops.conv_update(bcx.to(DEV), conv_w.to(DEV), dstate)
+    want = O.k_conv_update(bcx, conv_w, state)
+    assert torch.equal(dstate.cpu(), state)
+    assert torch.equal(got.cpu(), want)
+
+    QH, KH, D = 32, 8, 64
+    qkv = torch.randn(batch, (QH + 2 * KH) * D, dtype=dtype)
+    qw, kw = torch.randn(D, dtype=dtype), torch.randn(D, dtype=dtype)
+    pos = torch.tensor([3, 27, 101], dtype=torch.int32)
+    cos, sin = O.rope_tables(D, 1e7, 128)
+    q, k, v = ops.prepare_qkv(qkv.to(DEV), qw.to(DEV), kw.to(DEV), cos.to(DEV), sin.to(DEV), pos.to(DEV), QH, KH, D, 1e-5)
+    eq, ek, ev = O.k_prepare_qkv(qkv, qw, kw, cos, sin, pos, QH, KH, D, 1e-5)
+    assert q.shape == (batch, 1, QH, D) and k.shape == (batch, 1, KH, D)
+    assert torch.equal(v.cpu(), ev)
+    _close_mostly_exact(q, eq, dtype, 5e-3)
+    _close_mostly_exact(k, ek, dtype, 5e-3)
+
+
+@torch.inference_mode()
+def test_conv_update_masks_rows_and_follows_slot_ids(ops):
+    torch.manual_seed(3)
+    H = 256
+    state = torch.randn(5, H, 3).bfloat16()
+    bcx = torch.randn(3, 3 * H).bfloat16()
+    w = torch.randn(H, 3).bfloat16()
+    active = torch.tensor([True, False, True])
+    slots = torch.tensor([4, 2, -1], dtype=torch.int32)
+    active[2] = False  # padding rows are inactive and read slot 0
+    dstate = state.to(DEV)
+    got = ops.conv_update(bcx.to(DEV), w.to(DEV), dstate, active.to(DEV), slots.to(DEV))
+    want = O.k_conv_update(bcx, w, state, active, slots)
+    assert torch.equal(dstate.cpu(), state) and torch.equal(got.cpu(), want)
+
+
+@pytest.mark.parametrize("width", (129, 2048, 16384))
+@torch.inference_mode()
+def test_fused_activation_quantization_matches_separate_kernels_and_oracle(ops, width):
+    # tests/test_lfm25_fp8.py:14-33: the fused forms are bitwise the two-step forms
+    torch.manual_seed(10)
+    x, residual = torch.randn(17, width).bfloat16(), torch.randn(17, width).bfloat16()
+    weight = torch.randn(width).bfloat16()
+    dx, dr, dw = x.to(DEV), residual.to(DEV), weight.to(DEV)
+    normalized, expected_sum = ops.rms_norm(dx, dw, 1e-5, dr)
+    if width % 8 == 0:
+        expected, scales = ops.quantize_rows(normalized)
+    else:
+        expected, scales = ops.quantize_rows(normalized.contiguous())
+    actual, actual_scales, summed = ops.rms_norm_fp8(dx, dw, 1e-5, dr)
+    assert torch.equal(summed, expected_sum) and torch.equal(actual_scales, scales)
+    assert torch.equal(actual.view(torch.uint8), expected.view(torch.uint8))
+    oq, oscale, _ = O.k_rms_norm_fp8(x, weight, 1e-5, residual)
+    torch.testing.assert_close(actual_scales.cpu(), oscale, rtol=2 ** -7, atol=0)
+    same_scale = actual_scales.cpu() == oscale
+    assert same_scale.float().mean() > 0.8
+    mismatch = (actual.cpu().view(torch.uint8) != oq.view(torch.uint8))[same_scale].float().mean().item()
+    assert mismatch < 5e-3
+    projected = torch.randn(17, 2 * width).bfloat16()
+    expected, scales = ops.quantize_rows(ops.swiglu(projected.to(DEV)))
+    actual, actual_scales = ops.swiglu_fp8(projected.to(DEV))
+    assert torch.equal(actual_scales, scales) and torch.equal(actual.view(torch.uint8), expected.view(torch.uint8))
+
+
+@torch.inference_mode()
+def test_quantize_rows_is_bit_exact_with_oracle_and_rejects_bad_input(ops):
+    torch.manual_seed(5)
+    x = (torch.randn(33, 1000) * torch.logspace(-4, 3, 33)[:, None]).bfloat16()
+    x[4].zero_()
+    x.view(-1)[::97] *= 20
+    q, s = ops.quantize_rows(x.to(DEV))
+    oq, os_ = O.k_quantize_rows(x)
+    assert torch.equal(s.cpu(), os_)
+    assert torch.equal(q.cpu().view(torch.uint8), oq.view(torch.uint8))
+    with pytest.raises(ValueError):
+        ops.quantize_rows(x)  # CPU tensor
+    with pytest.raises(ValueError):
+        ops.quantize_rows(x.to(DEV).float())
+    with pytest.raises(ValueError):
+        ops.quantize_rows(torch.zeros(2, 40000, device=DEV, dtype=torch.bfloat16))
+
+
+@pytest.mark.parametrize("batch,width,outputs", [(3, 129, 193), (128, 2048, 512), (32, 8192, 128), (1, 2048, 3072),
+                                                 (257, 5632, 2048), (64, 2048, 1040)])
+@torch.inference_mode()
+def test_fp8_projection_matches_independently_dequantized_operands(ops, batch, width, outputs):
+    torch.manual_seed(42)
+    x = torch.randn(batch, width).bfloat16()
+    x.view(-1)[::101] *= 20  # outliers as in the GEMM benchmark inputs
+    weight = (torch.randn(outputs, width) * 0.025).bfloat16()
+    x[0].zero_()
+    weight[0].zero_()
+    packed = ops.PackedFP8Weight.from_weight(weight.to(DEV))
+    q, scale = ops.quantize_rows(x.to(DEV))
+    expected = O.k_fp8_linear(q.cpu(), scale.cpu(), packed.values.cpu(), packed.scales.cpu(), torch.float32)
+    actual = packed.linear(x.to(DEV))
+    assert actual.dtype == torch.bfloat16
+    err = (actual.float().cpu() - expected).norm() / expected.norm()
+    assert err < 1e-2  # relative error bar of the FP8 GEMM against the dequantised matmul
+    torch.testing.assert_close(actual.float().cpu(), expected, atol=0.02, rtol=0.015)
+    assert torch.isfinite(actual).all()
+    assert actual[0].count_nonzero() == actual[:, 0].count_nonzero() == 0
+    reference = (x.float() @ weight.float().T)
+    assert (actual.float().cpu() - reference).norm() / reference.norm() < 0.065
+    if width % 16 == 0:
+        for tile in range(6):
+            for split in (1, 2, 4):
+                got = packed.linear_quantized(q, scale, config=(tile, split))
+                torch.testing.assert_close(got.float().cpu(), expected, atol=0.02, rtol=0.015)
+        f32 = packed.linear_quantized(q, scale, dtype=torch.float32)
+        torch.testing.assert_close(f32.cpu(), expected, atol=1e-4, rtol=1e-4)
+
+
+@torch.inference_mode()
+def test_fp8_weight_refresh_reuses_buffers(ops):
+    # tests/test_lfm25_fp8.py:82-90: policy sync re-quantises in place
+    torch.manual_seed(1)
+    w = (torch.randn(64, 256, device=DEV) * 0.02).bfloat16()
+    packed = ops.PackedFP8Weight.from_weight(w)
+    ptrs = (packed.values.data_ptr(), packed.scales.data_ptr())
+    before = packed.values.clone()
+    w.normal_(std=0.05)
+    packed.refresh()
+    assert ptrs == (packed.values.data_ptr(), packed.scales.data_ptr())
+    assert not torch.equal(before.view(torch.uint8), packed.values.view(torch.uint8))
+    oq, os_ = O.k_quantize_rows(w.cpu())
+    assert torch.equal(packed.values.cpu().view(torch.uint8), oq.view(torch.uint8)) and torch.equal(packed.scales.cpu(), os_)
+
+
+@pytest.mark.parametrize("m,k,n", [(1, 2048, 6144), (5, 2048, 512), (256, 2048, 3072), (300, 5632, 2048), (64, 104, 72)])
+@torch.inference_mode()
+def test_bf16_linear_matches_fp32_matmul_of_the_same_operands(ops, m, k, n):
+    torch.manual_seed(7)
+    x, w = torch.randn(m, k).bfloat16(), (torch.randn(n, k) * 0.02).bfloat16()
+    expected = x.float() @ w.float().T
+    for tile, split in [(-1, 0), (0, 1), (2, 2), (4, 1), (5, 4)]:
+        got = ops.linear(x.to(DEV), w.to(DEV), tile=tile, split_k=split)
+        torch.testing.assert_close(got.float().cpu(), expected, atol=2e-3, rtol=2 ** -7)
+
+
+def _cache_tensors(batch, capacity, heads, dim, layout):
+    if layout == "HND":
+        k = torch.zeros(batch, heads, capacity, dim, device=DEV, dtype=torch.float8_e4m3fn).transpose(1, 2)
+        s = torch.zeros(batch, heads, capacity, device=DEV, dtype=torch.float32).transpose(1, 2)
+    else:
+        k = torch.zeros(batch, capacity, heads, dim, device=DEV, dtype=torch.float8_e4m3fn)
+        s = torch.zeros(batch, capacity, heads, device=DEV, dtype=torch.float32)
+    return k, torch.zeros_like(k), s, torch.zeros_like(s)
+
+
+@pytest.mark.parametrize("layout", ["NHD", "HND"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@torch.inference_mode()
+def test_scaled_storage_handles_strided_prefill_views_zeros_and_outliers(ops, layout, dtype):
+    torch.manual_seed(18)
+    kc, vc, ks, vs = _cache_tensors(5, 79, 3, 64, layout)
+    k = torch.randn(2, 37, 3, 64, dtype=dtype)
+    v = torch.randn_like(k)
+    k[0, 0].zero_(), v[0, 0].zero_()
+    k[1, :, 1] *= 100
+    v[1, :, 2] *= 0.0001
+    ops.store_kv(k.to(DEV), v.to(DEV), kc[2:4, :37], vc[2:4, :37], ks[2:4, :37], vs[2:4, :37])
+    ekq, eks, evq, evs = O.k_store_kv(k, v)
+    for values, scales, eq, es in ((kc, ks, ekq, eks), (vc, vs, evq, evs)):
+        assert torch.equal(scales[2:4, :37].cpu(), es)
+        assert torch.equal(values[2:4, :37].cpu().view(torch.uint8), eq.view(torch.uint8))
+        assert torch.count_nonzero(values[:2].float()) == 0
+        assert torch.count_nonzero(values[2:4, 37:].float()) == 0
+        assert torch.count_nonzero(values[4:].float()) == 0
+
+
+@torch.inference_mode()
+def test_append_preserves_inactive_histories_and_uses_independent_positions(ops):
+    kc, vc, ks, vs = _cache_tensors(3, 19, 2, 64, "HND")
+    k = torch.randn(3, 1, 2, 64, device=DEV, dtype=torch.bfloat16)
+    v = torch.randn_like(k)
+    positions = torch.tensor([3, 18, 7], device=DEV, dtype=torch.int32)
+    active = torch.tensor([True, False, True], device=DEV)
+    ops.store_kv(k, v, kc, vc, ks, vs, positions=positions, active=active)
+    assert torch.count_nonzero(kc[1].float()) == 0 and torch.count_nonzero(ks[1]) == 0
+    for row, pos in [(0, 3), (2, 7)]:
+        assert ks[row, pos].min() > 0
+        torch.testing.assert_close(kc[row, pos].float() * ks[row, pos, :, None], k[row, 0].float(), atol=.12, rtol=.05)
+        assert torch.count_nonzero(ks[row, :pos]) == 0 and torch.count_nonzero(ks[row, pos + 1:]) == 0
+    # slot indirection
+    slots = torch.tensor([2, 0, 1], device=DEV, dtype=torch.int32)
+    kc2, vc2, ks2, vs2 = _cache_tensors(3, 19, 2, 64, "NHD")
+    ops.store_kv(k, v, kc2, vc2, ks2, vs2, positions=positions, slot_ids=slots)
+    assert torch.equal(kc2[2, 3].view(torch.uint8), kc[0, 3].view(torch.uint8))
+    assert torch.count_nonzero(ks2[0, 18]) == 2
+
+
+@pytest.mark.parametrize("dim,groups", [(32, 1), (64, 4), (128, 2), (256, 1), (64, 8)])
+@pytest.mark.parametrize("fp8", [True, False])
+@torch.inference_mode()
+def test_decode_matches_independent_fp32_softmax_with_ragged_lengths_and_inactive_rows(ops, dim, groups, fp8):
+    torch.manual_seed(92)
+    batch, capacity, heads = 5, 1300, 2
+    k = torch.randn(batch, capacity, heads, dim).bfloat16()
+    v = torch.randn_like(k)
+    q = torch.randn(batch, 1, heads * groups, dim).bfloat16()
+    positions = torch.tensor([0, 36, 250, 250, 1299], dtype=torch.int32)
+    active = torch.tensor([True, True, True, False, True])
+    if fp8:
+        kc, vc, ks, vs = _cache_tensors(batch, capacity, heads, dim, "HND")
+        ops.store_kv(k.to(DEV), v.to(DEV), kc, vc, ks, vs)
+        hist = (kc.cpu(), vc.cpu(), ks.cpu(), vs.cpu())
+    else:
+        kc, vc, ks, vs = k.to(DEV), v.to(DEV), None, None
+        hist = (k, v, None, None)
+    actual = ops.attend(q.to(DEV), kc, vc, ks, vs, positions.to(DEV), active=active.to(DEV))
+    for row in (0, 1, 2, 4):
+        expected = O.k_attend(q[row, 0], hist[0][row], hist[1][row], int(positions[row]) + 1, dim ** -0.5,
+                              None if hist[2] is None else hist[2][row], None if hist[3] is None else hist[3][row])
+        torch.testing.assert_close(actual[row, 0].float().cpu(), expected, atol=0.012, rtol=0.025)
+    assert torch.count_nonzero(actual[3]) == 0
+    # slot indirection: rows read other slots, a negative slot is padding
+    slots = torch.tensor([4, 2, 1, -1, 0], dtype=torch.int32)
+    pos2 = positions[slots.clamp_min(0).long()]
+    moved = ops.attend(q.to(DEV), kc, vc, ks, vs, pos2.to(DEV), active=torch.tensor([True, True, True, False, True]).to(DEV),
+                       slot_ids=slots.to(DEV))
+    expected = O.k_attend(q[0, 0], hist[0][4], hist[1][4], 1300, dim ** -0.5,
+                          None if hist[2] is None else hist[2][4], None if hist[3] is None else hist[3][4])
+    torch.testing.assert_close(moved[0, 0].float().cpu(), expected, atol=0.012, rtol=0.025)
+    assert torch.count_nonzero(moved[3]) == 0
+
+
+@pytest.mark.parametrize("fp8", [True, False])
+@torch.inference_mode()
+def test_paged_slot_mapped_history_equals_dense_history(ops, fp8):
+    """Block-16 paged layout: the same tokens reached through a shuffled block table give the same output."""
+    torch.manual_seed(4)
+    batch, heads, groups, dim, page = 6, 8, 4, 64, 16
+    lengths = torch.tensor([1, 16, 17, 300, 1000, 777])
+    cap = 1008
+    k = torch.randn(batch, cap, heads, dim).bfloat16()
+    v = torch.randn_like(k)
+    q = torch.randn(batch, 1, heads * groups, dim).bfloat16().to(DEV)
+    positions = (lengths - 1).to(torch.int32).to(DEV)
+    blocks_per_row = cap // page
+    perm = torch.randperm(batch * blocks_per_row)
+    table = perm.view(batch, blocks_per_row).to(torch.int32)
+    if fp8:
+        kc, vc, ks, vs = _cache_tensors(batch, cap, heads, dim, "NHD")
+        ops.store_kv(k.to(DEV), v.to(DEV), kc, vc, ks, vs)
+    else:
+        kc, vc, ks, vs = k.to(DEV), v.to(DEV), None, None
+    dense = ops.attend(q, kc, vc, ks, vs, positions)
+
+    def to_pages(t):  # [batch, cap, ...] -> pool [pages, page, ...] under the block table
+        pool = torch.empty((batch * blocks_per_row, page, *t.shape[2:]), device=DEV, dtype=t.dtype)
+        src = t.reshape(batch * blocks_per_row, page, *t.shape[2:])
+        if t.dtype == torch.float8_e4m3fn:
+            pool.view(torch.uint8)[table.view(-1).long().to(DEV)] = src.view(torch.uint8)
+        else:
+            pool[table.view(-1).long().to(DEV)] = src
+        return pool
+    paged = ops.attend(q, to_pages(kc), to_pages(vc), None if ks is None else to_pages(ks), None if vs is None else to_pages(vs),
+                       positions, block_table=table.to(DEV), page=page)
+    assert torch.equal(paged, dense)
+
+
+@pytest.mark.parametrize("dim,qh,kh", [(64, 32, 8), (64, 4, 2), (32, 4, 4), (128, 4, 1)])
+@torch.inference_mode()
+def test_varlen_prefill_attention_matches_causal_sdpa(ops, dim, qh, kh):
+    torch.manual_seed(11)
+    lengths = [1, 7, 64, 65, 130, 33]
+    total = sum(lengths)
+    q = torch.randn(total, qh, dim).bfloat16()
+    k = torch.randn(total, kh, dim).bfloat16()
+    v = torch.randn(total, kh, dim).bfloat16()
+    cu = torch.tensor([0, *torch.tensor(lengths).cumsum(0).tolist()], dtype=torch.int32)
+    got = ops.prefill_attention(q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), max(lengths)).float().cpu()
+    for i, n in enumerate(lengths):
+        a, b = int(cu[i]), int(cu[i + 1])
+        want = O.causal_attention(q[a:b], k[a:b], v[a:b], dim ** -0.5)
+        torch.testing.assert_close(got[a:b], want, atol=0.02, rtol=0.02)
+
+
+@torch.inference_mode()
+def test_packed_prefill_conv_and_kv_store_match_per_sequence_oracle(ops):
+    torch.manual_seed(12)
+    H, lengths, slots = 128, [1, 2, 5, 3, 40], [4, 0, 2, 5, 1]
+    total = sum(lengths)
+    cu = torch.tensor([0, *torch.tensor(lengths).cumsum(0).tolist()], dtype=torch.int32)
+    bcx = torch.randn(total, 3 * H).bfloat16()
+    w = torch.randn(H, 3).bfloat16()
+    state = torch.ones(6, H, 3, device=DEV, dtype=torch.bfloat16)  # dirty state must be replaced
+    seq, pos = ops.build_token_map(cu.to(DEV), total)
+    assert seq.cpu().tolist() == [i for i, n in enumerate(lengths) for _ in range(n)]
+    assert pos.cpu().tolist() == [p for n in lengths for p in range(n)]
+    got = ops.conv_prefill(bcx.to(DEV), w.to(DEV), state, cu.to(DEV), seq, torch.tensor(slots, dtype=torch.int32, device=DEV))
+    b, c, x = bcx.float().chunk(3, -1)
+    bx = (b * x).bfloat16().float()
+    for i, n in enumerate(lengths):
+        a = int(cu[i])
+        padded = torch.cat((torch.zeros(2, H), bx[a:a + n]))
+        conv = sum(padded[j:j + n] * w.float()[:, j] for j in range(3))
+        want = (c[a:a + n] * conv.bfloat16().float()).bfloat16()
+        torch.testing.assert_close(got[a:a + n].cpu().float(), want.float(), atol=2e-2, rtol=2 ** -6)
+        assert torch.equal(state[slots[i]].cpu().float(), padded[-3:].T.contiguous())
+    assert torch.equal(state[3].cpu(), torch.ones(H, 3).bfloat16())
+    # KV store of the same packed batch into fp8 and bf16 caches
+    KH, D = 2, 64
+    k, v = torch.randn(total, KH, D).bfloat16(), torch.randn(total, KH, D).bfloat16()
+    kc, vc, ks, vs = _cache_tensors(6, 48, KH, D, "HND")
+    dslots = torch.tensor(slots, dtype=torch.int32, device=DEV)
+    ops.store_kv_packed(k.to(DEV), v.to(DEV), kc, vc, ks, vs, cu.to(DEV), seq, dslots)
+    kb = torch.zeros(6, 48, KH, D, device=DEV, dtype=torch.bfloat16)
+    vb = torch.zeros_like(kb)
+    ops.store_kv_packed(k.to(DEV), v.to(DEV), kb, vb, None, None, cu.to(DEV), seq, dslots)
+    ekq, eks, evq, evs = O.k_store_kv(k, v)
+    for i, n in enumerate(lengths):
+        a = int(cu[i])
+        assert torch.equal(kc[slots[i], :n].cpu().view(torch.uint8), ekq[a:a + n].view(torch.uint8))
+        assert torch.equal(vs[slots[i], :n].cpu(), evs[a:a + n])
+        assert torch.equal(kb[slots[i], :n].cpu(), k[a:a + n]) and torch.equal(vb[slots[i], :n].cpu(), v[a:a + n])
+        assert torch.count_nonzero(kb[slots[i], n:]) == 0
+
+
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16, torch.float32))
+@torch.inference_mode()
+def test_fused_sampling_greedy_and_raw_logprobs(ops, dtype):
+    torch.manual_seed(45)
+    logits = torch.randn(9, 128003, dtype=dtype)
+    logits[0, :8192] = -torch.inf  # fully masked tiles must not spoil the normaliser
+    logits[1, 12] = logits[1, 125000] = 20  # ties choose the first token
+    tokens, logprobs = ops.sample_logits(logits.to(DEV), temperature=0, seed=0, step=0, return_logprobs=True)
+    et, elp = O.greedy_with_logprob(logits)
+    assert torch.equal(tokens.cpu(), et)
+    torch.testing.assert_close(logprobs.cpu(), elp, atol=3e-6, rtol=2e-6)
+    sampled, raw = ops.sample_logits(logits.to(DEV), temperature=0.7, seed=31, step=4095, return_logprobs=True)
+    expected = logits.float().log_softmax(-1).gather(1, sampled.cpu()[:, None]).squeeze(1)
+    torch.testing.assert_close(raw.cpu(), expected, atol=3e-6, rtol=2e-6)
+    assert (sampled.cpu() >= 8192)[0]
+
+
+@torch.inference_mode()
+def test_fused_categorical_sampling_distribution_and_seed(ops):
+    probabilities = torch.tensor([0.05, 0.15, 0.3, 0.5], device=DEV)
+    logits = (probabilities.log() * 0.7).expand(20000, -1).contiguous()
+    kwargs = dict(temperature=0.7, seed=17, step=0, return_logprobs=False)
+    tokens, logprobs = ops.sample_logits(logits, **kwargs)
+    assert logprobs is None
+    torch.testing.assert_close(tokens.bincount(minlength=4) / tokens.numel(), probabilities, atol=0.012, rtol=0)
+    assert torch.equal(tokens, ops.sample_logits(logits, **kwargs)[0])
+    for seed, step in ((18, 0), (17, 64), (17, 4095)):
+        assert not torch.equal(tokens, ops.sample_logits(logits, **{**kwargs, "seed": seed, "step": step})[0])
+    # per-row streams: a row's draw depends only on its own (seed, step, temperature)
+    sampler = ops.RowSampler(logits[:64])
+    seeds = torch.arange(64, device=DEV)
+    steps = torch.arange(64, device=DEV) * 3
+    temps = torch.full((64,), 0.7, device=DEV)
+    temps[5] = 0.0
+    first = sampler.sample(logits[:64], seeds, steps, temps)[0].clone()
+    perm = torch.randperm(64, device=DEV)
+    second = sampler.sample(logits[:64], seeds[perm], steps[perm], temps[perm])[0]
+    assert torch.equal(second, first[perm]) and first[5].item() == 3
+
+
+@pytest.mark.parametrize("top_k,top_p", [(50, 0.95), (0, 0.9), (5, 1.0), (1, 0.5), (0, 0.3)])
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float32))
+@torch.inference_mode()
+def test_filtered_sampling_keeps_exactly_the_oracle_support(ops, top_k, top_p, dtype):
+    torch.manual_seed(8)
+    rows, vocab, temperature = 48, 5000, 0.8
+    logits = (torch.randn(rows, vocab) * 2.5).to(dtype)
+    filtered = O.top_k_top_p_filter(logits.float() / temperature, top_k, top_p)
+    allowed = torch.isfinite(filtered)
+    draws = []
+    for step in range(40):
+        tok, lp, kept = ops.sample_filtered(logits.to(DEV), temperature=temperature, top_k=top_k, top_p=top_p, seed=5,
+                                            step=step, return_kept=True)
+        draws.append(tok.cpu())
+        assert allowed.gather(1, tok.cpu()[:, None]).all(), "a draw fell outside the oracle's support"
+    # survivors: identical except when ties or fp32 cumulative-sum rounding sit exactly on the nucleus boundary
+    diff = (kept.cpu() - allowed.sum(1)).abs()
+    assert (diff <= 2).all() and (diff == 0).float().mean() >= 0.8
+    expected = logits.float().log_softmax(-1).gather(1, tok.cpu()[:, None])[:, 0]
+    torch.testing.assert_close(lp.cpu(), expected, atol=5e-6, rtol=2e-6)
+    again = ops.sample_filtered(logits.to(DEV), temperature=temperature, top_k=top_k, top_p=top_p, seed=5, step=39)[0]
+    assert torch.equal(again.cpu(), draws[-1])
+    if top_k == 1:
+        assert torch.equal(draws[0], logits.float().argmax(-1))
+
+
+@torch.inference_mode()
+def test_filtered_sampling_distribution_follows_renormalised_survivors(ops):
+    probs = torch.tensor([0.4, 0.3, 0.15, 0.1, 0.05])
+    logits = probs.log().expand(30000, -1).contiguous().to(DEV)
+    tok, _ = ops.sample_filtered(logits, temperature=1.0, top_k=0, top_p=0.75, seed=3, step=1)
+    freq = tok.bincount(minlength=5).float().cpu() / tok.numel()
+    torch.testing.assert_close(freq, torch.tensor([0.4, 0.3, 0, 0, 0]) / 0.7, atol=0.012, rtol=0)
+    tok, _ = ops.sample_filtered(logits, temperature=1.0, top_k=3, top_p=1.0, seed=3, step=2)
+    freq = tok.bincount(minlength=5).float().cpu() / tok.numel()
+    torch.testing.assert_close(freq, torch.tensor([0.4, 0.3, 0.15, 0, 0]) / 0.85, atol=0.012, rtol=0)
+
+
+@torch.inference_mode()
+def test_record_sample_and_slot_bookkeeping_follow_the_integer_oracle(ops):
+    V, cap, B, eos = 16, 6, 5, 7
+    pieces = ['<', '/', 'summary', '>', 'x'] + [''] * 11
+    table = torch.cat((torch.zeros(V, dtype=torch.int32), O.build_stop_table(pieces, ('</summary>',)).reshape(-1)))
+    dev = lambda t: t.to(DEV)
+    tokens = dev(torch.zeros(B, cap, dtype=torch.long)); logprobs = dev(torch.zeros(B, cap))
+    lengths = dev(torch.tensor([0, 5, 2, 0, 3], dtype=torch.int32)); limits = dev(torch.full((B,), 6, dtype=torch.int32))
+    reasons = dev(torch.zeros(B, dtype=torch.int8)); alive = dev(torch.tensor([True, True, True, False, True]))
+    pending = dev(torch.zeros(B, dtype=torch.bool)); inp = dev(torch.full((B,), -1, dtype=torch.long))
+    states = dev(torch.tensor([0, 0, 9, 0, 0])); offsets = dev(torch.tensor([0, 0, V, 0, 0]))
+    ignore = dev(torch.tensor([False, False, False, False, True])); rng = dev(torch.tensor([0, 10, 20, 30, 40]))
+    sampled = dev(torch.tensor([7, 4, 3, 9, 7])); logp = dev(torch.tensor([-1., -2., -3., -4., -5.]))
+    # row 2 sits in the automaton state reached after '</summary' so that '>' completes the stop
+    st = 0
+    for t in [0, 1, 2]:
+        st = int(table[V + st * V + t]) & 65535
+    states[2] = st
+    ops.record_sample(sampled, logp, tokens, logprobs, lengths, limits, reasons, alive, pending, inp, states, offsets,
+                      dev(table), ignore, rng, eos, V, cap)
+    assert reasons.cpu().tolist() == [1, 3, 2, 0, 0]
+    assert alive.cpu().tolist() == [False, False, False, False, True] == pending.cpu().tolist()
+    assert lengths.cpu().tolist() == [1, 6, 3, 0, 4] and rng.cpu().tolist() == [1, 11, 21, 30, 41]
+    assert inp.cpu().tolist() == [7, 4, 3, -1, 7]
+    assert tokens[1, 5].item() == 4 and logprobs[2, 2].item() == -3.0 and tokens[3].sum().item() == 0
+    # gather / scatter / advance over a compact batch
+    slots = dev(torch.tensor([3, -1, 0], dtype=torch.int32))
+    seq_lens = dev(torch.tensor([11, 22, 33, 44], dtype=torch.int32))
+    input_tokens = dev(torch.tensor([5, 6, 7, 8])); act = dev(torch.tensor([True, True, False, True]))
+    t = dev(torch.zeros(3, dtype=torch.long)); p = dev(torch.zeros(3, dtype=torch.int32)); m = dev(torch.zeros(3, dtype=torch.bool))
+    ops.gather_inputs(t, p, m, input_tokens, seq_lens, act, slots)
+    assert t.cpu().tolist() == [8, 0, 5] and p.cpu().tolist() == [44, 0, 11] and m.cpu().tolist() == [True, False, True]
+    logits = dev(torch.randn(3, 100).bfloat16()); saved = dev(torch.zeros(4, 100).bfloat16())
+    ops.scatter_logits(saved, logits, slots, m)
+    assert torch.equal(saved[3], logits[0]) and torch.equal(saved[0], logits[2]) and saved[1:3].count_nonzero() == 0
+    ops.advance_positions(seq_lens, p, slots, m)
+    assert seq_lens.cpu().tolist() == [12, 22, 33, 45]
+    masked = dev(torch.tensor([True, False, True, True]))
+    ops.advance_positions(seq_lens, seq_lens.clone(), None, masked)
+    assert seq_lens.cpu().tolist() == [13, 22, 34, 46]
+
+
+@torch.inference_mode()
+def test_behavior_head_reuses_the_sampler_normaliser(ops):
+    torch.manual_seed(2)
+    logits = torch.randn(4, 3000).bfloat16().to(DEV)
+    tok, lp = ops.sample_logits(logits, temperature=1.0, seed=1, step=0, return_logprobs=True)
+    ids, probs = ops.behavior_topk(logits, tok, lp, 8)
+    want = logits.float().log_softmax(-1).topk(8).values
+    torch.testing.assert_close(probs, want, atol=5e-6, rtol=1e-5)
+    with pytest.raises(ValueError):
+        ops.behavior_topk(logits, tok, lp, 129)
