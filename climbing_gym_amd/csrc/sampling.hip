@@ -318,7 +318,9 @@ sample_filtered_kernel(const T* logits, int64_t* tokens, float* logprobs, int32_
     const uint32_t k = order_key(x);
     if (!(k > kp || (k == kp && i <= cut))) continue;
     uint32_t rnd[4];
-    philox((uint32_t)(i >> 2), (uint32_t)((uint64_t)i >> 34), 0x5eed5eedu, 0u, (uint32_t)key64, (uint32_t)(key64 >> 32), rnd);
+    // per-row streams depend on the row's own (seed, step) only; a shared seed also counts the row
+    philox((uint32_t)(i >> 2), seeds ? 0u : (uint32_t)row, 0x5eed5eedu, seeds ? 0u : (uint32_t)((uint64_t)row >> 32),
+           (uint32_t)key64, (uint32_t)(key64 >> 32), rnd);
     const float score = x + gumbel(rnd[i & 3]);
     if (best_i == 0x7fffffff || score > best) { best = score; best_i = (int)i; }
   }

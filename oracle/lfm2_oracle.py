@@ -123,7 +123,8 @@ def greedy_with_logprob(logits: torch.Tensor):
     """argmax (first index on ties) and raw log-softmax of the pick (``lfm25_engine.py:1591-1597``)."""
     lf = logits.float()
     tok = lf.argmax(-1)
-    return tok, lf.gather(1, tok[:, None])[:, 0] - torch.logsumexp(lf, -1)
+    # the normaliser in float64: an fp32 running sum drops terms below half an ulp of a dominant one
+    return tok, (lf.double().gather(1, tok[:, None])[:, 0] - torch.logsumexp(lf.double(), -1)).float()
 
 
 # --------------------------------------------------------------------------- weights
@@ -482,8 +483,9 @@ def k_swiglu_fp8(x):
 
 
 def k_fp8_linear(xq, xs, wq, ws, dtype=torch.bfloat16):
-    """Dequantised matmul that ``lfm25_fp8.py:77-105`` approximates (fp32 accumulate)."""
-    return ((xq.float() @ wq.float().T) * xs[:, None] * ws[None, :]).to(dtype)
+    """Dequantised matmul that ``lfm25_fp8.py:77-105`` approximates; accumulated in float64 so the
+    expectation itself carries no summation error."""
+    return ((xq.double() @ wq.double().T) * xs.double()[:, None] * ws.double()[None, :]).to(dtype)
 
 
 def k_store_kv(k, v):

