@@ -1,0 +1,528 @@
+"""Token engine of the native LFM2 path on MI355X: prefill, fork, decode step, generate.
+
+Public surface and argument meaning follow the reference's `LFM25Engine`
+(lfm25_engine.py:479-1163); the arithmetic runs in this package's HIP kernels.  Two things differ
+by design and do not change results beyond GEMM rounding:
+
+* prefill runs a *packed* (varlen) batch through the same fused kernels as decode instead of a
+  right-padded batch through eager torch ops; the chunk planner that bounds a prefill by
+  `max_prefill_tokens` is the reference's (lfm25_engine.py:646-665), so chunks are the same;
+* the engine only exists on the GPU in bf16: there is no eager CPU path in this package.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import Any, Sequence
+
+import torch
+
+from . import ops
+from .cache import LFM25HybridCache
+from .config import LFM2Config, LFM25SamplingConfig
+from .weights import LFM25PackedWeights
+
+MAX_PACKED_TOKENS = 32768  # grid limit of the packed prefill kernels per launch
+
+
+@dataclass(frozen=True)
+class LFM25PrefixBatch:
+    cache: LFM25HybridCache
+    next_token_logits: torch.Tensor
+    prompt_lengths: torch.Tensor
+    input_ids: torch.Tensor
+
+    @property
+    def batch_size(self) -> int:
+        return int(self.prompt_lengths.numel())
+
+
+@dataclass
+class LFM25DecodeBatch:
+    cache: LFM25HybridCache
+    active_slot_ids: torch.Tensor
+    prompt_indices: torch.Tensor
+    repeat_indices: torch.Tensor
+    alive: torch.Tensor
+
+    @property
+    def batch_size(self) -> int:
+        return int(self.prompt_indices.numel())
+
+
+@dataclass(frozen=True)
+class LFM25StepOutput:
+    token_ids: torch.Tensor
+    raw_logprobs: torch.Tensor | None
+    sampling_logprobs: torch.Tensor | None
+    finished: torch.Tensor
+    finish_reasons: torch.Tensor
+    logits: torch.Tensor
+
+
+@dataclass(frozen=True)
+class LFM25GenerationOutput:
+    token_ids: torch.Tensor
+    lengths: torch.Tensor
+    logprobs: torch.Tensor | None
+    finish_reasons: torch.Tensor
+    topk_token_ids: torch.Tensor | None = None
+    topk_logprobs: torch.Tensor | None = None
+
+
+def plan_prefill_chunks(lengths: Sequence[int], budget: int):
+    """Contiguous groups (start, end, padded width) with (count * longest) <= budget; a group always takes
+    its first prompt (lfm25_engine.py:646-665)."""
+    groups, start, total = [], 0, len(lengths)
+    while start < total:
+        end, width = start, 0
+        while end < total:
+            widest = max(width, lengths[end])
+            if end > start and (end - start + 1) * widest > budget:
+                break
+            width, end = widest, end + 1
+        groups.append((start, end, width))
+        start = end
+    return groups
+
+
+def flatten_token_batches(input_ids: Sequence[Sequence[int]], *, device=None):
+    """Python prompts -> (flat ids int64, cu_seqlens int32, longest) (lfm25_engine.py:1799-1811)."""
+    if not input_ids:
+        raise ValueError("input_ids must contain at least one prompt")
+    lengths = [len(p) for p in input_ids]
+    if any(n <= 0 for n in lengths):
+        raise ValueError("empty prompts are not supported")
+    device = torch.device(device or "cpu")
+    flat = torch.tensor([t for p in input_ids for t in p], device=device, dtype=torch.long)
+    cu = torch.zeros(len(lengths) + 1, device=device, dtype=torch.int32)
+    cu[1:] = torch.tensor(lengths, device=device, dtype=torch.int32).cumsum(0)
+    return flat, cu, max(lengths)
+
+
+class LFM25Engine:
+    def __init__(self, weights: LFM25PackedWeights, *, max_model_len: int | None = None) -> None:
+        if weights.device.type != "cuda":
+            raise ValueError("this engine runs on the GPU only; weights must live on a HIP device")
+        if weights.dtype != torch.bfloat16:
+            raise ValueError("this engine computes in bfloat16")
+        cfg = weights.config
+        if cfg.conv_kernel_size != 3 or cfg.conv_bias:
+            raise ValueError("the short-conv kernels need bias-free convolutions of width 3")
+        if cfg.head_dim not in (32, 64, 128):
+            raise ValueError("head_dim must be one of {32, 64, 128}")
+        self.weights, self.config = weights, cfg
+        self.device, self.dtype = weights.device, weights.dtype
+        self.max_model_len = int(max_model_len or min(int(cfg.max_position_embeddings), 32768))
+        if self.max_model_len <= 0:
+            raise ValueError("max_model_len must be > 0")
+        if self.max_model_len > int(cfg.max_position_embeddings):
+            raise ValueError("max_model_len cannot exceed config.max_position_embeddings")
+        self._scaling = cfg.head_dim ** -0.5
+        self._cuda_decoder = None
+        self.policy_version = 0
+        # fp32 rotary tables [max_model_len, D/2] (lfm25_engine.py:1004-1012)
+        inv = 1.0 / (cfg.rope_theta ** (torch.arange(0, cfg.head_dim, 2, dtype=torch.float32, device=self.device) / cfg.head_dim))
+        angles = torch.arange(self.max_model_len, dtype=torch.float32, device=self.device)[:, None] * inv[None, :]
+        self._rope_cos, self._rope_sin = angles.cos().contiguous(), angles.sin().contiguous()
+
+    # ------------------------------------------------------------------ construction
+    @classmethod
+    def from_state_dict(cls, config: LFM2Config, state, *, device="cuda", dtype=torch.bfloat16, max_model_len=None):
+        return cls(LFM25PackedWeights.from_state_dict(config, state, device=torch.device(device), dtype=dtype),
+                   max_model_len=max_model_len)
+
+    @classmethod
+    def from_model(cls, model: Any, *, device=None, dtype=None, max_model_len=None):
+        first = next(model.parameters())
+        return cls(LFM25PackedWeights.from_model(model, device=torch.device(device or first.device),
+                                                 dtype=_resolve_dtype(dtype or first.dtype)), max_model_len=max_model_len)
+
+    @classmethod
+    def from_pretrained(cls, model_dir, *, device=None, dtype=None, max_model_len=None):
+        return cls(LFM25PackedWeights.from_pretrained(model_dir, device=torch.device(device or "cuda"),
+                                                      dtype=_resolve_dtype(dtype)), max_model_len=max_model_len)
+
+    # ------------------------------------------------------------------ lifecycle
+    @property
+    def _decoder_busy(self) -> bool:
+        return self._cuda_decoder is not None and self._cuda_decoder._active_session is not None
+
+    @torch.inference_mode()
+    def sync_from_model(self, model: Any, *, drain_timeout: int | float = 300) -> "LFM25Engine":
+        """In-place policy sync; captured graphs keep working and see the new weights (lfm25_engine.py:556-578)."""
+        timeout = float(drain_timeout)
+        if not math.isfinite(timeout) or timeout < 0.0:
+            raise ValueError("drain_timeout must be finite and >= 0")
+        if self._decoder_busy:
+            raise RuntimeError("Close the native generation session before synchronizing weights")
+        self.weights.copy_from_model_(model)
+        if self._cuda_decoder is not None:
+            self._cuda_decoder.refresh_weights()
+        self.policy_version += 1
+        return self
+
+    def enable_cuda_graphs(self, *, max_graphs: int = 2, bf16_weight_packing: bool = True, max_prefill_tokens: int = 4096,
+                           fp8_mlp: bool = False, fp8_kv: bool = False, adaptive_batching: bool = False,
+                           fp8_lm_head: bool = False, fp8_operators: bool = False, capture: bool = True) -> None:
+        """Same switch as the reference (lfm25_engine.py:980-997); graphs are HIP graphs.  `fp8_operators` extends
+        W8A8 to the QKV/out and conv in/out projections; `bf16_weight_packing` is accepted and ignored."""
+        from .decoder import LFM25HIPDecoder
+        if self._decoder_busy:
+            raise RuntimeError("Close the native generation session before reconfiguring CUDA graphs")
+        if self._cuda_decoder is not None:
+            self._cuda_decoder.clear()
+        self._cuda_decoder = LFM25HIPDecoder(self, max_graphs=max_graphs, max_prefill_tokens=max_prefill_tokens,
+                                             fp8_mlp=fp8_mlp, fp8_kv=fp8_kv, adaptive_batching=adaptive_batching,
+                                             fp8_lm_head=fp8_lm_head, fp8_operators=fp8_operators, capture=capture)
+
+    enable_hip_graphs = enable_cuda_graphs
+
+    def disable_cuda_graphs(self) -> None:
+        if self._cuda_decoder is not None:
+            self._cuda_decoder.clear()
+        self._cuda_decoder = None
+
+    def release_inference_buffers(self) -> None:
+        decoder = self._cuda_decoder
+        if decoder is None:
+            return
+        if decoder._active_session is not None:
+            raise RuntimeError("Close the native generation session before releasing inference buffers")
+        if not (decoder.graphs or decoder.fp8_weights):
+            return
+        torch.cuda.synchronize(self.device)
+        decoder.clear()
+        torch.cuda.empty_cache()
+
+    def generation_session(self, *, max_batch_size: int, max_new_tokens: int, cache_len: int | None = None,
+                           behavior_topk: int = 0, profile_timings: bool = False):
+        if self._cuda_decoder is None:
+            raise RuntimeError("generation_session requires enable_cuda_graphs()")
+        from .session import LFM25GenerationSession
+        return LFM25GenerationSession(self._cuda_decoder, max_batch_size=max_batch_size, max_new_tokens=max_new_tokens,
+                                      cache_len=cache_len, behavior_topk=behavior_topk, profile_timings=profile_timings)
+
+    # ------------------------------------------------------------------ cache
+    def _empty_cache(self, *, max_slots: int, max_seq_len: int, fp8_kv: bool = False) -> LFM25HybridCache:
+        if max_slots <= 0:
+            raise ValueError("max_slots must be > 0")
+        if max_seq_len <= 0:
+            raise ValueError("max_seq_len must be > 0")
+        if max_seq_len > self.max_model_len:
+            raise ValueError(f"max_seq_len={max_seq_len} exceeds engine max_model_len={self.max_model_len}")
+        cfg = self.config
+        return LFM25HybridCache.allocate(
+            attn_layers=self.weights.num_attention_layers, conv_layers=self.weights.num_conv_layers, slots=max_slots,
+            capacity=max_seq_len, kv_heads=cfg.num_key_value_heads, head_dim=cfg.head_dim, hidden=cfg.hidden_size,
+            kernel=cfg.conv_kernel_size, dtype=self.dtype, device=self.device, fp8_kv=fp8_kv)
+
+    # ------------------------------------------------------------------ shared layer walk
+    def _fp8(self):
+        return self._cuda_decoder.fp8_weights if self._cuda_decoder is not None else {}
+
+    def _norm_linear(self, x, norm_weight, residual, weight, fp8):
+        """residual-add + RMSNorm feeding a projection; W8A8 when the projection has an e4m3 copy."""
+        packed = fp8.get(id(weight))
+        if packed is not None:
+            q, scales, residual = ops.rms_norm_fp8(x, norm_weight, self.config.norm_eps, residual)
+            return packed.linear_quantized(q, scales, dtype=self.dtype), residual
+        normed, residual = ops.rms_norm(x, norm_weight, self.config.norm_eps, residual)
+        return ops.linear(normed, weight), residual
+
+    def _linear(self, x, weight, fp8):
+        packed = fp8.get(id(weight))
+        return packed.linear(x) if packed is not None else ops.linear(x, weight)
+
+    def _backbone(self, tokens, attention_op, conv_op, fp8):
+        """Embedding and all layers with the fused residual chain of lfm25_cuda.py:134-184: every RMSNorm also adds
+        the previous block's output into the running residual.  Returns (last MLP output, residual)."""
+        hidden = ops.embedding(tokens, self.weights.embed_tokens)
+        residual = None
+        for layer in self.weights.layers:
+            if layer.attention is not None:
+                op = layer.attention
+                qkv, residual = self._norm_linear(hidden, layer.operator_norm_weight, residual, op.qkv_weight, fp8)
+                mixed = self._linear(attention_op(op, qkv), op.out_weight, fp8)
+            else:
+                op = layer.conv
+                bcx, residual = self._norm_linear(hidden, layer.operator_norm_weight, residual, op.in_weight, fp8)
+                mixed = self._linear(conv_op(op, bcx), op.out_weight, fp8)
+            gate_up, residual = self._norm_linear(mixed, layer.ffn_norm_weight, residual, layer.w13_weight, fp8)
+            down = fp8.get(id(layer.w2_weight))
+            if down is not None:
+                q, scales = ops.swiglu_fp8(gate_up)
+                hidden = down.linear_quantized(q, scales, dtype=self.dtype)
+            else:
+                hidden = ops.linear(ops.swiglu(gate_up), layer.w2_weight)
+        return hidden, residual
+
+    def _head(self, hidden, residual, fp8):
+        logits, _ = self._norm_linear(hidden, self.weights.embedding_norm_weight, residual, self.weights.lm_head_weight, fp8)
+        return logits
+
+    # ------------------------------------------------------------------ decode step (one token per row)
+    def _decode_forward(self, cache: LFM25HybridCache, tokens, active=None, *, slot_ids=None, positions=None, fp8=None):
+        """One token for every row (lfm25_cuda.py:128-192).  Rows index cache slots directly, or through `slot_ids`
+        (then `positions` are the rows' lengths and -1 marks padding)."""
+        cfg = self.config
+        fp8 = self._fp8() if fp8 is None else fp8
+        positions = cache.seq_lens if positions is None else positions
+        rows = tokens.numel()
+
+        def attention_op(op, qkv):
+            q, k, v = ops.prepare_qkv(qkv, op.q_norm_weight, op.k_norm_weight, self._rope_cos, self._rope_sin, positions,
+                                      cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim, cfg.norm_eps)
+            i = op.cache_index
+            if cache.fp8:
+                out = ops.decode(q, k, v, cache.k_cache[i], cache.v_cache[i], cache.k_scales[i], cache.v_scales[i], positions,
+                                 active=active, scale=self._scaling, slot_ids=slot_ids)
+            else:
+                ops.append_bf16_kv(k, v, cache.k_cache[i], cache.v_cache[i], positions, slot_ids, active)
+                out = ops.attend(q, cache.k_cache[i], cache.v_cache[i], None, None, positions, active=active,
+                                 scale=self._scaling, slot_ids=slot_ids)
+            return out.view(rows, -1)
+
+        def conv_op(op, bcx):
+            return ops.conv_update(bcx, op.conv_weight, cache.conv_state[op.cache_index], active, slot_ids)
+
+        hidden, residual = self._backbone(tokens, attention_op, conv_op, fp8)
+        logits = self._head(hidden, residual, fp8)
+        ops.advance_positions(cache.seq_lens, positions, slot_ids, active)
+        return logits
+
+    # ------------------------------------------------------------------ prefill
+    def _prefill_packed(self, cache: LFM25HybridCache, tokens, lengths: Sequence[int], fp8):
+        """Forward a packed batch of whole prompts into cache rows 0..n-1; returns next-token logits [n, V]."""
+        cfg = self.config
+        count, total, longest = len(lengths), int(sum(lengths)), int(max(lengths))
+        if count > cache.max_slots:
+            raise RuntimeError("cache slot capacity exceeded")
+        if longest > cache.max_seq_len:
+            raise RuntimeError("cache capacity exceeded")
+        if longest > self.max_model_len:
+            raise RuntimeError("position exceeds engine max_model_len")
+        cu_host = torch.zeros(count + 1, dtype=torch.int32)
+        cu_host[1:] = torch.tensor(lengths, dtype=torch.int32).cumsum(0)
+        cu = cu_host.to(self.device)
+        seq_of_token, positions = ops.build_token_map(cu, total)
+        slots = torch.arange(count, device=self.device, dtype=torch.int32)
+
+        def attention_op(op, qkv):
+            q, k, v = ops.prepare_qkv(qkv, op.q_norm_weight, op.k_norm_weight, self._rope_cos, self._rope_sin, positions,
+                                      cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim, cfg.norm_eps)
+            i = op.cache_index
+            q, k, v = q.view(total, -1, cfg.head_dim), k.view(total, -1, cfg.head_dim), v.view(total, -1, cfg.head_dim)
+            ops.store_kv_packed(k, v, cache.k_cache[i], cache.v_cache[i],
+                                None if cache.k_scales is None else cache.k_scales[i],
+                                None if cache.v_scales is None else cache.v_scales[i], cu, seq_of_token, slots)
+            return ops.prefill_attention(q, k, v, cu, longest, self._scaling).view(total, -1)
+
+        def conv_op(op, bcx):
+            return ops.conv_prefill(bcx, op.conv_weight, cache.conv_state[op.cache_index], cu, seq_of_token, slots)
+
+        hidden, residual = self._backbone(tokens, attention_op, conv_op, fp8)
+        last = (cu[1:] - 1).long()
+        logits = self._head(hidden.index_select(0, last), residual.index_select(0, last), fp8)
+        cache.seq_lens[:count].copy_(cu[1:] - cu[:-1])
+        return logits
+
+    @torch.inference_mode()
+    def prefill(self, input_ids, cu_seqlens, max_seqlen: int, *, max_cache_len: int | None = None,
+                cache: LFM25HybridCache | None = None, max_prefill_tokens: int | None = None,
+                logits_buffer: torch.Tensor | None = None) -> LFM25PrefixBatch:
+        input_ids = input_ids.to(device=self.device, dtype=torch.long).reshape(-1)
+        cu_host = cu_seqlens.to(device="cpu", dtype=torch.long).reshape(-1)
+        if cu_host.numel() < 2:
+            raise ValueError("cu_seqlens must contain at least [0, total_tokens]")
+        if int(cu_host[0]) != 0:
+            raise ValueError("cu_seqlens must start at 0")
+        if int(cu_host[-1]) != int(input_ids.numel()):
+            raise ValueError("cu_seqlens[-1] must equal input_ids.numel()")
+        lengths = (cu_host[1:] - cu_host[:-1]).tolist()
+        if min(lengths) <= 0:
+            raise ValueError("empty prompts are not supported")
+        if max(lengths) > int(max_seqlen):
+            raise ValueError("max_seqlen is smaller than at least one prompt")
+        count = len(lengths)
+        cache_len = int(max_cache_len or max_seqlen)
+        if cache is None:
+            cache = self._empty_cache(max_slots=count, max_seq_len=cache_len)
+        elif cache.max_slots != count or cache.max_seq_len < cache_len:
+            raise ValueError("destination cache does not fit the prompt batch")
+        if max_prefill_tokens is not None and max_prefill_tokens <= 0:
+            raise ValueError("max_prefill_tokens must be positive")
+        shape = (count, self.config.vocab_size)
+        if logits_buffer is None:
+            logits_out = torch.empty(shape, device=self.device, dtype=self.dtype)
+        else:
+            if logits_buffer.shape != shape or logits_buffer.dtype != self.dtype or logits_buffer.device != self.weights.embed_tokens.device:
+                raise ValueError("logits buffer must match the prompt batch, vocabulary, device, and model dtype")
+            logits_out = logits_buffer
+        budget = MAX_PACKED_TOKENS if max_prefill_tokens is None else min(int(max_prefill_tokens), MAX_PACKED_TOKENS)
+        fp8 = self._fp8()
+        offsets = cu_host.tolist()
+        for start, end, _ in plan_prefill_chunks(lengths, budget):
+            logits = self._prefill_packed(cache.rows(start, end), input_ids[offsets[start]:offsets[end]], lengths[start:end], fp8)
+            logits_out[start:end].copy_(logits)
+        return LFM25PrefixBatch(cache, logits_out, torch.tensor(lengths, device=self.device, dtype=torch.int32), input_ids)
+
+    # ------------------------------------------------------------------ fork / decode_step
+    @torch.inference_mode()
+    def fork(self, prefix: LFM25PrefixBatch, repeats: int, *, max_cache_len: int | None = None) -> LFM25DecodeBatch:
+        if repeats <= 0:
+            raise ValueError("repeats must be > 0")
+        prompts = prefix.batch_size
+        total = prompts * int(repeats)
+        cache_len = int(max_cache_len or prefix.cache.max_seq_len)
+        if cache_len < prefix.cache.max_seq_len:
+            raise ValueError("max_cache_len cannot be smaller than the prefix cache")
+        cache = self._empty_cache(max_slots=total, max_seq_len=cache_len)
+        arange = lambda n: torch.arange(n, device=self.device, dtype=torch.long)
+        cache.copy_prefix_from(prefix.cache, arange(prompts).repeat_interleave(repeats), prefix.cache.max_seq_len)
+        return LFM25DecodeBatch(cache, arange(total), arange(prompts).repeat_interleave(repeats),
+                                arange(repeats).repeat(prompts), torch.ones(total, device=self.device, dtype=torch.bool))
+
+    @torch.inference_mode()
+    def _append_decode_tokens(self, cache: LFM25HybridCache, slot_ids, input_tokens):
+        """Eager decode of one token for the given slots with the reference's capacity checks
+        (lfm25_engine.py:1232-1243)."""
+        slot_ids = slot_ids.to(device=self.device, dtype=torch.long).reshape(-1)
+        input_tokens = input_tokens.to(device=self.device, dtype=torch.long).reshape(-1)
+        if slot_ids.numel() != input_tokens.numel():
+            raise ValueError("slot_ids and input_tokens must have matching lengths")
+        if torch.any(slot_ids < 0) or torch.any(slot_ids >= cache.max_slots):
+            raise ValueError("slot_ids contain an out-of-range cache slot")
+        positions = cache.seq_lens.index_select(0, slot_ids)
+        if torch.any(positions >= cache.max_seq_len):
+            raise RuntimeError("cache capacity exceeded")
+        if torch.any(positions >= self.max_model_len):
+            raise RuntimeError("position exceeds engine max_model_len")
+        active = torch.ones(slot_ids.numel(), device=self.device, dtype=torch.bool)
+        return self._decode_forward(cache, input_tokens, active, slot_ids=slot_ids.to(torch.int32), positions=positions.contiguous())
+
+    @torch.inference_mode()
+    def decode_step(self, state: LFM25DecodeBatch, input_tokens, sampling: LFM25SamplingConfig | None = None) -> LFM25StepOutput:
+        sampling = sampling or LFM25SamplingConfig()
+        input_tokens = input_tokens.to(device=self.device, dtype=torch.long).reshape(-1)
+        if input_tokens.numel() != state.active_slot_ids.numel():
+            raise ValueError("input_tokens must have one token per active slot")
+        logits = self._append_decode_tokens(state.cache, state.active_slot_ids, input_tokens)
+        tokens, raw = self._sample(logits, sampling, step=0)
+        reasons = self._finish_reasons(tokens, sampling)
+        keep = sampling.return_logprobs
+        return LFM25StepOutput(tokens, raw if keep else None, raw if keep else None, reasons != 0, reasons, logits)
+
+    # ------------------------------------------------------------------ sampling helpers
+    def _sample(self, logits, sampling: LFM25SamplingConfig, *, step: int, seen_token_mask=None):
+        """Greedy, full-support Gumbel-max, or temperature/top-k/top-p on the device; log-probabilities are the raw
+        log-softmax of the draw (lfm25_engine.py:1574-1609).  A repetition penalty is applied to an fp32 copy first."""
+        if seen_token_mask is not None and sampling.repetition_penalty != 1.0:
+            lf = logits.float()
+            penalised = torch.where(lf < 0, lf * sampling.repetition_penalty, lf / sampling.repetition_penalty)
+            logits = torch.where(seen_token_mask, penalised, lf)
+        if sampling.filtered:
+            return ops.sample_filtered(logits, temperature=sampling.temperature, top_k=sampling.top_k, top_p=sampling.top_p,
+                                       seed=sampling.seed, step=step)
+        return ops.sample_logits(logits, temperature=sampling.temperature, seed=sampling.seed, step=step, return_logprobs=True)
+
+    def _finish_reasons(self, token_ids, sampling: LFM25SamplingConfig):
+        reasons = torch.zeros_like(token_ids, dtype=torch.int8)
+        if not sampling.ignore_eos:
+            reasons[token_ids == int(self.config.eos_token_id)] = 1
+        for stop_id in sampling.stop_token_ids:
+            reasons[(reasons == 0) & (token_ids == int(stop_id))] = 2
+        return reasons
+
+    def _build_seen_token_mask(self, prefix: LFM25PrefixBatch, repeats: int, sampling: LFM25SamplingConfig):
+        if float(sampling.repetition_penalty) == 1.0:
+            return None
+        mask = torch.zeros((prefix.batch_size * repeats, self.config.vocab_size), device=self.device, dtype=torch.bool)
+        bounds = [0, *prefix.prompt_lengths.long().cumsum(0).tolist()]
+        for i, (a, b) in enumerate(zip(bounds[:-1], bounds[1:])):
+            mask[i * repeats:(i + 1) * repeats, prefix.input_ids[a:b].unique()] = True
+        return mask
+
+    # ------------------------------------------------------------------ generate
+    @torch.inference_mode()
+    def generate(self, input_ids, cu_seqlens, max_seqlen: int, repeats: int,
+                 sampling: LFM25SamplingConfig | None = None) -> LFM25GenerationOutput:
+        sampling = sampling or LFM25SamplingConfig()
+        if self._cuda_decoder is None:
+            # no graphs requested: the same loop with each step launched kernel by kernel
+            self.enable_cuda_graphs(capture=False)
+        return self._cuda_decoder.generate(input_ids, cu_seqlens, max_seqlen, repeats, sampling)
+
+    @torch.inference_mode()
+    def score_completions(self, prompts, completions, *, max_prefill_tokens: int = 4096, head_chunk_size: int = 256):
+        """Raw log-probabilities of given completions through the packed prefill kernels (lfm25_engine.py:1108-1163)."""
+        if len(prompts) != len(completions):
+            raise ValueError('prompts and completions must have equal lengths')
+        if max_prefill_tokens <= 0 or head_chunk_size <= 0:
+            raise ValueError('scoring chunk sizes must be positive')
+        if any(not p or not c for p, c in zip(prompts, completions)):
+            raise ValueError('scoring requires nonempty prompts and completions')
+        sequences = [list(p) + list(c) for p, c in zip(prompts, completions)]
+        if any(len(s) > self.max_model_len for s in sequences):
+            raise ValueError('scored sequence exceeds max_model_len')
+        cfg, fp8 = self.config, self._fp8()
+        result = [()] * len(sequences)
+        order = sorted(range(len(sequences)), key=lambda i: len(sequences[i]))
+        lengths = [len(sequences[i]) for i in order]
+        for start, end, width in plan_prefill_chunks(lengths, min(int(max_prefill_tokens), MAX_PACKED_TOKENS)):
+            group = order[start:end]
+            cache = self._empty_cache(max_slots=len(group), max_seq_len=width)
+            tokens = torch.tensor([t for i in group for t in sequences[i]], device=self.device, dtype=torch.long)
+            hidden = self._prefill_hidden(cache, tokens, [len(sequences[i]) for i in group], fp8)
+            rows, targets, base = [], [], 0
+            for i in group:
+                rows.extend(range(base + len(prompts[i]) - 1, base + len(sequences[i]) - 1))
+                targets.extend(completions[i])
+                base += len(sequences[i])
+            selected = hidden.index_select(0, torch.tensor(rows, device=self.device))
+            target = torch.tensor(targets, device=self.device, dtype=torch.long)
+            scores = []
+            for off in range(0, target.numel(), head_chunk_size):
+                logits = self._linear(selected[off:off + head_chunk_size].contiguous(), self.weights.lm_head_weight, {}).float()
+                pick = target[off:off + head_chunk_size]
+                scores.append(logits.gather(1, pick[:, None])[:, 0] - torch.logsumexp(logits, -1))
+            flat, cursor = torch.cat(scores).cpu().tolist(), 0
+            for i in group:
+                result[i] = tuple(flat[cursor:cursor + len(completions[i])])
+                cursor += len(completions[i])
+        return result
+
+    def _prefill_hidden(self, cache, tokens, lengths, fp8):
+        """Final-norm hidden states of every packed token (the `return_hidden` form of lfm25_engine.py:1097-1098)."""
+        count, total = len(lengths), int(sum(lengths))
+        cu_host = torch.zeros(count + 1, dtype=torch.int32)
+        cu_host[1:] = torch.tensor(lengths, dtype=torch.int32).cumsum(0)
+        cu = cu_host.to(self.device)
+        seq_of_token, positions = ops.build_token_map(cu, total)
+        slots = torch.arange(count, device=self.device, dtype=torch.int32)
+        cfg = self.config
+
+        def attention_op(op, qkv):
+            q, k, v = ops.prepare_qkv(qkv, op.q_norm_weight, op.k_norm_weight, self._rope_cos, self._rope_sin, positions,
+                                      cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim, cfg.norm_eps)
+            q, k, v = q.view(total, -1, cfg.head_dim), k.view(total, -1, cfg.head_dim), v.view(total, -1, cfg.head_dim)
+            return ops.prefill_attention(q, k, v, cu, int(max(lengths)), self._scaling).view(total, -1)
+
+        def conv_op(op, bcx):
+            return ops.conv_prefill(bcx, op.conv_weight, cache.conv_state[op.cache_index], cu, seq_of_token, slots)
+
+        hidden, residual = self._backbone(tokens, attention_op, conv_op, fp8)
+        return ops.rms_norm(hidden, self.weights.embedding_norm_weight, cfg.norm_eps, residual)[0]
+
+
+def _resolve_dtype(dtype):
+    if isinstance(dtype, torch.dtype):
+        return dtype
+    if dtype is None or str(dtype).lower() == "auto":
+        return torch.bfloat16
+    names = {"bf16": torch.bfloat16, "bfloat16": torch.bfloat16, "fp16": torch.float16, "float16": torch.float16,
+             "fp32": torch.float32, "float32": torch.float32}
+    try:
+        return names[str(dtype).strip().lower()]
+    except KeyError as exc:
+        raise ValueError(f"Unsupported dtype: {dtype!r}") from exc

@@ -226,8 +226,11 @@ def graph_capacity(cache_len: int, batch: int, max_model_len: int) -> int:
 class OracleEngine:
     """CPU restatement of ``LFM25Engine`` (eager path)."""
 
-    def __init__(self, cfg: OracleConfig, state, dtype=torch.float32, max_model_len: int | None = None):
-        self.cfg, self.dtype = cfg, dtype
+    def __init__(self, cfg: OracleConfig, state, dtype=torch.float32, max_model_len: int | None = None, fp8=()):
+        """``fp8`` names the parts that emulate W8A8 / e4m3-KV arithmetic: any of "mlp", "head", "operators", "kv"
+        (``lfm25_cuda.py:97-106,172-176``; "operators" is the QKV/out and conv in/out extension).  Emulation means
+        quantise-dequantise with the rules of ``k_quantize_rows`` / ``k_store_kv`` around an exact matmul."""
+        self.cfg, self.dtype, self.fp8 = cfg, dtype, frozenset(fp8)
         (self.embed, self.final_norm, self.head, self.layers,
          self.n_attn, self.n_conv) = pack_layers(cfg, state, dtype)
         self.max_model_len = int(max_model_len or min(cfg.max_position_embeddings, 32768))
@@ -242,19 +245,34 @@ class OracleEngine:
                            z(self.n_conv, slots, self.cfg.hidden_size, 3), torch.zeros(slots, dtype=torch.int32))
 
     # ---- shared pieces
+    def _lin(self, x, w, part):
+        """``F.linear``, or its W8A8 emulation when ``part`` is switched to FP8."""
+        if part not in self.fp8:
+            return F.linear(x, w)
+        xq, xs = k_quantize_rows(x.reshape(-1, x.shape[-1]))
+        wq, ws = k_quantize_rows(w)
+        return k_fp8_linear(xq, xs, wq, ws, x.dtype).reshape(*x.shape[:-1], w.shape[0])
+
+    def _kv(self, k, v):
+        """What a later decode step reads back from the cache: the tensors themselves, or their e4m3 round trip."""
+        if "kv" not in self.fp8:
+            return k, v
+        kq, ks, vq, vs = k_store_kv(k, v)
+        return (kq.float() * ks[..., None]).to(k.dtype), (vq.float() * vs[..., None]).to(v.dtype)
+
     def _mlp(self, layer, x):
         # bf16 runs w1 and w3 separately, fp32 fused (lfm25_engine.py:1300-1304).
         I = layer.w13.size(0) // 2
-        if x.dtype == torch.bfloat16:
+        if x.dtype == torch.bfloat16 and "mlp" not in self.fp8:
             g, u = F.linear(x, layer.w13[:I]), F.linear(x, layer.w13[I:])
         else:
-            g, u = F.linear(x, layer.w13).chunk(2, -1)
-        return F.linear(F.silu(g) * u, layer.w2)
+            g, u = self._lin(x, layer.w13, "mlp").chunk(2, -1)
+        return self._lin(F.silu(g) * u, layer.w2, "mlp")
 
     def _qkv_split(self, layer, x, fused_ok: bool):
         H, kvw = self.cfg.hidden_size, self.KH * self.D
-        if fused_ok and x.dtype != torch.bfloat16:
-            y = F.linear(x, layer.qkv)
+        if "operators" in self.fp8 or (fused_ok and x.dtype != torch.bfloat16):
+            y = self._lin(x, layer.qkv, "operators")
             q, k, v = y[..., :H], y[..., H:H + kvw], y[..., H + kvw:]
         else:  # three projections (lfm25_engine.py:1318-1321, 1377-1379)
             q, k, v = (F.linear(x, w) for w in layer.qkv.split((H, kvw, kvw)))
@@ -274,14 +292,13 @@ class OracleEngine:
                 k = rms_norm(k.reshape(B, T, self.KH, self.D), L.k_norm, self.cfg.norm_eps)
                 v = v.reshape(B, T, self.KH, self.D)
                 q, k = apply_rotary(q, cos, sin), apply_rotary(k, cos, sin)
-                cache.k[L.cache_index, :B, :T] = k
-                cache.v[L.cache_index, :B, :T] = v
+                cache.k[L.cache_index, :B, :T], cache.v[L.cache_index, :B, :T] = self._kv(k, v)
                 g = self.QH // self.KH
                 o = F.scaled_dot_product_attention(q.transpose(1, 2), k.repeat_interleave(g, 2).transpose(1, 2),
                                                    v.repeat_interleave(g, 2).transpose(1, 2), is_causal=True)
-                y = F.linear(o.transpose(1, 2).reshape(B, T, -1), L.out)
+                y = self._lin(o.transpose(1, 2).reshape(B, T, -1), L.out, "operators")
             else:
-                b, c, xp = F.linear(x, L.conv_in).chunk(3, -1)
+                b, c, xp = self._lin(x, L.conv_in, "operators").chunk(3, -1)
                 bx = b * xp
                 conv = F.conv1d(bx.transpose(1, 2), L.conv_w.unsqueeze(1), padding=2,
                                 groups=self.cfg.hidden_size)[..., :T].transpose(1, 2)
@@ -291,7 +308,7 @@ class OracleEngine:
                 idx = ln[:, None].long() + torch.arange(-3, 0)[None, :]
                 hist = bx.gather(1, idx.clamp_min(0)[:, :, None].expand(-1, -1, bx.size(-1)))
                 st.copy_(torch.where(idx[:, :, None] >= 0, hist, torch.zeros((), dtype=hist.dtype)).transpose(1, 2))
-                y = F.linear(c * conv, L.conv_out)
+                y = self._lin(c * conv, L.conv_out, "operators")
             h = h + y
             h = h + self._mlp(L, rms_norm(h, L.ffn_norm, self.cfg.norm_eps))
         if lengths is None:
@@ -300,7 +317,7 @@ class OracleEngine:
         else:
             cache.seq_lens[:B] = lengths.to(torch.int32)
             last = h[torch.arange(B), lengths.long() - 1]
-        return F.linear(rms_norm(last, self.final_norm, self.cfg.norm_eps), self.head)
+        return self._lin(rms_norm(last, self.final_norm, self.cfg.norm_eps), self.head, "head")
 
     def prefill(self, prompts: Sequence[Sequence[int]], cache: OracleCache | None = None,
                 cap: int | None = None, max_prefill_tokens: int | None = None):
@@ -338,8 +355,7 @@ class OracleEngine:
                 k = rms_norm(k.reshape(n, self.KH, self.D), L.k_norm, self.cfg.norm_eps)
                 q, k = apply_rotary(q, cos, sin), apply_rotary(k, cos, sin)
                 kc, vc = cache.k[L.cache_index], cache.v[L.cache_index]
-                kc[slots, pos] = k
-                vc[slots, pos] = v.reshape(n, self.KH, self.D)
+                kc[slots, pos], vc[slots, pos] = self._kv(k, v.reshape(n, self.KH, self.D))
                 g = self.QH // self.KH
                 outs = []
                 for r in range(n):  # per-row form, lfm25_engine.py:1562-1572
@@ -349,19 +365,19 @@ class OracleEngine:
                     s = torch.einsum("hd,htd->ht", q[r], kh) * self.scale
                     p = torch.softmax(s, -1, dtype=torch.float32).to(q.dtype)
                     outs.append(torch.einsum("ht,htd->hd", p, vh).reshape(-1))
-                y = F.linear(torch.stack(outs), L.out)
+                y = self._lin(torch.stack(outs), L.out, "operators")
             else:
-                b, c, xp = F.linear(x, L.conv_in).chunk(3, -1)
+                b, c, xp = self._lin(x, L.conv_in, "operators").chunk(3, -1)
                 bx = b * xp
                 st = cache.conv[L.cache_index]
                 new = torch.roll(st[slots], -1, -1)
                 new[:, :, -1] = bx
                 st[slots] = new
-                y = F.linear(c * (new * L.conv_w[None]).sum(-1), L.conv_out)
+                y = self._lin(c * (new * L.conv_w[None]).sum(-1), L.conv_out, "operators")
             h = h + y
             h = h + self._mlp(L, rms_norm(h, L.ffn_norm, self.cfg.norm_eps))
         cache.seq_lens[slots] += 1
-        return F.linear(rms_norm(h, self.final_norm, self.cfg.norm_eps), self.head)
+        return self._lin(rms_norm(h, self.final_norm, self.cfg.norm_eps), self.head, "head")
 
     # ---- sampling (lfm25_engine.py:1574-1609)
     def sample(self, logits, *, temperature=0.0, top_k=0, top_p=1.0, generator=None, seen=None, penalty=1.0):

@@ -209,3 +209,30 @@ def test_decode_attention_row_matches_causal_attention_last_row():
     kq, ks, vq, vs = O.k_store_kv(k, v)
     deq = O.k_attend(q[36], kq, vq, 37, D ** -0.5, ks, vs)
     torch.testing.assert_close(deq, full[36], atol=0.05, rtol=0.05)
+
+
+def test_w8a8_emulation_is_exact_on_grid_inputs_and_bounded_otherwise():
+    """Inputs that already sit on the e4m3 grid of their row (maximum mapped to 448) survive quantisation unchanged,
+    so the emulated projection equals the exact one; for arbitrary inputs the deviation obeys the half-ulp bound
+    |dy| <= sum |x||w| * ((1 + 2^-4)^2 - 1) of two relative roundings of at most 2^-4 each."""
+    from climbing_gym_amd.synthetic import TINY, random_state_dict
+    codes = torch.tensor([v for v, _ in _all_e4m3_values() if abs(v) >= 2 ** -6 or v == 0])
+    g = torch.Generator().manual_seed(9)
+    pick = lambda r, c: codes[torch.randint(0, len(codes), (r, c), generator=g)]
+    x, w = pick(6, 96) * 0.37, pick(10, 96) * 0.011
+    x[:, 0], w[:, 0] = 448 * 0.37, 448 * 0.011
+    cfg = O.OracleConfig(vocab_size=16, hidden_size=8, mlp_hidden_size=8, num_hidden_layers=1, num_attention_heads=2,
+                         num_key_value_heads=1, max_position_embeddings=8, layer_types=("conv",))
+    state = random_state_dict(hidden=8, mlp_hidden=8, layer_types=("conv",), q_heads=2, kv_heads=1, vocab=16)
+    eng = O.OracleEngine(cfg, state, torch.float32, 8, fp8=("mlp",))
+    torch.testing.assert_close(eng._lin(x, w, "mlp"), (x.double() @ w.double().T).float(), atol=1e-3, rtol=1e-5)
+    assert torch.equal(eng._lin(x, w, "head"), torch.nn.functional.linear(x, w))  # other parts stay exact
+    x, w = torch.randn(7, 200, generator=g), torch.randn(9, 200, generator=g) * 0.02
+    dy = (eng._lin(x, w, "mlp") - x @ w.T).abs()
+    bound = (x.abs() @ w.abs().T) * ((1 + 2 ** -4) ** 2 - 1) + 2 ** -6 * 448 ** -1 * (x.abs().amax(1)[:, None] * w.abs().sum(1)[None] + w.abs().amax(1)[None] * x.abs().sum(1)[:, None])
+    assert (dy <= bound).all() and dy.max() > 0
+    k, v = torch.randn(5, 2, 16, generator=g), torch.randn(5, 2, 16, generator=g)
+    kv = O.OracleEngine(cfg, state, torch.float32, 8, fp8=("kv",))
+    kq, vq = kv._kv(k, v)
+    assert ((kq - k).abs() <= k.abs() * 2 ** -4 + k.abs().amax(-1, keepdim=True) / 448 * 2 ** -7).all()
+    assert kv._kv(kq, vq)[0].sub(kq).abs().max() < 1e-6  # the round trip is idempotent
