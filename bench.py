@@ -1,0 +1,172 @@
+#!/usr/bin/env python
+"""Decode throughput of the LFM2.5-1.2B-shaped FP8 model at 256 ragged concurrent sequences on one MI355X.
+
+A step is one decode token for every sequence of the batch: HIP-graph replay of the fused decode step
+(FP8 W8A8 linears, e4m3 KV cache), on-device sampling and the record kernel.  Prompts (uniform lengths in
+[256, 2048], uniform token ids, seed 0) are prefilled before the timed region, so inputs are resident in
+HBM when timing starts.  Prints ONE JSON line with the throughput, the roofline of the dominant kernel
+(ragged GQA decode attention over the e4m3 cache, timed with HIP events on the launch stream) and the CPU
+baseline (the oracle's fp32 restatement of the reference CPU engine on a bounded sample of the same workload).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def parse_args():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=64)
+    p.add_argument("--warmup", type=int, default=8)
+    p.add_argument("--batch", type=int, default=256)
+    p.add_argument("--prompt-low", type=int, default=256)
+    p.add_argument("--prompt-high", type=int, default=2048)
+    p.add_argument("--max-model-len", type=int, default=8192)
+    p.add_argument("--precision", choices=("fp8", "bf16"), default="fp8")
+    p.add_argument("--cpu-seqs", type=int, default=4, help="sequences of the workload the CPU baseline runs (0 = skip)")
+    p.add_argument("--cpu-steps", type=int, default=8)
+    p.add_argument("--attn-samples", type=int, default=20, help="timed launches of the decode-attention kernel per layer")
+    return p.parse_args()
+
+
+def build_engine(args, state):
+    from climbing_gym_amd.config import LFM2Config
+    from climbing_gym_amd.engine import LFM25Engine
+    from climbing_gym_amd.synthetic import LFM2_1P2B
+    cfg = LFM2Config(vocab_size=LFM2_1P2B["vocab"], hidden_size=LFM2_1P2B["hidden"], mlp_hidden_size=LFM2_1P2B["mlp_hidden"],
+                     num_hidden_layers=16, num_attention_heads=32, num_key_value_heads=8,
+                     layer_types=LFM2_1P2B["layer_types"], max_position_embeddings=128000)
+    engine = LFM25Engine.from_state_dict(cfg, state, device="cuda", dtype=torch.bfloat16, max_model_len=args.max_model_len)
+    fp8 = args.precision == "fp8"
+    engine.enable_cuda_graphs(max_graphs=1, max_prefill_tokens=4096, fp8_mlp=fp8, fp8_kv=fp8, fp8_lm_head=fp8, fp8_operators=fp8)
+    return engine, cfg
+
+
+def time_decode_attention(engine, session, samples):
+    """Average duration (s) of one decode-attention call at the batch's current context lengths, from HIP events
+    recorded on the launch stream around back-to-back launches, and the algorithmic bytes of one call."""
+    from climbing_gym_amd import ops
+    cfg, cache = engine.config, session.entry.cache
+    rows = session.batch_size
+    q = torch.randn((rows, 1, cfg.num_attention_heads, cfg.head_dim), device="cuda", dtype=torch.bfloat16)
+    positions = (cache.seq_lens - 1).clamp_min(0).contiguous()
+    active = torch.ones(rows, device="cuda", dtype=torch.bool)
+    stream = torch.cuda.current_stream()
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    total_ms, launches = 0.0, 0
+    for layer in range(cache.k_cache.size(0)):
+        args = (q, cache.k_cache[layer], cache.v_cache[layer],
+                None if cache.k_scales is None else cache.k_scales[layer],
+                None if cache.v_scales is None else cache.v_scales[layer], positions)
+        ops.attend(*args, active=active, scale=engine._scaling)  # warm
+        begin.record(stream)
+        for _ in range(samples):
+            ops.attend(*args, active=active, scale=engine._scaling)
+        end.record(stream)
+        end.synchronize()
+        total_ms += begin.elapsed_time(end)
+        launches += samples
+    tokens = int((positions.long() + 1).sum())
+    kv_token = cfg.num_key_value_heads * cfg.head_dim * 2 * (1 if cache.fp8 else 2) + (cfg.num_key_value_heads * 2 * 4 if cache.fp8 else 0)
+    bytes_per_call = tokens * kv_token + 2 * rows * cfg.num_attention_heads * cfg.head_dim * 2
+    return total_ms / 1000 / launches, bytes_per_call, tokens
+
+
+def cpu_baseline(args, state, prompts):
+    """The oracle (fp32 restatement of the reference CPU engine) on the first `cpu_seqs` sequences of the workload:
+    prefill untimed, `cpu_steps` greedy decode steps timed on all host threads."""
+    from climbing_gym_amd.synthetic import LFM2_1P2B
+    from oracle.lfm2_oracle import OracleConfig, OracleEngine
+    torch.set_num_threads(max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))))
+    ocfg = OracleConfig(vocab_size=LFM2_1P2B["vocab"], hidden_size=LFM2_1P2B["hidden"], mlp_hidden_size=LFM2_1P2B["mlp_hidden"],
+                        num_hidden_layers=16, num_attention_heads=32, num_key_value_heads=8,
+                        layer_types=LFM2_1P2B["layer_types"])
+    oracle = OracleEngine(ocfg, state, torch.float32, max_model_len=args.max_model_len)
+    sample = prompts[:args.cpu_seqs]
+    with torch.inference_mode():
+        cache, logits = oracle.prefill(sample, cap=max(map(len, sample)) + args.cpu_steps + 1)
+        slots = torch.arange(len(sample))
+        tokens = logits.argmax(-1)
+        start = time.perf_counter()
+        for _ in range(args.cpu_steps):
+            logits = oracle.append_tokens(cache, slots, tokens)
+            tokens = logits.argmax(-1)
+        elapsed = time.perf_counter() - start
+    return {"value": round(len(sample) * args.cpu_steps / elapsed, 3), "unit": "tok/s", "cores": torch.get_num_threads(),
+            "kind": "port", "sample": f"first {len(sample)} of the {args.batch} sequences (fp32 weights), prefill untimed, "
+                                       f"{args.cpu_steps} greedy decode steps timed"}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one MI355X; --gpus {args.gpus} is not supported in this build "
+              "(the path shards by slots across independent engines with no collective in the step).", file=sys.stderr)
+        sys.exit(2)
+    from climbing_gym_amd.config import LFM25SamplingConfig
+    from climbing_gym_amd.synthetic import LFM2_1P2B, random_prompts, random_state_dict
+
+    state = random_state_dict(**LFM2_1P2B, seed=0)
+    prompts = random_prompts(args.batch, args.prompt_low, args.prompt_high, LFM2_1P2B["vocab"], seed=0)
+    engine, cfg = build_engine(args, state)
+    new_tokens = min(4096, args.max_model_len - max(map(len, prompts)))
+    sampling = [LFM25SamplingConfig(temperature=1.0, seed=1000 + i, max_new_tokens=new_tokens, ignore_eos=True)
+                for i in range(args.batch)]
+    with torch.inference_mode(), engine.generation_session(max_batch_size=args.batch, max_new_tokens=new_tokens,
+                                                            cache_len=args.max_model_len) as session:
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        session.admit(prompts, sampling)
+        torch.cuda.synchronize()
+        prefill_s = time.perf_counter() - t0
+        session.poll(steps=max(args.warmup, 1))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        finished = session.poll(steps=args.steps)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        assert not finished, "no sequence may finish inside the timed region"
+        attn_s, attn_bytes, ctx_tokens = time_decode_attention(engine, session, args.attn_samples)
+        kv_token = 6 * (attn_bytes - 2 * args.batch * 32 * 64 * 2) // max(ctx_tokens, 1)
+    fp8 = args.precision == "fp8"
+    weights = sum(w.numel() for w in set(engine.weights.linear_matrices())) * (1 if fp8 else 2)
+    step_bytes = weights + ctx_tokens * kv_token + args.batch * 122880 * 2 + args.batch * cfg.vocab_size * 2 * 2
+    ms_per_step = elapsed / args.steps * 1000
+    achieved = attn_bytes / attn_s / 1e9
+    line = {
+        "metric": "decode output tok/s @256 ragged seqs, LFM2.5-1.2B FP8; % HBM roofline",
+        "value": round(args.batch * args.steps / elapsed, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "fp8_e4m3 (W8A8, fp32 accumulate; bf16 activations)" if fp8 else "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"LFM2.5-1.2B-shaped random-init model, {args.precision} linears and KV cache, {args.batch} "
+                               f"concurrent sequences, prompts U[{args.prompt_low},{args.prompt_high}] tokens, temperature 1, "
+                               f"max_model_len {args.max_model_len}, HIP-graph decode step",
+                   "context_tokens": ctx_tokens, "prefill_tok_per_s": round(sum(map(len, prompts)) / prefill_s, 1),
+                   "step_algorithmic_bytes": step_bytes,
+                   "step_hbm_fraction": round(step_bytes / (ms_per_step / 1000) / 1e9 / HBM_PEAK_GBS, 4)},
+        "roofline": {"kernel": "decode_attn_kernel (ragged GQA decode attention, e4m3 KV)" if fp8 else "decode_attn_kernel (bf16 KV)",
+                     "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "avg_launch_us": round(attn_s * 1e6, 2), "algorithmic_bytes_per_launch": attn_bytes},
+    }
+    del session
+    engine.disable_cuda_graphs()
+    torch.cuda.empty_cache()
+    line["cpu_baseline"] = cpu_baseline(args, state, prompts) if args.cpu_seqs > 0 else None
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -96,7 +96,7 @@ struct DecodeArgs {
   const uint8_t* active;
   float *ws_acc, *ws_m, *ws_l;
   int64_t max_blocks, c0, c1, c2;
-  int page, QH, KH, D, G, nchunks;
+  int page, QH, KH, D, G, nchunks, chunk;
   float scale_log2e;
 };
 
@@ -246,6 +246,189 @@ __global__ void __launch_bounds__(256) decode_attn_kernel(DecodeArgs a) {
   }
 }
 
+// ----------------------------------------------------------------------------- e4m3 history on MFMA
+// Specialisation for the headline shape: e4m3 history, head_dim 64, a GQA group of at most 4 query heads.
+// A wave walks its token range in tiles of 64 tokens and never leaves registers except for a 512-byte P tile:
+//
+//   S = Q.K^T : sixteen v_mfma_f32_4x4x4_16B_bf16 (16 independent 4x4x4 blocks per instruction).  Block b
+//               multiplies Q[4 heads][4 dims] by K[tokens 4b..4b+3][4 dims], so lane l owns token l of the tile:
+//               it loads that token's 64-byte row with four 16-byte loads and ends with S[0..3][token l].
+//   softmax   : running maxima are wave-uniform and only raised (with a rescale) when some lane exceeds them,
+//               so per-lane partial sums of l and O can simply be added at the end.
+//   O += P.V  : lane (g16, q, i) loads V[token 4*g16+i (+16u)][dims 16q..16q+15]; every dword is a 4x4 byte block
+//               over the quad (4 tokens x 4 dims) which two DPP quad permutes + two v_perm transpose in
+//               registers, giving the B operand V[4 tokens][dim]; P comes back from LDS as the A operand.
+//               Block (g16, q) accumulates O[4 heads][dims 16q+4w..] over its own tokens; the four g16 partials
+//               are added once per wave.
+//
+// e4m3 -> bf16 conversion is v_cvt_scalef32_pk_bf16_fp8 (two values per instruction, scale 1).
+constexpr int kMfmaChunk = 1024;  // history tokens per workgroup (4 waves x 256)
+constexpr int kMfmaWaveTok = kMfmaChunk / 4;
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ s16x4 e4m3x4_to_bf16x4(int w) {
+  const bf16x2 lo = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false);
+  const bf16x2 hi = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true);
+  const bf16x4 v = {lo[0], lo[1], hi[0], hi[1]};
+  return __builtin_bit_cast(s16x4, v);
+}
+// 4x4 byte transpose across the four lanes of a quad: out.byte[k] of lane j = in.byte[j] of lane k.
+__device__ __forceinline__ int quad_transpose_bytes(int x, int lane) {
+  const int t = __builtin_amdgcn_mov_dpp(x, 0xB1, 0xf, 0xf, true);  // quad_perm [1,0,3,2]
+  const int y = __builtin_amdgcn_perm(t, x, (lane & 1) ? 0x03070105 : 0x06020400);
+  const int u = __builtin_amdgcn_mov_dpp(y, 0x4E, 0xf, 0xf, true);  // quad_perm [2,3,0,1]
+  return __builtin_amdgcn_perm(u, y, (lane & 2) ? 0x03020706 : 0x05040100);
+}
+
+template <bool PAGED>
+__global__ void __launch_bounds__(256) decode_attn_mfma_kernel(DecodeArgs a) {
+  constexpr int D = 64;
+  const int b = blockIdx.z, h = blockIdx.y, chunk = blockIdx.x;
+  if (a.active && !a.active[b]) return;
+  const int64_t slot = a.slot_ids ? a.slot_ids[b] : b;
+  if (slot < 0) return;
+  const int len = a.positions[b] + 1;
+  const int start = chunk * kMfmaChunk;
+  if (start >= len) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int g = lane & 3, vq = (lane >> 2) & 3, g16 = lane >> 4;
+
+  __shared__ __bf16 lds_p[4][4][64];
+  __shared__ float sm[4][4], sl[4][4], sacc[4][4][D];
+
+  // A operand of S = Q.K^T: Q[head g][dims 4s..4s+3] for s = 0..15 (zero rows beyond the group)
+  s16x4 qop[16];
+  {
+    const bool ok = g < a.G;
+    const __bf16* src = (const __bf16*)a.q + ((int64_t)b * a.QH + h * a.G + (ok ? g : 0)) * D;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      i32x4 w = {0, 0, 0, 0};
+      if (ok) w = *reinterpret_cast<const i32x4*>(src + 8 * c);
+      const i32x2 lo = {w[0], w[1]}, hi = {w[2], w[3]};
+      qop[2 * c] = __builtin_bit_cast(s16x4, lo);
+      qop[2 * c + 1] = __builtin_bit_cast(s16x4, hi);
+    }
+  }
+  auto token_offset = [&](int t) -> int64_t {
+    if (PAGED) {
+      const int64_t blk = a.block_table[(int64_t)b * a.max_blocks + t / a.page];
+      return blk * a.c0 + (int64_t)(t % a.page) * a.c1 + (int64_t)h * a.c2;
+    }
+    return slot * a.c0 + (int64_t)t * a.c1 + (int64_t)h * a.c2;
+  };
+
+  float m[4], l[4];
+  f32x4 acc[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { m[i] = -1.0e30f; l[i] = 0.f; acc[i] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+
+  const int wbeg = start + wave * kMfmaWaveTok;
+  int wend = wbeg + kMfmaWaveTok;
+  wend = wend < len ? wend : len;
+  const uint8_t* kbase = (const uint8_t*)a.kc;
+  const uint8_t* vbase = (const uint8_t*)a.vc;
+  for (int T = wbeg; T < wend; T += 64) {
+    // ---- loads: this lane's K row, its scales, and its four V slices
+    const int tk = T + lane;
+    const bool valid = tk < wend;
+    const int64_t koff = token_offset(valid ? tk : wend - 1);
+    i32x4 kreg[4], vreg[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) kreg[c] = *reinterpret_cast<const i32x4*>(kbase + koff + 16 * c);
+    const float sk = a.ks[koff / D], sv = a.vs[koff / D];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      int tv = T + 16 * u + 4 * g16 + g;
+      tv = tv < wend ? tv : wend - 1;
+      vreg[u] = *reinterpret_cast<const i32x4*>(vbase + token_offset(tv) + 16 * vq);
+    }
+    // ---- S[0..3][token lane]
+    f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+      for (int w = 0; w < 4; ++w)
+        s = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(qop[4 * c + w], e4m3x4_to_bf16x4(kreg[c][w]), s, 0, 0, 0);
+    const float kscale = a.scale_log2e * sk;
+    bool raise = false;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      s[i] = valid ? s[i] * kscale : -1.0e30f;
+      raise |= s[i] > m[i];
+    }
+    if (__any(raise)) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float mnew = fmaxf(m[i], wave_max(s[i]));
+        const float alpha = __builtin_amdgcn_exp2f(m[i] - mnew);
+        m[i] = mnew;
+        l[i] *= alpha;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) acc[w][i] *= alpha;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float p = valid ? __builtin_amdgcn_exp2f(s[i] - m[i]) : 0.f;
+      l[i] += p;
+      lds_p[wave][i][lane] = (__bf16)(p * sv);
+    }
+    // ---- O[0..3][dims 16*vq + 4w + g] += P . V over this lane group's tokens
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const i32x2 praw = *reinterpret_cast<const i32x2*>(&lds_p[wave][g][16 * u + 4 * g16]);
+      const s16x4 pop = __builtin_bit_cast(s16x4, praw);
+#pragma unroll
+      for (int w = 0; w < 4; ++w)
+        acc[w] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(pop, e4m3x4_to_bf16x4(quad_transpose_bytes(vreg[u][w], lane)), acc[w], 0, 0, 0);
+    }
+  }
+  // ---- wave totals: l over all lanes, O over the four token groups
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    l[i] = wave_sum(l[i]);
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      float v = acc[w][i];
+      v += __shfl_xor(v, 16, 64);
+      v += __shfl_xor(v, 32, 64);
+      acc[w][i] = v;
+    }
+  }
+  if (g16 == 0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int w = 0; w < 4; ++w) sacc[wave][i][16 * vq + 4 * w + g] = acc[w][i];
+    }
+    if (lane == 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { sm[wave][i] = m[i]; sl[wave][i] = l[i]; }
+    }
+  }
+  __syncthreads();
+  {
+    const int gi = threadIdx.x >> 6, d = threadIdx.x & 63;  // 4 heads x 64 dims = 256 threads
+    if (gi < a.G) {
+      float mm = sm[0][gi];
+#pragma unroll
+      for (int w = 1; w < 4; ++w) mm = fmaxf(mm, sm[w][gi]);
+      float lt = 0.f, ot = 0.f;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const float f = __builtin_amdgcn_exp2f(sm[w][gi] - mm);
+        lt = fmaf(sl[w][gi], f, lt);
+        ot = fmaf(sacc[w][gi][d], f, ot);
+      }
+      const int64_t prow = ((int64_t)b * a.QH + h * a.G + gi) * a.nchunks + chunk;
+      a.ws_acc[prow * D + d] = ot;
+      if (d == 0) { a.ws_m[prow] = mm; a.ws_l[prow] = lt; }
+    }
+  }
+}
+
 // Merge the chunk partials of one (row, query head); inactive or empty rows give zeros.
 template <typename T>
 __global__ void __launch_bounds__(64) decode_combine_kernel(DecodeArgs a) {
@@ -258,7 +441,7 @@ __global__ void __launch_bounds__(64) decode_combine_kernel(DecodeArgs a) {
     for (int d = threadIdx.x; d < a.D; d += 64) out[d] = Elem<T>::store(0.f);
     return;
   }
-  const int n = (len + kChunk - 1) / kChunk;
+  const int n = (len + a.chunk - 1) / a.chunk;
   const int64_t prow = ((int64_t)b * a.QH + qh) * a.nchunks;
   float mm = -1.0e30f;
   for (int c = 0; c < n; ++c) mm = fmaxf(mm, a.ws_m[prow + c]);
@@ -474,7 +657,7 @@ extern "C" int lfm2_store_kv_packed(const void* k, const void* v, void* k_cache,
 }
 
 extern "C" int64_t lfm2_decode_attention_workspace(int64_t B, int QH, int D, int64_t capacity) {
-  const int64_t nch = (capacity + kChunk - 1) / kChunk;
+  const int64_t nch = (capacity + kChunk - 1) / kChunk;  // the smaller chunk of the two kernels bounds both
   return B * QH * nch * (D + 2);
 }
 
@@ -493,8 +676,10 @@ extern "C" int lfm2_decode_attention(void* out, const void* q, const void* k_cac
   if (int e = check_head_dim("decode_attention", D)) return e;
   const int align = kv_fp8 ? 16 : 8;
   LFM2_REQUIRE(c0 % align == 0 && c1 % align == 0 && c2 % align == 0, "decode_attention: cache strides must be multiples of %d elements", align);
-  const int nch = (int)((capacity + kChunk - 1) / kChunk);
   const int G = QH / KH;
+  const bool mfma = kv_fp8 && D == 64 && G <= 4 && dtype == LFM2_DTYPE_BF16;
+  const int chunk = mfma ? kMfmaChunk : kChunk;
+  const int nch = (int)((capacity + chunk - 1) / chunk);
   DecodeArgs a;
   a.out = out; a.q = q; a.kc = k_cache; a.vc = v_cache; a.ks = k_scales; a.vs = v_scales;
   a.positions = positions; a.slot_ids = slot_ids; a.block_table = block_table; a.active = active;
@@ -502,9 +687,16 @@ extern "C" int lfm2_decode_attention(void* out, const void* q, const void* k_cac
   a.ws_m = workspace + B * QH * nch * D;
   a.ws_l = a.ws_m + B * QH * nch;
   a.max_blocks = max_blocks; a.c0 = c0; a.c1 = c1; a.c2 = c2;
-  a.page = page; a.QH = QH; a.KH = KH; a.D = D; a.G = G; a.nchunks = nch;
+  a.page = page; a.QH = QH; a.KH = KH; a.D = D; a.G = G; a.nchunks = nch; a.chunk = chunk;
   a.scale_log2e = scale * LFM2_LOG2E;
   hipStream_t s = (hipStream_t)stream;
+  if (mfma) {
+    const dim3 mgrid(nch, KH, B);
+    if (block_table) hipLaunchKernelGGL(decode_attn_mfma_kernel<true>, mgrid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(decode_attn_mfma_kernel<false>, mgrid, dim3(256), 0, s, a);
+    hipLaunchKernelGGL(decode_combine_kernel<__bf16>, dim3(B, QH), dim3(64), 0, s, a);
+    LFM2_LAUNCH_CHECK();
+  }
   const dim3 grid(nch, KH * ((G + kGB - 1) / kGB), B);
 #define DEC_(DD)                                                                                     \
   if (kv_fp8) hipLaunchKernelGGL((decode_attn_kernel<T, true, DD>), grid, dim3(256), 0, s, a);       \
