@@ -32,7 +32,8 @@ _SIGNATURES = {
     "lfm2_store_kv_fp8": "ppppppppp" "lliilllllllllip",
     "lfm2_append_kv": "ppppppp" "liilllip",
     "lfm2_store_kv_packed": "ppppppppp" "liillliip",
-    "lfm2_decode_attention": "pppppppppp" "lip" "liiillllfiip",
+    "lfm2_decode_attention": "pppppppppp" "lipp" "liiillllfiip",
+    "lfm2_decode_schedule": "pppp" "lp",
     "lfm2_prefill_attention": "ppppp" "lliiifip",
     "lfm2_build_token_map": "ppp" "llp",
     "lfm2_gather_inputs": "ppppppp" "lp",
@@ -48,6 +49,7 @@ _INT64_RESULT = {
     "lfm2_fp8_gemm_workspace": "lll",
     "lfm2_bf16_gemm_workspace": "lll",
     "lfm2_decode_attention_workspace": "liil",
+    "lfm2_decode_schedule_size": "ll",
 }
 _CTYPE = {"p": ctypes.c_void_p, "l": ctypes.c_int64, "i": ctypes.c_int, "f": ctypes.c_float}
 

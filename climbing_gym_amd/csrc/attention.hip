@@ -95,6 +95,7 @@ struct DecodeArgs {
   const int32_t *positions, *slot_ids, *block_table;
   const uint8_t* active;
   float *ws_acc, *ws_m, *ws_l;
+  const int32_t* schedule;  // [0] = number of (row, chunk) items, then the pairs
   int64_t max_blocks, c0, c1, c2;
   int page, QH, KH, D, G, nchunks, chunk;
   float scale_log2e;
@@ -281,21 +282,22 @@ __device__ __forceinline__ int quad_transpose_bytes(int x, int lane) {
   return __builtin_amdgcn_perm(u, y, (lane & 2) ? 0x03020706 : 0x05040100);
 }
 
+// The grid is persistent: workgroups stride over the (row, chunk, KV head) items of a schedule that a tiny kernel
+// builds from the rows' current lengths, so a ragged batch in a large-capacity cache launches no empty workgroups.
 template <bool PAGED>
 __global__ void __launch_bounds__(256) decode_attn_mfma_kernel(DecodeArgs a) {
   constexpr int D = 64;
-  const int b = blockIdx.z, h = blockIdx.y, chunk = blockIdx.x;
-  if (a.active && !a.active[b]) return;
-  const int64_t slot = a.slot_ids ? a.slot_ids[b] : b;
-  if (slot < 0) return;
-  const int len = a.positions[b] + 1;
-  const int start = chunk * kMfmaChunk;
-  if (start >= len) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int g = lane & 3, vq = (lane >> 2) & 3, g16 = lane >> 4;
-
   __shared__ __bf16 lds_p[4][4][64];
   __shared__ float sm[4][4], sl[4][4], sacc[4][4][D];
+  const int items = a.schedule[0] * a.KH;
+  for (int item = blockIdx.x; item < items; item += gridDim.x) {
+  const int pair = item / a.KH, h = item % a.KH;
+  const int b = a.schedule[2 + 2 * pair], chunk = a.schedule[3 + 2 * pair];
+  const int64_t slot = a.slot_ids ? a.slot_ids[b] : b;
+  const int len = a.positions[b] + 1;
+  const int start = chunk * kMfmaChunk;
 
   // A operand of S = Q.K^T: Q[head g][dims 4s..4s+3] for s = 0..15 (zero rows beyond the group)
   s16x4 qop[16];
@@ -427,6 +429,38 @@ __global__ void __launch_bounds__(256) decode_attn_mfma_kernel(DecodeArgs a) {
       if (d == 0) { a.ws_m[prow] = mm; a.ws_l[prow] = lt; }
     }
   }
+  __syncthreads();  // the LDS tiles are reused by the next item
+  }
+}
+
+// One workgroup turns the rows' lengths into the item list of the persistent kernel: row b contributes
+// ceil((positions[b]+1) / chunk) items unless it is inactive or padding.
+__global__ void __launch_bounds__(1024)
+decode_schedule_kernel(int32_t* schedule, const int32_t* positions, const uint8_t* active, const int32_t* slot_ids, int B,
+                       int chunk) {
+  __shared__ int scan[1024];
+  __shared__ int carry;
+  if (threadIdx.x == 0) carry = 0;
+  __syncthreads();
+  for (int base = 0; base < B; base += 1024) {
+    const int b = base + threadIdx.x;
+    int n = 0;
+    if (b < B && (!active || active[b]) && (!slot_ids || slot_ids[b] >= 0)) n = (positions[b] + chunk) / chunk;
+    scan[threadIdx.x] = n;
+    __syncthreads();
+    for (int o = 1; o < 1024; o <<= 1) {
+      const int v = threadIdx.x >= o ? scan[threadIdx.x - o] : 0;
+      __syncthreads();
+      scan[threadIdx.x] += v;
+      __syncthreads();
+    }
+    const int first = carry + scan[threadIdx.x] - n;
+    for (int c = 0; c < n; ++c) { schedule[2 + 2 * (first + c)] = b; schedule[3 + 2 * (first + c)] = c; }
+    __syncthreads();
+    if (threadIdx.x == 1023) carry += scan[1023];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) { schedule[0] = carry; schedule[1] = chunk; }
 }
 
 // Merge the chunk partials of one (row, query head); inactive or empty rows give zeros.
@@ -656,15 +690,30 @@ extern "C" int lfm2_store_kv_packed(const void* k, const void* v, void* k_cache,
   LFM2_LAUNCH_CHECK();
 }
 
+static int64_t schedule_ints(int64_t B, int64_t capacity) {
+  return 2 + 2 * B * ((capacity + kMfmaChunk - 1) / kMfmaChunk);
+}
+
 extern "C" int64_t lfm2_decode_attention_workspace(int64_t B, int QH, int D, int64_t capacity) {
   const int64_t nch = (capacity + kChunk - 1) / kChunk;  // the smaller chunk of the two kernels bounds both
-  return B * QH * nch * (D + 2);
+  return B * QH * nch * (D + 2) + schedule_ints(B, capacity);
+}
+
+extern "C" int64_t lfm2_decode_schedule_size(int64_t B, int64_t capacity) { return schedule_ints(B, capacity); }
+
+extern "C" int lfm2_decode_schedule(int32_t* schedule, const int32_t* positions, const uint8_t* active,
+                                    const int32_t* slot_ids, int64_t B, void* stream) {
+  LFM2_REQUIRE(B > 0 && schedule && positions, "decode_schedule: bad arguments");
+  hipLaunchKernelGGL(decode_schedule_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, schedule, positions, active,
+                     slot_ids, (int)B, kMfmaChunk);
+  LFM2_LAUNCH_CHECK();
 }
 
 extern "C" int lfm2_decode_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
                                      const float* k_scales, const float* v_scales, const int32_t* positions,
                                      const uint8_t* active, const int32_t* slot_ids, const int32_t* block_table,
-                                     int64_t max_blocks, int page, float* workspace, int64_t B, int QH, int KH, int D,
+                                     int64_t max_blocks, int page, const int32_t* schedule, float* workspace, int64_t B,
+                                     int QH, int KH, int D,
                                      int64_t capacity, int64_t c0, int64_t c1, int64_t c2, float scale, int kv_fp8,
                                      int dtype, void* stream) {
   LFM2_REQUIRE(B > 0 && QH > 0 && KH > 0 && capacity > 0, "decode_attention: empty shape");
@@ -686,12 +735,22 @@ extern "C" int lfm2_decode_attention(void* out, const void* q, const void* k_cac
   a.ws_acc = workspace;
   a.ws_m = workspace + B * QH * nch * D;
   a.ws_l = a.ws_m + B * QH * nch;
+  a.schedule = nullptr;
   a.max_blocks = max_blocks; a.c0 = c0; a.c1 = c1; a.c2 = c2;
   a.page = page; a.QH = QH; a.KH = KH; a.D = D; a.G = G; a.nchunks = nch; a.chunk = chunk;
   a.scale_log2e = scale * LFM2_LOG2E;
   hipStream_t s = (hipStream_t)stream;
   if (mfma) {
-    const dim3 mgrid(nch, KH, B);
+    if (schedule == nullptr) {  // no shared schedule from the caller: build one in the tail of the workspace
+      int32_t* own = reinterpret_cast<int32_t*>(workspace + B * QH * ((capacity + kChunk - 1) / kChunk) * (D + 2));
+      hipLaunchKernelGGL(decode_schedule_kernel, dim3(1), dim3(1024), 0, s, own, positions, active, slot_ids, (int)B, kMfmaChunk);
+      schedule = own;
+    }
+    a.schedule = schedule;
+    // 3 workgroups per CU is what the kernel's register use allows on the 256 CUs; never more than the worst case
+    int64_t blocks = (int64_t)B * nch * KH;
+    blocks = blocks < 768 ? blocks : 768;
+    const dim3 mgrid((unsigned)blocks);
     if (block_table) hipLaunchKernelGGL(decode_attn_mfma_kernel<true>, mgrid, dim3(256), 0, s, a);
     else hipLaunchKernelGGL(decode_attn_mfma_kernel<false>, mgrid, dim3(256), 0, s, a);
     hipLaunchKernelGGL(decode_combine_kernel<__bf16>, dim3(B, QH), dim3(64), 0, s, a);

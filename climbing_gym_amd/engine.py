@@ -269,6 +269,8 @@ class LFM25Engine:
         fp8 = self._fp8() if fp8 is None else fp8
         positions = cache.seq_lens if positions is None else positions
         rows = tokens.numel()
+        # the attention layers of one step see the same lengths: build the work list of the attention kernel once
+        schedule = ops.decode_schedule(positions, active, slot_ids, capacity=cache.max_seq_len) if cache.fp8 else None
 
         def attention_op(op, qkv):
             q, k, v = ops.prepare_qkv(qkv, op.q_norm_weight, op.k_norm_weight, self._rope_cos, self._rope_sin, positions,
@@ -276,7 +278,7 @@ class LFM25Engine:
             i = op.cache_index
             if cache.fp8:
                 out = ops.decode(q, k, v, cache.k_cache[i], cache.v_cache[i], cache.k_scales[i], cache.v_scales[i], positions,
-                                 active=active, scale=self._scaling, slot_ids=slot_ids)
+                                 active=active, scale=self._scaling, slot_ids=slot_ids, schedule=schedule)
             else:
                 ops.append_bf16_kv(k, v, cache.k_cache[i], cache.v_cache[i], positions, slot_ids, active)
                 out = ops.attend(q, cache.k_cache[i], cache.v_cache[i], None, None, positions, active=active,

@@ -224,8 +224,17 @@ def store_kv_packed(k, v, k_cache, v_cache, k_scales, v_scales, cu_seqlens, seq_
          k.size(0), k.size(1), k.size(2), c0, c1, c2, int(k_scales is not None), _code(k.dtype))
 
 
+def decode_schedule(positions, active=None, slot_ids=None, *, capacity: int):
+    """Work list of the persistent decode-attention kernel for the rows' current lengths; one list serves every
+    attention layer of a decode step (pass it to `attend(..., schedule=...)`)."""
+    rows = positions.numel()
+    schedule = torch.empty(query("lfm2_decode_schedule_size", rows, int(capacity)), device=positions.device, dtype=torch.int32)
+    call("lfm2_decode_schedule", schedule, positions, active, slot_ids, rows)
+    return schedule
+
+
 def attend(q, k_cache, v_cache, k_scales, v_scales, positions, *, active=None, scale=None, config=None,
-           slot_ids=None, window=0, block_table=None, page=16):
+           slot_ids=None, window=0, block_table=None, page=16, schedule=None):
     """lfm25_fp8_kv.py:138-167 (e4m3 history + scales) and flash_attn_with_kvcache of lfm25_cuda.py:156-165
     (`k_scales is None`: history in the model dtype).  Attends over positions [0, positions[b]]; inactive rows
     return zeros.  With `block_table` the caches are page pools [pages, page, KV heads, dim]."""
@@ -240,17 +249,18 @@ def attend(q, k_cache, v_cache, k_scales, v_scales, positions, *, active=None, s
     ws = torch.empty(query("lfm2_decode_attention_workspace", batch, query_heads, dim, capacity),
                      device=q.device, dtype=torch.float32)
     call("lfm2_decode_attention", out, q, k_cache, v_cache, k_scales, v_scales, positions, active, slot_ids,
-         block_table, 0 if block_table is None else block_table.size(1), page, ws, batch, query_heads, heads, dim,
+         block_table, 0 if block_table is None else block_table.size(1), page, schedule, ws, batch, query_heads, heads, dim,
          capacity, c0, c1, c2, float(scale if scale is not None else dim ** -0.5), int(k_scales is not None),
          _code(q.dtype))
     return out
 
 
-def decode(q, k, v, k_cache, v_cache, k_scales, v_scales, positions, *, active=None, scale=None, slot_ids=None, window=0):
+def decode(q, k, v, k_cache, v_cache, k_scales, v_scales, positions, *, active=None, scale=None, slot_ids=None, window=0,
+           schedule=None):
     """lfm25_fp8_kv.py:170-172: append the new token, then attend."""
     store_kv(k, v, k_cache, v_cache, k_scales, v_scales, positions=positions, active=active, slot_ids=slot_ids)
     return attend(q, k_cache, v_cache, k_scales, v_scales, positions, active=active, scale=scale, slot_ids=slot_ids,
-                  window=window)
+                  window=window, schedule=schedule)
 
 
 def prefill_attention(q, k, v, cu_seqlens, max_seqlen: int, scale: float | None = None):

@@ -119,14 +119,23 @@ int lfm2_store_kv_packed(const void* k, const void* v, void* k_cache, void* v_ca
  * q [B,QH,D]; history rows [0, positions[b]] of slot slot_ids[b] (or b); out [B,QH,D];
  * inactive rows produce zeros.  block_table int32[B,max_blocks] or NULL: when given, token t of
  * row b lives in page block_table[b*max_blocks + t/page] at in-page index t%page and c0 is the
- * page stride (slot-mapped paged layout).  workspace: lfm2_decode_attention_workspace() floats. */
+ * page stride (slot-mapped paged layout).  workspace: lfm2_decode_attention_workspace() floats (4-byte words). */
 int lfm2_decode_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
                           const float* k_scales, const float* v_scales, const int32_t* positions,
                           const uint8_t* active, const int32_t* slot_ids, const int32_t* block_table,
-                          int64_t max_blocks, int page, float* workspace, int64_t B, int QH, int KH, int D,
-                          int64_t capacity, int64_t c0, int64_t c1, int64_t c2, float scale, int kv_fp8,
-                          int dtype, void* stream);
+                          int64_t max_blocks, int page, const int32_t* schedule, float* workspace, int64_t B,
+                          int QH, int KH, int D, int64_t capacity, int64_t c0, int64_t c1, int64_t c2, float scale,
+                          int kv_fp8, int dtype, void* stream);
 int64_t lfm2_decode_attention_workspace(int64_t B, int QH, int D, int64_t capacity);
+
+/* Work list of the persistent decode-attention kernel: one (row, 1024-token chunk) item per chunk of every active
+ * row's history.  It depends only on positions/active/slot_ids, so the attention layers of one decode step can
+ * share it (pass it as `schedule`; NULL makes lfm2_decode_attention build its own in the workspace).
+ * schedule: int32[lfm2_decode_schedule_size(B, capacity)].  No counterpart in the reference, whose Triton grid is
+ * (rows, KV heads, splits) with a fixed split count (lfm25_fp8_kv.py:145-150). */
+int lfm2_decode_schedule(int32_t* schedule, const int32_t* positions, const uint8_t* active, const int32_t* slot_ids,
+                         int64_t B, void* stream);
+int64_t lfm2_decode_schedule_size(int64_t B, int64_t capacity);
 
 /* flash_attn_func(causal=True) of lfm25_engine.py:1415-1417 in varlen form: q [T,QH,D], k,v [T,KH,D]
  * packed by cu_seqlens int32[nseq+1]; out [T,QH,D]. */
