@@ -1,15 +1,15 @@
 // "NT" GEMMs of the LFM2 linear layers on MFMA: out[M,N] = A[M,K] . W[N,K]^T.
 //
-//   fp8  : A, W are OCP e4m3 bytes, v_mfma_f32_16x16x32_fp8_fp8, epilogue * a_scale[m] * w_scale[n]
+//   fp8  : A, W are OCP e4m3 bytes, v_mfma_f32_16x16x128_f8f6f4 (unit block scales), epilogue * a_scale[m] * w_scale[n]
 //   bf16 : v_mfma_f32_16x16x32_bf16, plain epilogue
 //
 // Both operands are K-contiguous, so the kernel works on 16-byte chunks of K for either type:
 // a workgroup stages a BM x 128 B tile of A and a BN x 128 B tile of W per step through LDS
-// (double buffered, one barrier per step, next tile prefetched into registers during the MFMAs).
+// (double buffered, one barrier per step, the next two tiles in flight in registers during the MFMAs).
 // Chunks are XOR-swizzled by row so the 16-lane column reads of the MFMA operand layout spread
-// over all banks.  A lane of lane-group g = lane/16 takes chunks g and g+4 of its row for both
-// operands, so the contraction order inside a 128 B step is permuted identically on both sides
-// and needs no shuffles.  W is the MFMA "A" operand, so a lane ends with four consecutive output
+// over all banks.  A lane of lane-group g = lane/16 takes the same chunks of its row for both
+// operands (2g, 2g+1 for e4m3; g, g+4 for bf16), so the contraction order inside a 128 B step is
+// permuted identically on both sides and needs no shuffles.  W is the MFMA "A" operand, so a lane ends with four consecutive output
 // columns of one row and stores 8 bytes at a time.
 //
 // Workgroup ids are remapped so that the M-tiles sharing one W tile run back to back on the same
@@ -23,17 +23,32 @@ constexpr int kChunksPerRow = kStepBytes / 16;
 
 __device__ __forceinline__ int lds_slot(int row, int chunk) { return row * kChunksPerRow + (chunk ^ (row & 7)); }
 
-template <int EB> struct Mfma;
-template <> struct Mfma<1> {  // e4m3: one 16 B chunk feeds two K=32 instructions
-  static __device__ __forceinline__ f32x4 run(const i32x4& w, const i32x4& a, f32x4 acc) {
-    long w0 = ((long)(unsigned)w[1] << 32) | (unsigned)w[0], w1 = ((long)(unsigned)w[3] << 32) | (unsigned)w[2];
-    long a0 = ((long)(unsigned)a[1] << 32) | (unsigned)a[0], a1 = ((long)(unsigned)a[3] << 32) | (unsigned)a[2];
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w0, a0, acc, 0, 0, 0);
-    return __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w1, a1, acc, 0, 0, 0);
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+
+// One K step (128 bytes per row) of a 16x16 output tile.  `lds_w`/`lds_a` point at the staged tiles, `wrow`/`arow`
+// are the lane's rows.  Both operands take the same chunks per lane group, so the K order inside the step is
+// permuted identically on both sides.
+template <int EB> struct StepMfma;
+template <> struct StepMfma<1> {
+  // e4m3: lane group g owns chunks 2g, 2g+1 (32 bytes) -> one v_mfma_f32_16x16x128_f8f6f4 (unit scales)
+  typedef i32x8 frag;
+  static constexpr int PASSES = 1;
+  static __device__ __forceinline__ frag load(const i32x4* tile, int row, int lgrp, int) {
+    const i32x4 lo = tile[lds_slot(row, 2 * lgrp)], hi = tile[lds_slot(row, 2 * lgrp + 1)];
+    return frag{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  }
+  static __device__ __forceinline__ f32x4 run(const frag& w, const frag& a, f32x4 acc) {
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(w, a, acc, 0, 0, 0, 0, 0, 0);
   }
 };
-template <> struct Mfma<2> {  // bf16: one chunk is one K=32 operand
-  static __device__ __forceinline__ f32x4 run(const i32x4& w, const i32x4& a, f32x4 acc) {
+template <> struct StepMfma<2> {
+  // bf16: two passes; in pass h lane group g owns chunk g + 4h (8 values) -> v_mfma_f32_16x16x32_bf16
+  typedef i32x4 frag;
+  static constexpr int PASSES = 2;
+  static __device__ __forceinline__ frag load(const i32x4* tile, int row, int lgrp, int pass) {
+    return tile[lds_slot(row, lgrp + 4 * pass)];
+  }
+  static __device__ __forceinline__ f32x4 run(const frag& w, const frag& a, f32x4 acc) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, w), __builtin_bit_cast(bf16x8, a), acc, 0, 0, 0);
   }
 };
@@ -44,7 +59,7 @@ __device__ __forceinline__ void store_out(void* out, int out_dtype, int64_t idx,
   else ((float*)out)[idx] = v;
 }
 
-template <int EB, int BM, int BN, int WM, int WN>
+template <int EB, int BM, int BN, int WM, int WN, bool KTAIL>
 __global__ void __launch_bounds__(WM * WN * 64)
 gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_t* __restrict__ A,
                const uint8_t* __restrict__ W, const float* __restrict__ a_scales, const float* __restrict__ w_scales,
@@ -71,45 +86,60 @@ gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_
   const int wm = wave % WM, wn = wave / WM;
   const int lrow = lane & 15, lgrp = lane >> 4;
 
-  i32x4 ra[A_PER], rw[W_PER];
-  auto fetch = [&](int64_t step) {
+  // Two register sets give a prefetch distance of two K steps with only two LDS buffers: while step s is
+  // multiplied out of LDS buffer s&1, set (s+1)&1 holds step s+1 in flight and set s&1 is refilled with step s+2.
+  i32x4 ra[2][A_PER], rw[2][W_PER];
+  // Loads are unconditional (addresses clamped into the operand, out-of-range chunks zeroed by a select): with
+  // no branch between issue and use the compiler keeps them in flight across the MFMAs of two K steps.
+  auto fetch = [&](int64_t step, int set) {
+    step = step < nsteps ? step : nsteps - 1;
     const int64_t kb = (step0 + step) * kStepBytes;
 #pragma unroll
     for (int i = 0; i < A_PER; ++i) {
-      const int idx = tid + i * NT;
+      int idx = tid + i * NT;
+      if (A_CHUNKS % NT != 0) idx = idx < A_CHUNKS ? idx : A_CHUNKS - 1;
       const int row = idx / kChunksPerRow, c = idx % kChunksPerRow;
-      i32x4 v = {0, 0, 0, 0};
-      if ((A_CHUNKS % NT == 0 || idx < A_CHUNKS) && kb + c * 16 < Kb) {
-        int gr = m_base + row;
-        gr = gr < M ? gr : M - 1;
-        v = *reinterpret_cast<const i32x4*>(A + (int64_t)gr * Kb + kb + c * 16);
+      int gr = m_base + row;
+      gr = gr < M ? gr : M - 1;
+      const int64_t ko = kb + c * 16;
+      if (KTAIL) {  // K bytes not a multiple of the step: chunks past the end read a valid address and become zero
+        const bool ok = ko < Kb;
+        const i32x4 v = *reinterpret_cast<const i32x4*>(A + (int64_t)gr * Kb + (ok ? ko : Kb - 16));
+        const i32x4 zero = {0, 0, 0, 0};
+        ra[set][i] = ok ? v : zero;
+      } else {
+        ra[set][i] = *reinterpret_cast<const i32x4*>(A + (int64_t)gr * Kb + ko);
       }
-      ra[i] = v;
     }
 #pragma unroll
     for (int i = 0; i < W_PER; ++i) {
-      const int idx = tid + i * NT;
+      int idx = tid + i * NT;
+      if (W_CHUNKS % NT != 0) idx = idx < W_CHUNKS ? idx : W_CHUNKS - 1;
       const int row = idx / kChunksPerRow, c = idx % kChunksPerRow;
-      i32x4 v = {0, 0, 0, 0};
-      if ((W_CHUNKS % NT == 0 || idx < W_CHUNKS) && kb + c * 16 < Kb) {
-        int gr = n_base + row;
-        gr = gr < N ? gr : N - 1;
-        v = *reinterpret_cast<const i32x4*>(W + (int64_t)gr * Kb + kb + c * 16);
+      int gr = n_base + row;
+      gr = gr < N ? gr : N - 1;
+      const int64_t ko = kb + c * 16;
+      if (KTAIL) {
+        const bool ok = ko < Kb;
+        const i32x4 v = *reinterpret_cast<const i32x4*>(W + (int64_t)gr * Kb + (ok ? ko : Kb - 16));
+        const i32x4 zero = {0, 0, 0, 0};
+        rw[set][i] = ok ? v : zero;
+      } else {
+        rw[set][i] = *reinterpret_cast<const i32x4*>(W + (int64_t)gr * Kb + ko);
       }
-      rw[i] = v;
     }
   };
-  auto stash = [&](int buf) {
+  auto stash = [&](int set, int buf) {
 #pragma unroll
     for (int i = 0; i < A_PER; ++i) {
       const int idx = tid + i * NT;
-      if (A_CHUNKS % NT == 0 || idx < A_CHUNKS) lds[buf][lds_slot(idx / kChunksPerRow, idx % kChunksPerRow)] = ra[i];
+      if (A_CHUNKS % NT == 0 || idx < A_CHUNKS) lds[buf][lds_slot(idx / kChunksPerRow, idx % kChunksPerRow)] = ra[set][i];
     }
 #pragma unroll
     for (int i = 0; i < W_PER; ++i) {
       const int idx = tid + i * NT;
       if (W_CHUNKS % NT == 0 || idx < W_CHUNKS)
-        lds[buf][A_CHUNKS + lds_slot(idx / kChunksPerRow, idx % kChunksPerRow)] = rw[i];
+        lds[buf][A_CHUNKS + lds_slot(idx / kChunksPerRow, idx % kChunksPerRow)] = rw[set][i];
     }
   };
 
@@ -119,33 +149,60 @@ gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_
 #pragma unroll
     for (int j = 0; j < NI; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  if (nsteps > 0) {
-    fetch(0);
-    stash(0);
-  }
-  __syncthreads();
-  for (int64_t s = 0; s < nsteps; ++s) {
-    const int buf = (int)(s & 1);
-    if (s + 1 < nsteps) fetch(s + 1);
+  auto multiply = [&](int buf) {
+    typedef typename StepMfma<EB>::frag frag;
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int c = lgrp + 4 * h;
-      i32x4 fa[MI], fw[NI];
+    for (int pass = 0; pass < StepMfma<EB>::PASSES; ++pass) {
+      frag fa[MI], fw[NI];
 #pragma unroll
-      for (int i = 0; i < MI; ++i) fa[i] = lds[buf][lds_slot(wm * TM + i * 16 + lrow, c)];
+      for (int i = 0; i < MI; ++i) fa[i] = StepMfma<EB>::load(&lds[buf][0], wm * TM + i * 16 + lrow, lgrp, pass);
 #pragma unroll
-      for (int j = 0; j < NI; ++j) fw[j] = lds[buf][A_CHUNKS + lds_slot(wn * TN + j * 16 + lrow, c)];
+      for (int j = 0; j < NI; ++j) fw[j] = StepMfma<EB>::load(&lds[buf][A_CHUNKS], wn * TN + j * 16 + lrow, lgrp, pass);
 #pragma unroll
       for (int i = 0; i < MI; ++i)
 #pragma unroll
-        for (int j = 0; j < NI; ++j) acc[i][j] = Mfma<EB>::run(fw[j], fa[i], acc[i][j]);
+        for (int j = 0; j < NI; ++j) acc[i][j] = StepMfma<EB>::run(fw[j], fa[i], acc[i][j]);
     }
-    if (s + 1 < nsteps) stash(buf ^ 1);
+  };
+
+  if (nsteps > 0) {
+    fetch(0, 0);
+    fetch(1, 1);
+    stash(0, 0);
+  }
+  __syncthreads();
+  // Steps beyond the last one are clamped re-reads whose data is never multiplied.
+  // sched_barrier keeps the scheduler from sinking the prefetch loads down to their use after the MFMAs.
+  for (int64_t s = 0; s < nsteps; s += 2) {
+    fetch(s + 2, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(0);
+    __builtin_amdgcn_sched_barrier(0);
+    stash(1, 1);
     __syncthreads();
+    if (s + 1 < nsteps) {
+      fetch(s + 3, 1);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(1);
+      __builtin_amdgcn_sched_barrier(0);
+      stash(0, 0);
+      __syncthreads();
+    }
   }
 
   // Epilogue: lane holds out[m = .. + lrow][n = .. + 4*lgrp + r], r = 0..3.
   const bool split = partial != nullptr;
+  auto finish = [&](f32x4 v, int m, int n, float sa) {  // scale (row then column) and store up to 4 columns
+    if (a_scales)
+      for (int r = 0; r < 4; ++r) v[r] = (v[r] * sa) * (n + r < N ? w_scales[n + r] : 0.f);
+    const int64_t idx = (int64_t)m * N + n;
+    if (out_dtype == LFM2_DTYPE_BF16 && n + 3 < N && (N & 3) == 0) {
+      bf16x4 o = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
+      *reinterpret_cast<bf16x4*>((__bf16*)out + idx) = o;
+    } else {
+      for (int r = 0; r < 4 && n + r < N; ++r) store_out(out, out_dtype, idx + r, v[r]);
+    }
+  };
 #pragma unroll
   for (int i = 0; i < MI; ++i) {
     const int m = m_base + wm * TM + i * 16 + lrow;
@@ -155,27 +212,21 @@ gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_
     for (int j = 0; j < NI; ++j) {
       const int n = n_base + wn * TN + j * 16 + 4 * lgrp;
       if (n >= N) continue;
-      f32x4 v = acc[i][j];
       if (split) {
         float* dst = partial + ((int64_t)blockIdx.y * M + m) * N + n;
-        if (n + 3 < N && (N & 3) == 0) *reinterpret_cast<f32x4*>(dst) = v;
-        else for (int r = 0; r < 4 && n + r < N; ++r) dst[r] = v[r];
-        continue;
-      }
-      if (a_scales)
-        for (int r = 0; r < 4; ++r) v[r] = (v[r] * sa) * (n + r < N ? w_scales[n + r] : 0.f);
-      const int64_t idx = (int64_t)m * N + n;
-      if (out_dtype == LFM2_DTYPE_BF16 && n + 3 < N && (N & 3) == 0) {
-        bf16x4 o = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
-        *reinterpret_cast<bf16x4*>((__bf16*)out + idx) = o;
+        if (n + 3 < N && (N & 3) == 0) *reinterpret_cast<f32x4*>(dst) = acc[i][j];
+        else for (int r = 0; r < 4 && n + r < N; ++r) dst[r] = acc[i][j][r];
       } else {
-        for (int r = 0; r < 4 && n + r < N; ++r) store_out(out, out_dtype, idx + r, v[r]);
+        finish(acc[i][j], m, n, sa);
       }
     }
   }
 }
 
-// Sum split-K partials in split order, then scale (lfm25_fp8.py:94-105 order: row scale, column scale).
+// Sum split-K partials in split order, then scale (row scale, then column scale).  A separate launch on purpose:
+// the eight XCDs have private L2s, so partials written by workgroups on other XCDs are only visible to a reader
+// cheaply at a kernel boundary; an in-kernel "last workgroup reduces" scheme needs device-scope fences that write
+// back and invalidate L2 and measured ten times slower.
 __global__ void __launch_bounds__(256)
 reduce_split_kernel(void* out, const float* partial, const float* a_scales, const float* w_scales, int64_t M, int64_t N,
                     int splits, int out_dtype) {
@@ -211,27 +262,29 @@ gemm_naive_kernel(void* out, const uint8_t* A, const uint8_t* W, const float* a_
 }
 
 struct TileInfo { int bm, bn; };
-constexpr int kNumTiles = 6;
-constexpr TileInfo kTiles[kNumTiles] = {{16, 64}, {32, 64}, {64, 64}, {128, 64}, {128, 128}, {64, 128}};
+constexpr int kNumTiles = 9;
+constexpr TileInfo kTiles[kNumTiles] = {{16, 64}, {32, 64}, {64, 64}, {128, 64}, {128, 128}, {64, 128},
+                                        {128, 128}, {64, 128}, {128, 64}};
 
 struct Plan { int tile, splits; };
 
-// Default tile/split choice: the largest tile that still gives every CU work, then split K until
-// the chip (256 CUs) is covered, keeping at least four 128-byte steps per split.
+// Default tile/split choice, from sweeps on MI355X at M = 256 (decode) and M = 4096 (prefill): the 8-wave 128x128
+// tile once it alone fills the 256 CUs, otherwise the largest smaller tile that gives every CU about two
+// workgroups; K is split (2 or 4 ways) only for long-K shapes that still leave CUs idle.
 Plan default_plan(int64_t M, int64_t N, int64_t Kb) {
+  auto count = [&](int t) { return ((M + kTiles[t].bm - 1) / kTiles[t].bm) * ((N + kTiles[t].bn - 1) / kTiles[t].bn); };
   int tile;
   if (M <= 16) tile = 0;
   else if (M <= 32) tile = 1;
-  else if (M <= 64) tile = 2;
-  else {
-    const int64_t big = ((M + 127) / 128) * ((N + 127) / 128);
-    const int64_t mid = ((M + 127) / 128) * ((N + 63) / 64);
-    tile = big >= 512 ? 4 : (mid >= 384 ? 3 : 2);
-  }
-  const int64_t tiles = ((M + kTiles[tile].bm - 1) / kTiles[tile].bm) * ((N + kTiles[tile].bn - 1) / kTiles[tile].bn);
+  else if (count(6) >= 256) tile = 6;
+  else if (count(2) >= 512) tile = 2;
+  else if (count(1) >= 256 || M <= 64) tile = M <= 64 ? 2 : 1;
+  else tile = 2;
   const int64_t steps = (Kb + kStepBytes - 1) / kStepBytes;
   int splits = 1;
-  while (tiles * splits < 256 && splits < 16 && steps / (splits * 2) >= 4) splits *= 2;
+  if (steps >= 64 && count(tile) < 128) {  // only very long, very narrow products are worth a second pass over partials
+    while (count(tile) * splits < 256 && splits < 4 && steps / (splits * 2) >= 16) splits *= 2;
+  }
   return {tile, splits};
 }
 
@@ -241,8 +294,13 @@ void launch_tile(void* out, float* partial, const uint8_t* A, const uint8_t* W, 
   const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   const int64_t steps = (Kb + kStepBytes - 1) / kStepBytes;
   const int per = (int)((steps + splits - 1) / splits);
-  hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN>), dim3((tiles + 7) / 8 * 8, splits), dim3(WM * WN * 64), 0, s, out,
-                     splits > 1 ? partial : nullptr, A, W, as, ws, M, N, Kb, per, out_dtype);
+  const dim3 grid((tiles + 7) / 8 * 8, splits), block(WM * WN * 64);
+  if (Kb % kStepBytes == 0)
+    hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN, false>), grid, block, 0, s, out, splits > 1 ? partial : nullptr, A, W,
+                       as, ws, M, N, Kb, per, out_dtype);
+  else
+    hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN, true>), grid, block, 0, s, out, splits > 1 ? partial : nullptr, A, W,
+                       as, ws, M, N, Kb, per, out_dtype);
 }
 
 template <int EB>
@@ -278,18 +336,15 @@ int gemm_entry(const char* name, void* out, const void* a, const float* as, cons
     TILE_(3, 128, 64, 2, 2);
     TILE_(4, 128, 128, 2, 2);
     TILE_(5, 64, 128, 2, 2);
+    TILE_(6, 128, 128, 2, 4);
+    TILE_(7, 64, 128, 2, 4);
+    TILE_(8, 128, 64, 4, 2);
   }
 #undef TILE_
   if (plan.splits > 1)
     hipLaunchKernelGGL(reduce_split_kernel, dim3(ceil_div(M * N, 256)), dim3(256), 0, s, out, workspace, as, ws, M, N,
                        plan.splits, out_dtype);
   LFM2_LAUNCH_CHECK();
-}
-
-int64_t workspace_floats(int64_t M, int64_t N, int64_t Kb) {
-  if (Kb % 16 != 0) return 0;
-  // Upper bound over every split choice the entry point accepts (<= 16 splits).
-  return 16 * M * N;
 }
 
 }  // namespace

@@ -163,7 +163,7 @@ def test_fp8_projection_matches_independently_dequantized_operands(ops, batch, w
     reference = (x.float() @ weight.float().T)
     assert (actual.float().cpu() - reference).norm() / reference.norm() < 0.065
     if width % 16 == 0:
-        for tile in range(6):
+        for tile in range(9):
             for split in (1, 2, 4):
                 got = packed.linear_quantized(q, scale, config=(tile, split))
                 torch.testing.assert_close(got.float().cpu(), expected, atol=0.02, rtol=0.015)
@@ -194,7 +194,7 @@ def test_bf16_linear_matches_fp32_matmul_of_the_same_operands(ops, m, k, n):
     torch.manual_seed(7)
     x, w = torch.randn(m, k).bfloat16(), (torch.randn(n, k) * 0.02).bfloat16()
     expected = x.float() @ w.float().T
-    for tile, split in [(-1, 0), (0, 1), (2, 2), (4, 1), (5, 4)]:
+    for tile, split in [(-1, 0), (0, 1), (2, 2), (4, 1), (5, 4), (6, 1), (7, 2), (8, 1)]:
         got = ops.linear(x.to(DEV), w.to(DEV), tile=tile, split_k=split)
         torch.testing.assert_close(got.float().cpu(), expected, atol=2e-3, rtol=2 ** -7)
 
