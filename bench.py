@@ -54,7 +54,8 @@ def build_engine(args, state):
 
 
 def time_decode_attention(engine, session, samples):
-    """Average duration (s) of one decode-attention call at the batch's current context lengths, from HIP events
+    """Average duration (s) of one decode-attention call (the persistent split kernel plus its combine kernel, over the
+    work list the decode step shares between its layers) at the batch's current context lengths, from HIP events
     recorded on the launch stream around back-to-back launches, and the algorithmic bytes of one call."""
     from climbing_gym_amd import ops
     cfg, cache = engine.config, session.entry.cache
@@ -62,6 +63,7 @@ def time_decode_attention(engine, session, samples):
     q = torch.randn((rows, 1, cfg.num_attention_heads, cfg.head_dim), device="cuda", dtype=torch.bfloat16)
     positions = (cache.seq_lens - 1).clamp_min(0).contiguous()
     active = torch.ones(rows, device="cuda", dtype=torch.bool)
+    schedule = ops.decode_schedule(positions, active, capacity=cache.max_seq_len) if cache.fp8 else None
     stream = torch.cuda.current_stream()
     begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     total_ms, launches = 0.0, 0
@@ -69,10 +71,10 @@ def time_decode_attention(engine, session, samples):
         args = (q, cache.k_cache[layer], cache.v_cache[layer],
                 None if cache.k_scales is None else cache.k_scales[layer],
                 None if cache.v_scales is None else cache.v_scales[layer], positions)
-        ops.attend(*args, active=active, scale=engine._scaling)  # warm
+        ops.attend(*args, active=active, scale=engine._scaling, schedule=schedule)  # warm
         begin.record(stream)
         for _ in range(samples):
-            ops.attend(*args, active=active, scale=engine._scaling)
+            ops.attend(*args, active=active, scale=engine._scaling, schedule=schedule)
         end.record(stream)
         end.synchronize()
         total_ms += begin.elapsed_time(end)
@@ -81,6 +83,30 @@ def time_decode_attention(engine, session, samples):
     kv_token = cfg.num_key_value_heads * cfg.head_dim * 2 * (1 if cache.fp8 else 2) + (cfg.num_key_value_heads * 2 * 4 if cache.fp8 else 0)
     bytes_per_call = tokens * kv_token + 2 * rows * cfg.num_attention_heads * cfg.head_dim * 2
     return total_ms / 1000 / launches, bytes_per_call, tokens
+
+
+def calibration_copy():
+    """One plain elementwise copy of known size (256 MiB read, 256 MiB written).  It costs nothing measurable in a
+    normal run; under `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` its counter reading gives the factor that turns
+    the decode-attention kernel's counter readings into bytes."""
+    src = torch.ones(64 << 20, device="cuda", dtype=torch.int32)
+    dst = torch.empty_like(src)
+    torch.mul(src, 1, out=dst)
+    torch.cuda.synchronize()
+
+
+def measured_traffic(args, attn_bytes):
+    """HBM bytes per decode-attention call: the ratio of counter-measured to algorithmic bytes in the committed
+    FETCH_SIZE / WRITE_SIZE summary (taken on this workload a few decode steps earlier or later), applied to this
+    run's algorithmic bytes.  None when the summary is absent or was taken on another workload."""
+    path = os.path.join(ROOT, "profiles", "decode_attention_hbm_traffic.json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        rec = json.load(f)
+    same = (rec.get("batch") == args.batch and rec.get("precision") == args.precision
+            and rec.get("prompt_range") == [args.prompt_low, args.prompt_high])
+    return int(rec["ratio"] * attn_bytes) if same else None
 
 
 def cpu_baseline(args, state, prompts):
@@ -138,6 +164,7 @@ def main():
         elapsed = time.perf_counter() - t0
         assert not finished, "no sequence may finish inside the timed region"
         attn_s, attn_bytes, ctx_tokens = time_decode_attention(engine, session, args.attn_samples)
+        calibration_copy()
         kv_token = 6 * (attn_bytes - 2 * args.batch * 32 * 64 * 2) // max(ctx_tokens, 1)
     fp8 = args.precision == "fp8"
     weights = sum(w.numel() for w in set(engine.weights.linear_matrices())) * (1 if fp8 else 2)
@@ -156,9 +183,10 @@ def main():
                    "context_tokens": ctx_tokens, "prefill_tok_per_s": round(sum(map(len, prompts)) / prefill_s, 1),
                    "step_algorithmic_bytes": step_bytes,
                    "step_hbm_fraction": round(step_bytes / (ms_per_step / 1000) / 1e9 / HBM_PEAK_GBS, 4)},
-        "roofline": {"kernel": "decode_attn_kernel (ragged GQA decode attention, e4m3 KV)" if fp8 else "decode_attn_kernel (bf16 KV)",
+        "roofline": {"kernel": "decode_attn_mfma_kernel + decode_combine_kernel (one ragged GQA decode-attention call, e4m3 KV)"
+                               if fp8 else "decode_attn_kernel + decode_combine_kernel (bf16 KV)",
                      "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(args, attn_bytes),
                      "avg_launch_us": round(attn_s * 1e6, 2), "algorithmic_bytes_per_launch": attn_bytes},
     }
     del session
