@@ -25,6 +25,10 @@ _SIGNATURES = {
     "lfm2_swiglu_fp8": "pppllip",
     "lfm2_quantize_rows": "pppllip",
     "lfm2_conv_update": "pppppp" "lllip",
+    "lfm2_conv_update_fp8": "ppppppp" "lllip",
+    "lfm2_prepare_qkv_store": "ppppppppppppp" "liiilflllii" "p",
+    "lfm2_rms_norm_fp8_split": "pppp" "i" "pppp" "llfip",
+    "lfm2_fp8_gemm_partials": "ppp" "llliip",
     "lfm2_prepare_qkv": "ppppppppp" "liiilfip",
     "lfm2_conv_prefill": "ppppppp" "llllip",
     "lfm2_fp8_gemm": "pppppp" "llliiip",
@@ -32,7 +36,7 @@ _SIGNATURES = {
     "lfm2_store_kv_fp8": "ppppppppp" "lliilllllllllip",
     "lfm2_append_kv": "ppppppp" "liilllip",
     "lfm2_store_kv_packed": "ppppppppp" "liillliip",
-    "lfm2_decode_attention": "pppppppppp" "lipp" "liiillllfiip",
+    "lfm2_decode_attention": "pppppppppp" "lipp" "liiillllfiippp",
     "lfm2_decode_schedule": "pppp" "lp",
     "lfm2_prefill_attention": "ppppp" "lliiifip",
     "lfm2_build_token_map": "ppp" "llp",
@@ -47,6 +51,7 @@ _SIGNATURES = {
 }
 _INT64_RESULT = {
     "lfm2_fp8_gemm_workspace": "lll",
+    "lfm2_fp8_gemm_default_splits": "lll",
     "lfm2_bf16_gemm_workspace": "lll",
     "lfm2_decode_attention_workspace": "liil",
     "lfm2_decode_schedule_size": "ll",

@@ -489,6 +489,69 @@ __global__ void __launch_bounds__(64) decode_combine_kernel(DecodeArgs a) {
   }
 }
 
+// The same merge for a whole row (all query heads) followed by the row's e4m3 quantisation, for callers whose next
+// step is an FP8 projection: values are rounded to the model dtype first, exactly as the two separate launches do.
+// Sixteen waves per row, wave w owning query heads w, w+16, ...; with NC > 0 the chunk loops are fully unrolled over
+// NC predicated iterations so that all of a lane's partial loads are in flight together (the partials were written
+// by other XCDs and come from beyond the local L2, so each dependent round costs a full memory latency).
+template <typename T, int NC>
+__global__ void __launch_bounds__(1024) decode_combine_fp8_kernel(DecodeArgs a, uint8_t* q_out, float* q_scales) {
+  constexpr int kMaxPerLane = 4, kWavesPerRow = 16;
+  __shared__ float red[kWavesPerRow];
+  const int b = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int len = a.positions[b] + 1;
+  if (a.active && !a.active[b]) len = 0;
+  if (a.slot_ids && a.slot_ids[b] < 0) len = 0;
+  const int n = len > 0 ? (len + a.chunk - 1) / a.chunk : 0;
+  const int per_head = (a.D + 63) / 64;
+  float y[kMaxPerLane];
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < kMaxPerLane; ++i) {
+    const int qh = wave + kWavesPerRow * (i / per_head), d = lane + 64 * (i % per_head);
+    y[i] = 0.f;
+    if (qh < a.QH && d < a.D && n > 0) {
+      const int64_t prow = ((int64_t)b * a.QH + qh) * a.nchunks;
+      float mm = -1.0e30f, lt = 0.f, o = 0.f;
+      if constexpr (NC > 0) {
+        float m[NC], l[NC], acc[NC];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+          const int cc = c < n ? c : 0;
+          m[c] = a.ws_m[prow + cc]; l[c] = a.ws_l[prow + cc]; acc[c] = a.ws_acc[(prow + cc) * a.D + d];
+        }
+#pragma unroll
+        for (int c = 0; c < NC; ++c) if (c < n) mm = fmaxf(mm, m[c]);
+#pragma unroll
+        for (int c = 0; c < NC; ++c) if (c < n) lt = fmaf(l[c], exp2f(m[c] - mm), lt);
+#pragma unroll
+        for (int c = 0; c < NC; ++c) if (c < n) o = fmaf(acc[c], exp2f(m[c] - mm), o);
+      } else {
+        for (int c = 0; c < n; ++c) mm = fmaxf(mm, a.ws_m[prow + c]);
+        for (int c = 0; c < n; ++c) lt = fmaf(a.ws_l[prow + c], exp2f(a.ws_m[prow + c] - mm), lt);
+        for (int c = 0; c < n; ++c) o = fmaf(a.ws_acc[(prow + c) * a.D + d], exp2f(a.ws_m[prow + c] - mm), o);
+      }
+      y[i] = round_to<T>(o * (1.0f / fmaxf(lt, 1.0e-20f)));
+      amax = fmaxf(amax, fabsf(y[i]));
+    }
+  }
+  amax = block_max<kWavesPerRow>(amax, red);
+  const float scale = fmaxf(amax / LFM2_E4M3_MAX, 1.0e-12f);
+  if (threadIdx.x == 0) q_scales[b] = scale;
+  uint8_t* dst = q_out + (int64_t)b * a.QH * a.D;
+#pragma unroll
+  for (int i = 0; i < kMaxPerLane; ++i) {
+    const int qh = wave + kWavesPerRow * (i / per_head), d = lane + 64 * (i % per_head);
+    if (qh < a.QH && d < a.D) dst[qh * a.D + d] = to_e4m3(y[i] / scale);
+  }
+}
+
+template <typename T>
+void launch_combine_fp8(const DecodeArgs& a, int64_t B, uint8_t* out_q, float* out_scales, hipStream_t s) {
+  if (a.nchunks <= 8) hipLaunchKernelGGL((decode_combine_fp8_kernel<T, 8>), dim3(B), dim3(1024), 0, s, a, out_q, out_scales);
+  else hipLaunchKernelGGL((decode_combine_fp8_kernel<T, 0>), dim3(B), dim3(1024), 0, s, a, out_q, out_scales);
+}
+
 // ===================================================================================== prefill attention
 template <typename T> struct HalfMfma;
 template <> struct HalfMfma<__bf16> {
@@ -715,8 +778,11 @@ extern "C" int lfm2_decode_attention(void* out, const void* q, const void* k_cac
                                      int64_t max_blocks, int page, const int32_t* schedule, float* workspace, int64_t B,
                                      int QH, int KH, int D,
                                      int64_t capacity, int64_t c0, int64_t c1, int64_t c2, float scale, int kv_fp8,
-                                     int dtype, void* stream) {
+                                     int dtype, uint8_t* out_q, float* out_scales, void* stream) {
   LFM2_REQUIRE(B > 0 && QH > 0 && KH > 0 && capacity > 0, "decode_attention: empty shape");
+  LFM2_REQUIRE((out_q == nullptr) == (out_scales == nullptr), "decode_attention: quantised output needs values and scales");
+  LFM2_REQUIRE(out_q != nullptr || out != nullptr, "decode_attention: no output");
+  LFM2_REQUIRE(out_q == nullptr || (int64_t)((QH + 15) / 16) * ((D + 63) / 64) <= 4, "decode_attention: quantised output supports at most 4096 values per row");
   LFM2_REQUIRE(QH % KH == 0, "decode_attention: %d query heads not divisible by %d KV heads", QH, KH);
   LFM2_REQUIRE(positions && workspace, "decode_attention: positions and workspace are required");
   LFM2_REQUIRE(!kv_fp8 || (k_scales && v_scales), "decode_attention: e4m3 history without scales");
@@ -753,7 +819,8 @@ extern "C" int lfm2_decode_attention(void* out, const void* q, const void* k_cac
     const dim3 mgrid((unsigned)blocks);
     if (block_table) hipLaunchKernelGGL(decode_attn_mfma_kernel<true>, mgrid, dim3(256), 0, s, a);
     else hipLaunchKernelGGL(decode_attn_mfma_kernel<false>, mgrid, dim3(256), 0, s, a);
-    hipLaunchKernelGGL(decode_combine_kernel<__bf16>, dim3(B, QH), dim3(64), 0, s, a);
+    if (out_q) launch_combine_fp8<__bf16>(a, B, out_q, out_scales, s);
+    else hipLaunchKernelGGL(decode_combine_kernel<__bf16>, dim3(B, QH), dim3(64), 0, s, a);
     LFM2_LAUNCH_CHECK();
   }
   const dim3 grid(nch, KH * ((G + kGB - 1) / kGB), B);
@@ -765,7 +832,8 @@ extern "C" int lfm2_decode_attention(void* out, const void* q, const void* k_cac
     case 64: DEC_(64); break;
     case 128: DEC_(128); break;
     default: DEC_(256); break;
-  } hipLaunchKernelGGL(decode_combine_kernel<T>, dim3(B, QH), dim3(64), 0, s, a));
+  } if (out_q) launch_combine_fp8<T>(a, B, out_q, out_scales, s);
+    else hipLaunchKernelGGL(decode_combine_kernel<T>, dim3(B, QH), dim3(64), 0, s, a));
 #undef DEC_
   LFM2_LAUNCH_CHECK();
 }

@@ -89,10 +89,21 @@ extern "C" int lfm2_embedding(void* out, const void* table, const int64_t* token
 // ------------------------------------------------------------------------------------ RMSNorm (+e4m3)
 // NV = 16-byte vectors per thread held in registers; NV == 0 selects the scalar path that
 // recomputes values from global memory in each pass (any H).
+// With `split.partial` set the input row is not read from `x` but rebuilt from split-K partial products of an FP8
+// projection, sum over splits in split order, times the row's activation scale, times the column's weight scale,
+// rounded to T: the value the projection's own reduce pass would have stored.
+struct SplitInput {
+  const float* partial;   // [splits, M, H] or NULL
+  const float* a_scales;  // [M]
+  const float* w_scales;  // [H]
+  int64_t stride;         // M * H
+  int splits;
+};
+
 template <typename T, int NV, bool ADD, bool FP8>
 __global__ void __launch_bounds__(kThreads)
 rms_norm_kernel(T* out, uint8_t* q, float* scales, T* summed, const T* x, const T* w, const T* res, int64_t H,
-                float eps) {
+                float eps, SplitInput split) {
   __shared__ float red[kWaves];
   const int64_t row = blockIdx.x;
   constexpr int N = Vec<T>::N;
@@ -107,7 +118,20 @@ rms_norm_kernel(T* out, uint8_t* q, float* scales, T* summed, const T* x, const 
     for (int j = 0; j < NV; ++j) {
       const int64_t i = (int64_t)(j * kThreads + threadIdx.x) * N;
       if (i < H) {
-        load_vec<T>(x + i, v[j]);
+        if (split.partial) {
+          const float sa = split.a_scales[row];
+#pragma unroll
+          for (int e = 0; e < N; ++e) v[j][e] = 0.f;
+          for (int sp = 0; sp < split.splits; ++sp) {
+            const float* p = split.partial + sp * split.stride + row * H + i;
+#pragma unroll
+            for (int e = 0; e < N; ++e) v[j][e] += p[e];
+          }
+#pragma unroll
+          for (int e = 0; e < N; ++e) v[j][e] = round_to<T>((v[j][e] * sa) * split.w_scales[i + e]);
+        } else {
+          load_vec<T>(x + i, v[j]);
+        }
         if (ADD) {
           float r[N];
           load_vec<T>(res + i, r);
@@ -198,11 +222,12 @@ template <typename T> static int pick_nv(int64_t width) {
 
 template <typename T, bool ADD, bool FP8>
 static void launch_rms(void* out, uint8_t* q, float* scales, void* summed, const void* x, const void* w,
-                       const void* res, int64_t M, int64_t H, float eps, hipStream_t s) {
+                       const void* res, int64_t M, int64_t H, float eps, hipStream_t s,
+                       SplitInput split = SplitInput{nullptr, nullptr, nullptr, 0, 0}) {
   const int nv = pick_nv<T>(H);
 #define RMS_(NVV)                                                                                            \
   hipLaunchKernelGGL((rms_norm_kernel<T, NVV, ADD, FP8>), dim3(M), dim3(kThreads), 0, s, (T*)out, q, scales, \
-                     (T*)summed, (const T*)x, (const T*)w, (const T*)res, H, eps)
+                     (T*)summed, (const T*)x, (const T*)w, (const T*)res, H, eps, split)
   LAUNCH_NV(nv, RMS_(1), RMS_(2), RMS_(4), RMS_(8), RMS_(16), RMS_(0));
 #undef RMS_
 }
@@ -224,6 +249,21 @@ extern "C" int lfm2_rms_norm_fp8(uint8_t* q, float* scales, void* summed, const 
   hipStream_t s = (hipStream_t)stream;
   DISPATCH_DTYPE(dtype, if (residual) launch_rms<T, true, true>(nullptr, q, scales, summed, x, weight, residual, M, H, eps, s);
                  else launch_rms<T, false, true>(nullptr, q, scales, nullptr, x, weight, nullptr, M, H, eps, s));
+  LFM2_LAUNCH_CHECK();
+}
+
+extern "C" int lfm2_rms_norm_fp8_split(uint8_t* q, float* scales, void* summed, const float* partial, int splits,
+                                       const float* a_scales, const float* w_scales, const void* weight,
+                                       const void* residual, int64_t M, int64_t H, float eps, int dtype, void* stream) {
+  LFM2_REQUIRE(M > 0 && H > 0, "rms_norm_fp8_split: empty shape");
+  LFM2_REQUIRE(partial && a_scales && w_scales && splits >= 1, "rms_norm_fp8_split: partial products and both scale vectors are required");
+  LFM2_REQUIRE(residual == nullptr || summed != nullptr, "rms_norm_fp8_split: residual given without a summed output");
+  const int vec = dtype == LFM2_DTYPE_F32 ? 4 : 8;
+  LFM2_REQUIRE(H % vec == 0 && H <= (int64_t)16 * kThreads * vec, "rms_norm_fp8_split: width %ld is not a multiple of %d or too wide", (long)H, vec);
+  const SplitInput split{partial, a_scales, w_scales, M * H, splits};
+  hipStream_t s = (hipStream_t)stream;
+  DISPATCH_DTYPE(dtype, if (residual) launch_rms<T, true, true>(nullptr, q, scales, summed, nullptr, weight, residual, M, H, eps, s, split);
+                 else launch_rms<T, false, true>(nullptr, q, scales, nullptr, nullptr, weight, nullptr, M, H, eps, s, split));
   LFM2_LAUNCH_CHECK();
 }
 
@@ -333,26 +373,71 @@ extern "C" int lfm2_quantize_rows(uint8_t* q, float* scales, const void* x, int6
 }
 
 // ------------------------------------------------------------------------------------ short-conv update
+// One channel of the gated short conv: taps (state[1], state[2], b*x) with weights w[0..2]; returns c * conv and the
+// new state entry b*x, every product and the tap sum rounded to T as the reference's kernel rounds them.
+template <typename T>
+__device__ __forceinline__ float conv_channel(float b, float c, float x, float s0, float s1, float w0, float w1, float w2,
+                                              float* bx_out) {
+  const float bx = round_to<T>(b * x);
+  const float p0 = round_to<T>(s0 * w0), p1 = round_to<T>(s1 * w1), p2 = round_to<T>(bx * w2);
+  const float conv = round_to<T>((p0 + p1) + p2);
+  *bx_out = bx;
+  return round_to<T>(c * conv);
+}
+
+// Eight consecutive channels of one row with 16-byte accesses (16-bit T): 3 loads of the (B, C, x) thirds, 3 of the
+// weights [8][3], 3 loads and 3 stores of the state [8][3].
+template <typename T>
+__device__ __forceinline__ void conv_group8(const T* in, const T* w, T* st, int64_t H, int64_t col, bool on, float* y) {
+  float b[8], c[8], x[8], wt[24], s[24];
+  load_vec<T>(in + col, b);
+  load_vec<T>(in + H + col, c);
+  load_vec<T>(in + 2 * H + col, x);
+#pragma unroll
+  for (int v = 0; v < 3; ++v) { load_vec<T>(w + col * 3 + 8 * v, wt + 8 * v); load_vec<T>(st + col * 3 + 8 * v, s + 8 * v); }
+  float ns[24];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    float bx;
+    y[e] = conv_channel<T>(b[e], c[e], x[e], s[3 * e + 1], s[3 * e + 2], wt[3 * e], wt[3 * e + 1], wt[3 * e + 2], &bx);
+    ns[3 * e] = s[3 * e + 1]; ns[3 * e + 1] = s[3 * e + 2]; ns[3 * e + 2] = bx;
+  }
+  if (on) {
+#pragma unroll
+    for (int v = 0; v < 3; ++v) store_vec<T>(st + col * 3 + 8 * v, ns + 8 * v);
+  }
+}
+
 template <typename T>
 __global__ void __launch_bounds__(kThreads)
 conv_update_kernel(T* out, const T* bcx, const T* w, T* state, const uint8_t* active, const int32_t* slot_ids, int64_t H) {
   const int64_t row = blockIdx.y;
-  const int64_t col = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-  if (col >= H) return;
   int64_t slot = row;
   if (slot_ids) { const int32_t s = slot_ids[row]; slot = s < 0 ? 0 : s; }
   const bool on = active ? active[row] != 0 : true;
   const T* in = bcx + row * 3 * H;
-  const float b = Elem<T>::load(in[col]), c = Elem<T>::load(in[H + col]), x = Elem<T>::load(in[2 * H + col]);
-  const float bx = round_to<T>(b * x);
-  T* st = state + (slot * H + col) * 3;
-  const T t1 = st[1], t2 = st[2];
-  const float s0 = Elem<T>::load(t1), s1 = Elem<T>::load(t2);
-  const float w0 = Elem<T>::load(w[col * 3]), w1 = Elem<T>::load(w[col * 3 + 1]), w2 = Elem<T>::load(w[col * 3 + 2]);
-  const float p0 = round_to<T>(s0 * w0), p1 = round_to<T>(s1 * w1), p2 = round_to<T>(bx * w2);
-  const float conv = round_to<T>((p0 + p1) + p2);
-  if (on) { st[0] = t1; st[1] = t2; st[2] = Elem<T>::store(bx); }
-  out[row * H + col] = Elem<T>::store(c * conv);
+  T* st = state + slot * H * 3;
+  if constexpr (sizeof(T) == 2) {
+    if (H % 8 == 0) {
+      const int64_t col = ((int64_t)blockIdx.x * kThreads + threadIdx.x) * 8;
+      if (col >= H) return;
+      float y[8];
+      conv_group8<T>(in, w, st, H, col, on, y);
+      store_vec<T>(out + row * H + col, y);
+      return;
+    }
+  }
+  for (int e = 0; e < 8; ++e) {
+    const int64_t col = ((int64_t)blockIdx.x * kThreads + threadIdx.x) * 8 + e;
+    if (col >= H) return;
+    float bx;
+    const T t1 = st[col * 3 + 1], t2 = st[col * 3 + 2];
+    const float y = conv_channel<T>(Elem<T>::load(in[col]), Elem<T>::load(in[H + col]), Elem<T>::load(in[2 * H + col]),
+                                    Elem<T>::load(t1), Elem<T>::load(t2), Elem<T>::load(w[col * 3]),
+                                    Elem<T>::load(w[col * 3 + 1]), Elem<T>::load(w[col * 3 + 2]), &bx);
+    if (on) { st[col * 3] = t1; st[col * 3 + 1] = t2; st[col * 3 + 2] = Elem<T>::store(bx); }
+    out[row * H + col] = Elem<T>::store(y);
+  }
 }
 
 extern "C" int lfm2_conv_update(void* out, const void* bcx, const void* weight, void* state, const uint8_t* active,
@@ -360,9 +445,62 @@ extern "C" int lfm2_conv_update(void* out, const void* bcx, const void* weight, 
   LFM2_REQUIRE(M > 0 && H > 0 && slots > 0, "conv_update: empty shape");
   LFM2_REQUIRE(slot_ids != nullptr || M <= slots, "conv_update: %ld rows but only %ld state slots", (long)M, (long)slots);
   LFM2_REQUIRE(M <= 65535, "conv_update: more than 65535 rows");
-  DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(conv_update_kernel<T>, dim3(ceil_div(H, kThreads), M), dim3(kThreads), 0,
+  DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(conv_update_kernel<T>, dim3(ceil_div(H, kThreads * 8), M), dim3(kThreads), 0,
                                            (hipStream_t)stream, (T*)out, (const T*)bcx, (const T*)weight, (T*)state,
                                            active, slot_ids, H));
+  LFM2_LAUNCH_CHECK();
+}
+
+// conv_update followed by per-row e4m3 quantisation of its (model-dtype rounded) output, in one launch: one
+// workgroup per row keeps the row's outputs in registers between the amax reduction and the conversion.
+// NG = groups of eight consecutive channels per thread (H <= NG * 2048, H a multiple of 8, 16-bit T).
+template <typename T, int NG>
+__global__ void __launch_bounds__(kThreads)
+conv_update_fp8_kernel(uint8_t* q, float* scales, const T* bcx, const T* w, T* state, const uint8_t* active,
+                       const int32_t* slot_ids, int64_t H) {
+  __shared__ float red[kWaves];
+  const int64_t row = blockIdx.x;
+  int64_t slot = row;
+  if (slot_ids) { const int32_t s = slot_ids[row]; slot = s < 0 ? 0 : s; }
+  const bool on = active ? active[row] != 0 : true;
+  const T* in = bcx + row * 3 * H;
+  T* st = state + slot * H * 3;
+  float y[NG][8];
+  float amax = 0.f;
+#pragma unroll
+  for (int g = 0; g < NG; ++g) {
+    const int64_t col = ((int64_t)g * kThreads + threadIdx.x) * 8;
+    if (col < H) {
+      conv_group8<T>(in, w, st, H, col, on, y[g]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(y[g][e]));
+    }
+  }
+  amax = block_max<kWaves>(amax, red);
+  const float scale = fmaxf(amax / LFM2_E4M3_MAX, 1.0e-12f);
+  if (threadIdx.x == 0) scales[row] = scale;
+#pragma unroll
+  for (int g = 0; g < NG; ++g) {
+    const int64_t col = ((int64_t)g * kThreads + threadIdx.x) * 8;
+    if (col < H) store_e4m3<8>(q + row * H + col, y[g], scale);
+  }
+}
+
+extern "C" int lfm2_conv_update_fp8(uint8_t* q, float* scales, const void* bcx, const void* weight, void* state,
+                                    const uint8_t* active, const int32_t* slot_ids, int64_t M, int64_t H, int64_t slots,
+                                    int dtype, void* stream) {
+  LFM2_REQUIRE(M > 0 && H > 0 && slots > 0, "conv_update_fp8: empty shape");
+  LFM2_REQUIRE(slot_ids != nullptr || M <= slots, "conv_update_fp8: %ld rows but only %ld state slots", (long)M, (long)slots);
+  LFM2_REQUIRE(H % 8 == 0 && H <= 2 * 8 * kThreads, "conv_update_fp8: width %ld is not a multiple of 8 or above %d", (long)H, 2 * 8 * kThreads);
+  hipStream_t s = (hipStream_t)stream;
+#define CU_(TT, NGG) hipLaunchKernelGGL((conv_update_fp8_kernel<TT, NGG>), dim3(M), dim3(kThreads), 0, s, q, scales, \
+                                        (const TT*)bcx, (const TT*)weight, (TT*)state, active, slot_ids, H)
+  switch (dtype) {
+    case LFM2_DTYPE_BF16: if (H <= 8 * kThreads) CU_(__bf16, 1); else CU_(__bf16, 2); break;
+    case LFM2_DTYPE_F16: if (H <= 8 * kThreads) CU_(_Float16, 1); else CU_(_Float16, 2); break;
+    default: LFM2_FAIL(LFM2_ERR_UNSUPPORTED, "conv_update_fp8: dtype %d is not bf16/f16", dtype);
+  }
+#undef CU_
   LFM2_LAUNCH_CHECK();
 }
 
@@ -450,14 +588,149 @@ prepare_qkv_kernel(T* q, T* k, T* v, const T* x, const T* qw, const T* kw, const
   }
 }
 
+// One wave per (row, head) unit for the usual head sizes: units 0..QH-1 are query heads, QH..QH+KH-1 key heads (both
+// normalised and rotated), the rest value heads (copied).  A lane holds elements lane, lane+64, ...; the rotate-half
+// partner is the lane D/2 away (D <= 64) or another register of the same lane (D >= 128).  With STORE the key and
+// value heads go straight into the cache row of the token (model dtype, or e4m3 with one scale per token and head,
+// quantised from the value rounded to the model dtype exactly as a separate store of the rounded tensor would).
+struct PrepArgs {
+  void *q, *k, *v;
+  const void *x, *qw, *kw;
+  const float *cosT, *sinT;
+  const int32_t *positions, *slot_ids;
+  const uint8_t* active;
+  void *kc, *vc;
+  float *ks, *vs;
+  int64_t M, max_positions, c0, c1, c2;
+  int QH, KH;
+  float eps;
+};
+
+template <typename T, int D, int STORE>  // STORE 0: q, k, v tensors; 1: cache in the model dtype; 2: e4m3 cache
+__global__ void __launch_bounds__(kThreads) prepare_qkv_wave_kernel(PrepArgs a) {
+  constexpr int R = (D + 63) / 64, half = D / 2;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int U = a.QH + 2 * a.KH;
+  const int64_t unit = (int64_t)blockIdx.x * kWaves + wave;
+  if (unit >= a.M * U) return;
+  const int64_t row = unit / U;
+  const int u = (int)(unit % U);
+  const T* src = (const T*)a.x + row * U * D + (int64_t)u * D;
+  const bool on = D >= 64 || lane < D;
+  float val[R];
+#pragma unroll
+  for (int i = 0; i < R; ++i) val[i] = on ? Elem<T>::load(src[lane + 64 * i]) : 0.f;
+  if (u < a.QH + a.KH) {
+    const T* wgt = u < a.QH ? (const T*)a.qw : (const T*)a.kw;
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < R; ++i) ss += val[i] * val[i];
+    ss = wave_sum(ss);
+    const float rstd = 1.0f / sqrtf(ss / (float)D + a.eps);
+    int64_t pos = a.positions[row];
+    pos = pos < 0 ? 0 : (pos >= a.max_positions ? a.max_positions - 1 : pos);
+    float w[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      const float n = round_to<T>(val[i] * rstd);
+      w[i] = on ? round_to<T>(n * Elem<T>::load(wgt[lane + 64 * i])) : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      const int d = lane + 64 * i;
+      const int t = on ? d % half : 0;
+      const float c = round_to<T>(a.cosT[pos * half + t]);
+      const float sn = round_to<T>(a.sinT[pos * half + t]);
+      const float partner = D >= 128 ? w[i ^ (D / 128)] : __shfl_xor(w[i], half, 64);
+      const float left = round_to<T>(w[i] * c), right = round_to<T>(partner * sn);
+      val[i] = round_to<T>(d < half ? left - right : left + right);
+    }
+  }
+  if (u < a.QH) {
+    T* dst = (T*)a.q + (row * a.QH + u) * D;
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+      if (on) dst[lane + 64 * i] = Elem<T>::store(val[i]);
+    return;
+  }
+  const bool is_v = u >= a.QH + a.KH;
+  const int h = is_v ? u - a.QH - a.KH : u - a.QH;
+  if (STORE == 0) {
+    T* dst = (T*)(is_v ? a.v : a.k) + (row * a.KH + h) * D;
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+      if (on) dst[lane + 64 * i] = Elem<T>::store(val[i]);
+    return;
+  }
+  if (a.active && !a.active[row]) return;
+  const int64_t slot = a.slot_ids ? a.slot_ids[row] : row;
+  const int64_t at = a.positions[row];
+  if (slot < 0 || at < 0) return;
+  const int64_t dst = slot * a.c0 + at * a.c1 + (int64_t)h * a.c2;
+  if (STORE == 1) {
+    T* out = (T*)(is_v ? a.vc : a.kc) + dst;
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+      if (on) out[lane + 64 * i] = Elem<T>::store(val[i]);
+  } else {
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < R; ++i) amax = fmaxf(amax, fabsf(val[i]));
+    amax = wave_max(amax);
+    const float sc = fmaxf(amax / LFM2_E4M3_MAX, 1.0e-12f);
+    uint8_t* out = (uint8_t*)(is_v ? a.vc : a.kc) + dst;
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+      if (on) out[lane + 64 * i] = to_e4m3(val[i] / sc);
+    if (lane == 0) (is_v ? a.vs : a.ks)[dst / D] = sc;
+  }
+}
+
+template <typename T, int STORE>
+int launch_prepare(const PrepArgs& a, int D, hipStream_t s) {
+  const int64_t units = a.M * (a.QH + 2 * a.KH);
+  const dim3 grid(ceil_div(units, kWaves)), block(kThreads);
+  switch (D) {
+    case 32: hipLaunchKernelGGL((prepare_qkv_wave_kernel<T, 32, STORE>), grid, block, 0, s, a); break;
+    case 64: hipLaunchKernelGGL((prepare_qkv_wave_kernel<T, 64, STORE>), grid, block, 0, s, a); break;
+    case 128: hipLaunchKernelGGL((prepare_qkv_wave_kernel<T, 128, STORE>), grid, block, 0, s, a); break;
+    case 256: hipLaunchKernelGGL((prepare_qkv_wave_kernel<T, 256, STORE>), grid, block, 0, s, a); break;
+    default: return 1;
+  }
+  return 0;
+}
+
 extern "C" int lfm2_prepare_qkv(void* q, void* k, void* v, const void* x, const void* q_weight, const void* k_weight,
                                 const float* cos, const float* sin, const int32_t* positions, int64_t M, int QH, int KH,
                                 int D, int64_t max_positions, float eps, int dtype, void* stream) {
   LFM2_REQUIRE(M > 0 && QH > 0 && KH > 0, "prepare_qkv: empty shape");
   LFM2_REQUIRE(D > 0 && D <= 256 && D % 2 == 0, "prepare_qkv: head_dim %d not in (0,256] or odd", D);
   LFM2_REQUIRE(max_positions > 0, "prepare_qkv: empty rotary table");
+  if (D == 32 || D == 64 || D == 128 || D == 256) {
+    const PrepArgs a{q, k, v, x, q_weight, k_weight, cos, sin, positions, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
+                     M, max_positions, 0, 0, 0, QH, KH, eps};
+    DISPATCH_DTYPE(dtype, (launch_prepare<T, 0>(a, D, (hipStream_t)stream)));
+    LFM2_LAUNCH_CHECK();
+  }
   DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(prepare_qkv_kernel<T>, dim3(M), dim3(kThreads), 0, (hipStream_t)stream, (T*)q,
                                            (T*)k, (T*)v, (const T*)x, (const T*)q_weight, (const T*)k_weight, cos, sin,
                                            positions, QH, KH, D, max_positions, eps));
+  LFM2_LAUNCH_CHECK();
+}
+
+extern "C" int lfm2_prepare_qkv_store(void* q, const void* x, const void* q_weight, const void* k_weight, const float* cos,
+                                      const float* sin, const int32_t* positions, void* k_cache, void* v_cache,
+                                      float* k_scales, float* v_scales, const uint8_t* active, const int32_t* slot_ids,
+                                      int64_t M, int QH, int KH, int D, int64_t max_positions, float eps, int64_t c0,
+                                      int64_t c1, int64_t c2, int kv_fp8, int dtype, void* stream) {
+  LFM2_REQUIRE(M > 0 && QH > 0 && KH > 0, "prepare_qkv_store: empty shape");
+  LFM2_REQUIRE(D == 32 || D == 64 || D == 128 || D == 256, "prepare_qkv_store: head_dim %d not in {32,64,128,256}", D);
+  LFM2_REQUIRE(max_positions > 0, "prepare_qkv_store: empty rotary table");
+  LFM2_REQUIRE(k_cache && v_cache && positions, "prepare_qkv_store: caches and positions are required");
+  LFM2_REQUIRE(!kv_fp8 || (k_scales && v_scales), "prepare_qkv_store: e4m3 cache without scale tensors");
+  const PrepArgs a{q, nullptr, nullptr, x, q_weight, k_weight, cos, sin, positions, slot_ids, active, k_cache, v_cache,
+                   k_scales, v_scales, M, max_positions, c0, c1, c2, QH, KH, eps};
+  if (kv_fp8) { DISPATCH_DTYPE(dtype, (launch_prepare<T, 2>(a, D, (hipStream_t)stream))); }
+  else { DISPATCH_DTYPE(dtype, (launch_prepare<T, 1>(a, D, (hipStream_t)stream))); }
   LFM2_LAUNCH_CHECK();
 }

@@ -294,22 +294,23 @@ Plan default_plan(int64_t M, int64_t N, int64_t Kb) {
 
 template <int EB, int BM, int BN, int WM, int WN>
 void launch_tile(void* out, float* partial, const uint8_t* A, const uint8_t* W, const float* as, const float* ws, int M,
-                 int N, int64_t Kb, int splits, int out_dtype, hipStream_t s) {
+                 int N, int64_t Kb, int splits, int out_dtype, bool keep_partials, hipStream_t s) {
   const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   const int64_t steps = (Kb + kStepBytes - 1) / kStepBytes;
   const int per = (int)((steps + splits - 1) / splits);
   const dim3 grid((tiles + 7) / 8 * 8, splits), block(WM * WN * 64);
   if (Kb % kStepBytes == 0)
-    hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN, false>), grid, block, 0, s, out, splits > 1 ? partial : nullptr, A, W,
+    hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN, false>), grid, block, 0, s, out, (splits > 1 || keep_partials) ? partial : nullptr, A, W,
                        as, ws, M, N, Kb, per, out_dtype);
   else
-    hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN, true>), grid, block, 0, s, out, splits > 1 ? partial : nullptr, A, W,
+    hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN, true>), grid, block, 0, s, out, (splits > 1 || keep_partials) ? partial : nullptr, A, W,
                        as, ws, M, N, Kb, per, out_dtype);
 }
 
 template <int EB>
 int gemm_entry(const char* name, void* out, const void* a, const float* as, const void* w, const float* ws,
-               float* workspace, int64_t M, int64_t N, int64_t K, int out_dtype, int tile, int split_k, void* stream) {
+               float* workspace, int64_t M, int64_t N, int64_t K, int out_dtype, int tile, int split_k, void* stream,
+               bool reduce = true) {
   LFM2_REQUIRE(M > 0 && N > 0 && K > 0, "%s: empty shape", name);
   LFM2_REQUIRE(M < (1 << 30) && N < (1 << 30), "%s: M or N too large", name);
   LFM2_REQUIRE(out_dtype >= LFM2_DTYPE_BF16 && out_dtype <= LFM2_DTYPE_F32, "%s: bad output dtype", name);
@@ -317,6 +318,7 @@ int gemm_entry(const char* name, void* out, const void* a, const float* as, cons
   const uint8_t *A = (const uint8_t*)a, *W = (const uint8_t*)w;
   const int64_t Kb = K * EB;
   if (Kb % 16 != 0 || ((uintptr_t)a | (uintptr_t)w) % 16 != 0) {
+    LFM2_REQUIRE(reduce, "%s: partial products need K bytes and pointers aligned to 16", name);
     hipLaunchKernelGGL(gemm_naive_kernel<EB>, dim3(ceil_div(M * N, 256)), dim3(256), 0, s, out, A, W, as, ws, M, N, K, out_dtype);
     LFM2_LAUNCH_CHECK();
   }
@@ -331,8 +333,9 @@ int gemm_entry(const char* name, void* out, const void* a, const float* as, cons
   // every split must own at least one step
   while (plan.splits > 1 && (steps + plan.splits - 1) / plan.splits * (plan.splits - 1) >= steps) --plan.splits;
   LFM2_REQUIRE(plan.splits == 1 || workspace != nullptr, "%s: split-K needs a workspace", name);
+  LFM2_REQUIRE(reduce || workspace != nullptr, "%s: partial products need a destination", name);
 #define TILE_(ID, BM, BN, WM, WN) \
-  case ID: launch_tile<EB, BM, BN, WM, WN>(out, workspace, A, W, as, ws, (int)M, (int)N, Kb, plan.splits, out_dtype, s); break
+  case ID: launch_tile<EB, BM, BN, WM, WN>(out, workspace, A, W, as, ws, (int)M, (int)N, Kb, plan.splits, out_dtype, !reduce, s); break
   switch (plan.tile) {
     TILE_(0, 16, 64, 1, 4);
     TILE_(1, 32, 64, 2, 2);
@@ -345,7 +348,7 @@ int gemm_entry(const char* name, void* out, const void* a, const float* as, cons
     TILE_(8, 128, 64, 4, 2);
   }
 #undef TILE_
-  if (plan.splits > 1)
+  if (plan.splits > 1 && reduce)
     hipLaunchKernelGGL(reduce_split_kernel, dim3(ceil_div(M * N, 256)), dim3(256), 0, s, out, workspace, as, ws, M, N,
                        plan.splits, out_dtype);
   LFM2_LAUNCH_CHECK();
@@ -359,6 +362,20 @@ extern "C" int lfm2_fp8_gemm(void* out, const uint8_t* a_q, const float* a_scale
   LFM2_REQUIRE(a_scales && w_scales, "fp8_gemm: scales are required");
   LFM2_REQUIRE(split_k <= 16, "fp8_gemm: split_k above 16");
   return gemm_entry<1>("fp8_gemm", out, a_q, a_scales, w_q, w_scales, workspace, M, N, K, out_dtype, tile, split_k, stream);
+}
+
+extern "C" int lfm2_fp8_gemm_partials(float* partials, const uint8_t* a_q, const uint8_t* w_q, int64_t M, int64_t N,
+                                      int64_t K, int tile, int split_k, void* stream) {
+  LFM2_REQUIRE(split_k >= 1 && split_k <= 16, "fp8_gemm_partials: split_k %d not in [1,16]", split_k);
+  const int64_t steps = (K + kStepBytes - 1) / kStepBytes;
+  LFM2_REQUIRE(split_k <= steps && (steps + split_k - 1) / split_k * (split_k - 1) < steps,
+               "fp8_gemm_partials: %d splits leave one without a K step", split_k);
+  return gemm_entry<1>("fp8_gemm_partials", nullptr, a_q, nullptr, w_q, nullptr, partials, M, N, K, LFM2_DTYPE_F32, tile,
+                       split_k, stream, false);
+}
+
+extern "C" int64_t lfm2_fp8_gemm_default_splits(int64_t M, int64_t N, int64_t K) {
+  return K % 16 == 0 ? default_plan(M, N, K).splits : 1;
 }
 
 extern "C" int64_t lfm2_fp8_gemm_workspace(int64_t M, int64_t N, int64_t K) {

@@ -227,16 +227,22 @@ class LFM25Engine:
         if packed is not None:
             q, scales, residual = ops.rms_norm_fp8(x, norm_weight, self.config.norm_eps, residual)
             return packed.linear_quantized(q, scales, dtype=self.dtype), residual
+        if isinstance(x, ops.SplitProduct):
+            x = x.materialize()
         normed, residual = ops.rms_norm(x, norm_weight, self.config.norm_eps, residual)
         return ops.linear(normed, weight), residual
 
     def _linear(self, x, weight, fp8):
+        """Out projection of an operator; `x` is a tensor or, from a fused producer, (e4m3 rows, scales)."""
         packed = fp8.get(id(weight))
+        if isinstance(x, tuple):
+            return packed.linear_quantized(x[0], x[1], dtype=self.dtype)
         return packed.linear(x) if packed is not None else ops.linear(x, weight)
 
-    def _backbone(self, tokens, attention_op, conv_op, fp8):
+    def _backbone(self, tokens, attention_op, conv_op, fp8, *, defer_reduce=False):
         """Embedding and all layers with the fused residual chain of lfm25_cuda.py:134-184: every RMSNorm also adds
-        the previous block's output into the running residual.  Returns (last MLP output, residual)."""
+        the previous block's output into the running residual.  Returns (last MLP output, residual).  With
+        `defer_reduce` (decode) a split-K down projection hands its partial sums to the next norm."""
         hidden = ops.embedding(tokens, self.weights.embed_tokens)
         residual = None
         for layer in self.weights.layers:
@@ -252,7 +258,7 @@ class LFM25Engine:
             down = fp8.get(id(layer.w2_weight))
             if down is not None:
                 q, scales = ops.swiglu_fp8(gate_up)
-                hidden = down.linear_quantized(q, scales, dtype=self.dtype)
+                hidden = down.linear_quantized(q, scales, dtype=self.dtype, defer_reduce=defer_reduce)
             else:
                 hidden = ops.linear(ops.swiglu(gate_up), layer.w2_weight)
         return hidden, residual
@@ -273,22 +279,28 @@ class LFM25Engine:
         schedule = ops.decode_schedule(positions, active, slot_ids, capacity=cache.max_seq_len) if cache.fp8 else None
 
         def attention_op(op, qkv):
-            q, k, v = ops.prepare_qkv(qkv, op.q_norm_weight, op.k_norm_weight, self._rope_cos, self._rope_sin, positions,
-                                      cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim, cfg.norm_eps)
+            # QK norm + RoPE with the new token's keys and values written straight into the cache, then attention over
+            # [0, position]; rows come back already quantised when the out projection is W8A8
             i = op.cache_index
-            if cache.fp8:
-                out = ops.decode(q, k, v, cache.k_cache[i], cache.v_cache[i], cache.k_scales[i], cache.v_scales[i], positions,
-                                 active=active, scale=self._scaling, slot_ids=slot_ids, schedule=schedule)
-            else:
-                ops.append_bf16_kv(k, v, cache.k_cache[i], cache.v_cache[i], positions, slot_ids, active)
-                out = ops.attend(q, cache.k_cache[i], cache.v_cache[i], None, None, positions, active=active,
-                                 scale=self._scaling, slot_ids=slot_ids)
-            return out.view(rows, -1)
+            k_scales = cache.k_scales[i] if cache.fp8 else None
+            v_scales = cache.v_scales[i] if cache.fp8 else None
+            q = ops.prepare_qkv_store(qkv, op.q_norm_weight, op.k_norm_weight, self._rope_cos, self._rope_sin, positions,
+                                      cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim, cfg.norm_eps,
+                                      cache.k_cache[i], cache.v_cache[i], k_scales, v_scales, active=active,
+                                      slot_ids=slot_ids)
+            quantized = (id(op.out_weight) in fp8
+                         and -(-cfg.num_attention_heads // 16) * -(-cfg.head_dim // 64) <= 4)  # the fused combine's row limit
+            out = ops.attend(q, cache.k_cache[i], cache.v_cache[i], k_scales, v_scales, positions, active=active,
+                             scale=self._scaling, slot_ids=slot_ids, schedule=schedule, quantized=quantized)
+            return out if quantized else out.view(rows, -1)
 
         def conv_op(op, bcx):
-            return ops.conv_update(bcx, op.conv_weight, cache.conv_state[op.cache_index], active, slot_ids)
+            state = cache.conv_state[op.cache_index]
+            if id(op.out_weight) in fp8 and op.conv_weight.size(0) <= 4096 and op.conv_weight.size(0) % 8 == 0:
+                return ops.conv_update_fp8(bcx, op.conv_weight, state, active, slot_ids)
+            return ops.conv_update(bcx, op.conv_weight, state, active, slot_ids)
 
-        hidden, residual = self._backbone(tokens, attention_op, conv_op, fp8)
+        hidden, residual = self._backbone(tokens, attention_op, conv_op, fp8, defer_reduce=True)
         logits = self._head(hidden, residual, fp8)
         ops.advance_positions(cache.seq_lens, positions, slot_ids, active)
         return logits

@@ -59,8 +59,40 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: torch.
     return out, summed
 
 
+@dataclass
+class SplitProduct:
+    """An FP8 projection left as split-K partial sums (`PackedFP8Weight.linear_quantized(..., defer_reduce=True)`):
+    the value is round((sum of partials) * a_scales[m] * w_scales[n]) in `dtype`.  `rms_norm_fp8` folds that reduction
+    into its own pass; `materialize()` gives the ordinary tensor."""
+    partials: torch.Tensor   # [splits, M, N] fp32
+    a_scales: torch.Tensor
+    w_scales: torch.Tensor
+    dtype: torch.dtype
+
+    @property
+    def shape(self):
+        return self.partials.shape[1:]
+
+    def materialize(self) -> torch.Tensor:
+        total = self.partials[0].clone()
+        for part in self.partials[1:]:
+            total += part
+        return ((total * self.a_scales[:, None]) * self.w_scales[None, :]).to(self.dtype)
+
+
 def rms_norm_fp8(x, weight, eps, residual=None):
-    """lfm25_fp8.py:57-64: (e4m3 rows, per-row scales, x+residual)."""
+    """lfm25_fp8.py:57-64: (e4m3 rows, per-row scales, x+residual).  `x` may be a `SplitProduct`."""
+    if isinstance(x, SplitProduct):
+        _check(weight, residual)
+        rows, width = x.shape
+        q = torch.empty((rows, width), device=weight.device, dtype=FP8)
+        scales = torch.empty(rows, device=weight.device, dtype=torch.float32)
+        if residual is None:
+            raise ValueError("a deferred projection can only feed a norm that adds a residual")
+        summed = torch.empty((rows, width), device=weight.device, dtype=x.dtype)
+        call("lfm2_rms_norm_fp8_split", q, scales, summed, x.partials, x.partials.size(0), x.a_scales, x.w_scales, weight,
+             residual, rows, width, float(eps), _code(x.dtype))
+        return q, scales, summed
     _check(x, weight, residual)
     q = torch.empty(x.shape, device=x.device, dtype=FP8)
     scales = torch.empty(_rows(x), device=x.device, dtype=torch.float32)
@@ -110,6 +142,35 @@ def conv_update(bcx, weight, state, active=None, slot_ids=None):
     call("lfm2_conv_update", out, bcx, weight, state, active, slot_ids, bcx.size(0), width, state.size(0),
          _code(bcx.dtype))
     return out
+
+
+def conv_update_fp8(bcx, weight, state, active=None, slot_ids=None):
+    """`conv_update` followed by `quantize_rows` of its output (lfm25_cuda.py:146-149 in front of an FP8 out
+    projection) as one launch; returns (e4m3 rows, per-row scales)."""
+    _check(bcx, weight, state, active, slot_ids)
+    width = weight.size(0)
+    q = torch.empty((bcx.size(0), width), device=bcx.device, dtype=FP8)
+    scales = torch.empty(bcx.size(0), device=bcx.device, dtype=torch.float32)
+    call("lfm2_conv_update_fp8", q, scales, bcx, weight, state, active, slot_ids, bcx.size(0), width, state.size(0),
+         _code(bcx.dtype))
+    return q, scales
+
+
+def prepare_qkv_store(x, q_weight, k_weight, cos, sin, positions, q_heads: int, kv_heads: int, head_dim: int, eps: float,
+                      k_cache, v_cache, k_scales=None, v_scales=None, *, active=None, slot_ids=None):
+    """`prepare_qkv` (lfm25_cuda_kernels.py:143-151) fused with the decode-step KV append (`store_kv` of
+    lfm25_fp8_kv.py:58-69 when scale tensors are given, `append_bf16_kv` of lfm25_batching.py:66-69 otherwise):
+    returns q [M,1,QH,D]; keys and values go straight into the cache views at `positions`."""
+    _check(x, q_weight, k_weight, cos, sin, positions, active, slot_ids)
+    if positions.dtype != torch.int32:
+        raise ValueError("positions must be int32")
+    m = x.size(0)
+    q = torch.empty((m, 1, q_heads, head_dim), device=x.device, dtype=x.dtype)
+    c0, c1, c2 = _cache_strides(k_cache)
+    call("lfm2_prepare_qkv_store", q, x, q_weight, k_weight, cos, sin, positions, k_cache, v_cache, k_scales, v_scales,
+         active, slot_ids, m, q_heads, kv_heads, head_dim, cos.size(0), float(eps), c0, c1, c2,
+         int(k_scales is not None), _code(x.dtype))
+    return q
 
 
 def prepare_qkv(x, q_weight, k_weight, cos, sin, positions, q_heads: int, kv_heads: int, head_dim: int, eps: float):
@@ -175,13 +236,20 @@ class PackedFP8Weight:
         values, scales = quantize_rows(x)
         return self.linear_quantized(values, scales, dtype=x.dtype, config=config)
 
-    def linear_quantized(self, x, scales, *, dtype=torch.bfloat16, config=None):
-        """config = (tile index, split_k) overrides the default tile choice."""
+    def linear_quantized(self, x, scales, *, dtype=torch.bfloat16, config=None, defer_reduce=False):
+        """config = (tile index, split_k) overrides the default tile choice.  With `defer_reduce`, a product the
+        default plan splits along K comes back as a `SplitProduct` for `rms_norm_fp8` to reduce."""
         batch, width = x.shape
         rows = self.values.size(0)
         if width != self.values.size(1):
             raise ValueError("FP8 activation and weight widths differ")
         tile, split_k = (-1, 0) if config is None else (int(config[0]), int(config[1]) if len(config) > 1 else 0)
+        if defer_reduce and config is None:
+            splits = query("lfm2_fp8_gemm_default_splits", batch, rows, width)
+            if splits > 1:
+                partials = torch.empty((splits, batch, rows), device=x.device, dtype=torch.float32)
+                call("lfm2_fp8_gemm_partials", partials, x, self.values, batch, rows, width, -1, splits)
+                return SplitProduct(partials, scales, self.scales, dtype)
         out = torch.empty((batch, rows), device=x.device, dtype=dtype)
         need = query("lfm2_fp8_gemm_workspace", batch, rows, width) if split_k == 0 else max(split_k, 1) * batch * rows
         ws = torch.empty(need, device=x.device, dtype=torch.float32) if need and split_k != 1 else None
@@ -234,7 +302,7 @@ def decode_schedule(positions, active=None, slot_ids=None, *, capacity: int):
 
 
 def attend(q, k_cache, v_cache, k_scales, v_scales, positions, *, active=None, scale=None, config=None,
-           slot_ids=None, window=0, block_table=None, page=16, schedule=None):
+           slot_ids=None, window=0, block_table=None, page=16, schedule=None, quantized=False):
     """lfm25_fp8_kv.py:138-167 (e4m3 history + scales) and flash_attn_with_kvcache of lfm25_cuda.py:156-165
     (`k_scales is None`: history in the model dtype).  Attends over positions [0, positions[b]]; inactive rows
     return zeros.  With `block_table` the caches are page pools [pages, page, KV heads, dim]."""
@@ -245,14 +313,19 @@ def attend(q, k_cache, v_cache, k_scales, v_scales, positions, *, active=None, s
     heads = k_cache.size(2)
     c0, c1, c2 = _cache_strides(k_cache)
     capacity = k_cache.size(1) if block_table is None else block_table.size(1) * page
-    out = torch.empty_like(q)
     ws = torch.empty(query("lfm2_decode_attention_workspace", batch, query_heads, dim, capacity),
                      device=q.device, dtype=torch.float32)
+    if quantized:  # rows come back as (e4m3 [B, QH*D], per-row scales), ready for an FP8 out projection
+        out = None
+        out_q = torch.empty((batch, query_heads * dim), device=q.device, dtype=FP8)
+        out_scales = torch.empty(batch, device=q.device, dtype=torch.float32)
+    else:
+        out, out_q, out_scales = torch.empty_like(q), None, None
     call("lfm2_decode_attention", out, q, k_cache, v_cache, k_scales, v_scales, positions, active, slot_ids,
          block_table, 0 if block_table is None else block_table.size(1), page, schedule, ws, batch, query_heads, heads, dim,
          capacity, c0, c1, c2, float(scale if scale is not None else dim ** -0.5), int(k_scales is not None),
-         _code(q.dtype))
-    return out
+         _code(q.dtype), out_q, out_scales)
+    return (out_q, out_scales) if quantized else out
 
 
 def decode(q, k, v, k_cache, v_cache, k_scales, v_scales, positions, *, active=None, scale=None, slot_ids=None, window=0,

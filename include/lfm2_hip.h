@@ -43,6 +43,14 @@ int lfm2_rms_norm(void* out, void* summed, const void* x, const void* weight, co
 int lfm2_rms_norm_fp8(uint8_t* q, float* scales, void* summed, const void* x, const void* weight,
                       const void* residual, int64_t M, int64_t H, float eps, int dtype, void* stream);
 
+/* rms_norm_fp8 whose input x[M,H] is given as split-K partial products of an FP8 projection:
+ * x = round((sum_s partial[s]) * a_scales[m] * w_scales[h]) in the model dtype, i.e. what lfm2_fp8_gemm would have
+ * stored; then exactly lfm2_rms_norm_fp8.  Fuses the projection's reduce pass into the norm that follows it in
+ * lfm25_cuda.py:166-184. */
+int lfm2_rms_norm_fp8_split(uint8_t* q, float* scales, void* summed, const float* partial, int splits,
+                            const float* a_scales, const float* w_scales, const void* weight, const void* residual,
+                            int64_t M, int64_t H, float eps, int dtype, void* stream);
+
 /* swiglu of lfm25_cuda_kernels.py:58-72.  x [M,2I] (gate first) -> out [M,I]. */
 int lfm2_swiglu(void* out, const void* x, int64_t M, int64_t I, int dtype, void* stream);
 
@@ -58,11 +66,29 @@ int lfm2_quantize_rows(uint8_t* q, float* scales, const void* x, int64_t M, int6
 int lfm2_conv_update(void* out, const void* bcx, const void* weight, void* state, const uint8_t* active,
                      const int32_t* slot_ids, int64_t M, int64_t H, int64_t slots, int dtype, void* stream);
 
+/* conv_update followed by quantize_rows of its output (lfm25_cuda.py:146-149 with an FP8 out projection) in one
+ * launch: q uint8[M,H], scales float[M]; the values quantised are the model-dtype roundings lfm2_conv_update
+ * stores.  H <= 4096. */
+int lfm2_conv_update_fp8(uint8_t* q, float* scales, const void* bcx, const void* weight, void* state,
+                         const uint8_t* active, const int32_t* slot_ids, int64_t M, int64_t H, int64_t slots,
+                         int dtype, void* stream);
+
 /* prepare_qkv of lfm25_cuda_kernels.py:113-151.  x [M,(QH+2KH)*D]; cos/sin float[P,D/2];
  * positions int32[M] -> q [M,QH,D], k [M,KH,D], v [M,KH,D]. */
 int lfm2_prepare_qkv(void* q, void* k, void* v, const void* x, const void* q_weight, const void* k_weight,
                      const float* cos, const float* sin, const int32_t* positions, int64_t M, int QH, int KH,
                      int D, int64_t max_positions, float eps, int dtype, void* stream);
+
+/* prepare_qkv followed by the decode-step KV append (store_kv of lfm25_fp8_kv.py:58-94 when kv_fp8, append_bf16_kv of
+ * lfm25_adaptive.py:66 otherwise) in one launch: q [M,QH,D] is returned, the rotated keys and the values of row m go
+ * to cache position positions[m] of slot slot_ids[m] (or m) unless the row is inactive, its slot id negative or its
+ * position negative.  Caches are addressed as slot*c0 + position*c1 + head*c2 (elements); e4m3 scales sit at that
+ * address divided by D.  D in {32,64,128,256}. */
+int lfm2_prepare_qkv_store(void* q, const void* x, const void* q_weight, const void* k_weight, const float* cos,
+                           const float* sin, const int32_t* positions, void* k_cache, void* v_cache, float* k_scales,
+                           float* v_scales, const uint8_t* active, const int32_t* slot_ids, int64_t M, int QH, int KH,
+                           int D, int64_t max_positions, float eps, int64_t c0, int64_t c1, int64_t c2, int kv_fp8,
+                           int dtype, void* stream);
 
 /* Packed-prefill short conv (F.conv1d path of lfm25_engine.py:1478-1511 on a varlen batch).
  * bcx [T,3H]; seq_of_token/pos_of_token int32[T]; seq_start int32[nseq+1] (cu_seqlens);
@@ -81,6 +107,13 @@ int lfm2_conv_prefill(void* out, void* state, const void* bcx, const void* weigh
 int lfm2_fp8_gemm(void* out, const uint8_t* a_q, const float* a_scales, const uint8_t* w_q,
                   const float* w_scales, float* workspace, int64_t M, int64_t N, int64_t K, int out_dtype,
                   int tile, int split_k, void* stream);
+/* The same product left as split-K partial sums: partials float[split_k, M, N], unscaled (no activation or weight
+ * scale applied), split s covering its contiguous share of K.  For a consumer that folds the reduction into its own
+ * pass (lfm2_rms_norm_fp8_split).  No counterpart in the reference, which always materialises the projection. */
+int lfm2_fp8_gemm_partials(float* partials, const uint8_t* a_q, const uint8_t* w_q, int64_t M, int64_t N, int64_t K,
+                           int tile, int split_k, void* stream);
+/* Split count lfm2_fp8_gemm would choose for a shape (1 = no split). */
+int64_t lfm2_fp8_gemm_default_splits(int64_t M, int64_t N, int64_t K);
 /* Workspace floats lfm2_fp8_gemm needs for a shape under its default choice (0 = none). */
 int64_t lfm2_fp8_gemm_workspace(int64_t M, int64_t N, int64_t K);
 
@@ -120,12 +153,15 @@ int lfm2_store_kv_packed(const void* k, const void* v, void* k_cache, void* v_ca
  * inactive rows produce zeros.  block_table int32[B,max_blocks] or NULL: when given, token t of
  * row b lives in page block_table[b*max_blocks + t/page] at in-page index t%page and c0 is the
  * page stride (slot-mapped paged layout).  workspace: lfm2_decode_attention_workspace() floats (4-byte words). */
+/* (out_q uint8[B,QH*D] with out_scales float[B], both or neither: when given, the rows are stored per-row e4m3
+ * quantised, as lfm2_quantize_rows of the model-dtype result would, and `out` is not written.) */
 int lfm2_decode_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
                           const float* k_scales, const float* v_scales, const int32_t* positions,
                           const uint8_t* active, const int32_t* slot_ids, const int32_t* block_table,
                           int64_t max_blocks, int page, const int32_t* schedule, float* workspace, int64_t B,
                           int QH, int KH, int D, int64_t capacity, int64_t c0, int64_t c1, int64_t c2, float scale,
-                          int kv_fp8, int dtype, void* stream);
+                          int kv_fp8, int dtype, uint8_t* out_q, float* out_scales,
+                          void* stream);
 int64_t lfm2_decode_attention_workspace(int64_t B, int QH, int D, int64_t capacity);
 
 /* Work list of the persistent decode-attention kernel: one (row, 1024-token chunk) item per chunk of every active

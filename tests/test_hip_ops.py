@@ -514,3 +514,114 @@ def test_behavior_head_reuses_the_sampler_normaliser(ops):
     torch.testing.assert_close(probs, want, atol=5e-6, rtol=1e-5)
     with pytest.raises(ValueError):
         ops.behavior_topk(logits, tok, lp, 129)
+
+
+# ------------------------------------------------------------------------------------------------ fused decode launches
+@pytest.mark.parametrize("dim,qh,kh", [(64, 32, 8), (32, 4, 4), (128, 4, 2), (256, 2, 1)])
+@pytest.mark.parametrize("fp8", [True, False])
+@torch.inference_mode()
+def test_prepare_qkv_with_cache_append_equals_the_two_separate_launches(ops, dim, qh, kh, fp8):
+    """One launch (QK norm + RoPE + KV append) against prepare_qkv followed by store_kv / append_bf16_kv, which the
+    tests above pin to the oracle: q, cache bytes and scales must be identical, untouched cache rows stay untouched."""
+    torch.manual_seed(5)
+    rows, slots, cap = 7, 9, 40
+    x = torch.randn(rows, (qh + 2 * kh) * dim, dtype=torch.bfloat16, device=DEV)
+    qw, kw = (torch.randn(dim, dtype=torch.bfloat16, device=DEV) for _ in range(2))
+    cos, sin = (t.to(DEV) for t in O.rope_tables(dim, 1e6, 64))
+    positions = torch.tensor([0, 5, 39, 17, 3, 8, 21], dtype=torch.int32, device=DEV)
+    slot_ids = torch.tensor([4, 0, 8, -1, 2, 6, 1], dtype=torch.int32, device=DEV)
+    active = torch.tensor([1, 1, 1, 0, 0, 1, 1], dtype=torch.bool, device=DEV)
+
+    def caches():
+        torch.manual_seed(6)
+        if fp8:
+            kc = torch.randint(0, 255, (slots, kh, cap, dim), dtype=torch.uint8, device=DEV).view(torch.float8_e4m3fn)
+            vc = torch.randint(0, 255, (slots, kh, cap, dim), dtype=torch.uint8, device=DEV).view(torch.float8_e4m3fn)
+            ks, vs = (torch.rand(slots, kh, cap, device=DEV) for _ in range(2))
+            return kc.transpose(1, 2), vc.transpose(1, 2), ks.transpose(1, 2), vs.transpose(1, 2)
+        kc, vc = (torch.randn(slots, cap, kh, dim, dtype=torch.bfloat16, device=DEV) for _ in range(2))
+        return kc, vc, None, None
+
+    kc0, vc0, ks0, vs0 = caches()
+    q0, k0, v0 = ops.prepare_qkv(x, qw, kw, cos, sin, positions, qh, kh, dim, 1e-5)
+    if fp8:
+        ops.store_kv(k0, v0, kc0, vc0, ks0, vs0, positions=positions, active=active, slot_ids=slot_ids)
+    else:
+        ops.append_bf16_kv(k0, v0, kc0, vc0, positions, slot_ids, active)
+    kc1, vc1, ks1, vs1 = caches()
+    q1 = ops.prepare_qkv_store(x, qw, kw, cos, sin, positions, qh, kh, dim, 1e-5, kc1, vc1, ks1, vs1, active=active,
+                               slot_ids=slot_ids)
+    torch.cuda.synchronize()
+    assert torch.equal(q0, q1)
+    as_bytes = (lambda t: t.contiguous().view(torch.uint8)) if fp8 else (lambda t: t.contiguous().view(torch.int16))
+    assert torch.equal(as_bytes(kc0), as_bytes(kc1)) and torch.equal(as_bytes(vc0), as_bytes(vc1))
+    if fp8:
+        assert torch.equal(ks0, ks1) and torch.equal(vs0, vs1)
+
+
+@pytest.mark.parametrize("width", (256, 2048, 4096))
+@torch.inference_mode()
+def test_conv_update_with_quantised_output_equals_the_two_separate_launches(ops, width):
+    torch.manual_seed(11)
+    rows, slots = 6, 8
+    bcx = torch.randn(rows, 3 * width, dtype=torch.bfloat16, device=DEV)
+    weight = torch.randn(width, 3, dtype=torch.bfloat16, device=DEV)
+    state = torch.randn(slots, width, 3, dtype=torch.bfloat16, device=DEV)
+    slot_ids = torch.tensor([3, 0, 7, 5, 1, 2], dtype=torch.int32, device=DEV)
+    active = torch.tensor([1, 0, 1, 1, 0, 1], dtype=torch.bool, device=DEV)
+    s0, s1 = state.clone(), state.clone()
+    expected = ops.quantize_rows(ops.conv_update(bcx, weight, s0, active, slot_ids))
+    q, scales = ops.conv_update_fp8(bcx, weight, s1, active, slot_ids)
+    torch.cuda.synchronize()
+    assert torch.equal(q.view(torch.uint8), expected[0].view(torch.uint8))
+    assert torch.equal(scales, expected[1])
+    assert torch.equal(s0.view(torch.int16), s1.view(torch.int16))
+
+
+@pytest.mark.parametrize("dim,qh,kh", [(64, 32, 8), (128, 4, 2), (32, 4, 4)])
+@pytest.mark.parametrize("fp8", [True, False])
+@torch.inference_mode()
+def test_decode_attention_with_quantised_rows_equals_quantising_its_output(ops, dim, qh, kh, fp8):
+    torch.manual_seed(23)
+    rows, cap = 5, 1300
+    q = torch.randn(rows, 1, qh, dim, dtype=torch.bfloat16, device=DEV)
+    if fp8:
+        kc = torch.randint(0, 120, (rows, kh, cap, dim), dtype=torch.uint8, device=DEV).view(torch.float8_e4m3fn).transpose(1, 2)
+        vc = torch.randint(0, 120, (rows, kh, cap, dim), dtype=torch.uint8, device=DEV).view(torch.float8_e4m3fn).transpose(1, 2)
+        ks, vs = (torch.rand(rows, kh, cap, device=DEV).transpose(1, 2) * 0.05 for _ in range(2))
+    else:
+        kc, vc = (torch.randn(rows, cap, kh, dim, dtype=torch.bfloat16, device=DEV) for _ in range(2))
+        ks = vs = None
+    positions = torch.tensor([0, 1299, 511, 1024, 77], dtype=torch.int32, device=DEV)
+    active = torch.tensor([1, 1, 0, 1, 1], dtype=torch.bool, device=DEV)
+    plain = ops.attend(q, kc, vc, ks, vs, positions, active=active)
+    expected = ops.quantize_rows(plain.view(rows, -1))
+    got = ops.attend(q, kc, vc, ks, vs, positions, active=active, quantized=True)
+    torch.cuda.synchronize()
+    assert torch.equal(got[0].view(torch.uint8), expected[0].view(torch.uint8))
+    assert torch.equal(got[1], expected[1])
+
+
+@torch.inference_mode()
+def test_split_k_partials_reduce_inside_the_following_norm(ops):
+    """A down projection left as split-K partial sums and reduced by the norm that follows it gives the bytes the
+    materialised projection followed by rms_norm_fp8 gives (lfm25_cuda.py:166-184 order of roundings)."""
+    torch.manual_seed(29)
+    rows, width, outputs = 256, 5632, 2048
+    act = torch.randn(rows, width, dtype=torch.bfloat16, device=DEV)
+    weight = ops.PackedFP8Weight.from_weight(torch.randn(outputs, width, dtype=torch.bfloat16, device=DEV) * 0.02)
+    norm_w = torch.randn(outputs, dtype=torch.bfloat16, device=DEV)
+    residual = torch.randn(rows, outputs, dtype=torch.bfloat16, device=DEV)
+    xq, xs = ops.quantize_rows(act)
+    deferred = weight.linear_quantized(xq, xs, defer_reduce=True)
+    assert isinstance(deferred, ops.SplitProduct) and deferred.partials.size(0) > 1
+    whole = weight.linear_quantized(xq, xs)
+    assert torch.equal(deferred.materialize().view(torch.int16), whole.view(torch.int16))
+    expected = ops.rms_norm_fp8(whole, norm_w, 1e-5, residual)
+    got = ops.rms_norm_fp8(deferred, norm_w, 1e-5, residual)
+    torch.cuda.synchronize()
+    assert torch.equal(got[0].view(torch.uint8), expected[0].view(torch.uint8))
+    assert torch.equal(got[1], expected[1])
+    assert torch.equal(got[2].view(torch.int16), expected[2].view(torch.int16))
+    small = weight.linear_quantized(xq[:8].contiguous(), xs[:8].contiguous(), defer_reduce=True)
+    assert isinstance(small, torch.Tensor)  # nothing to defer when the plan does not split
