@@ -292,11 +292,25 @@ __global__ void __launch_bounds__(256) decode_attn_mfma_kernel(DecodeArgs a) {
   __shared__ __bf16 lds_p[4][4][64];
   __shared__ float sm[4][4], sl[4][4], sacc[4][4][D];
   const int items = a.schedule[0] * a.KH;
+  // An item's row, chunk, length and slot sit behind three dependent loads; the next item's are fetched while the
+  // current one is processed so that chain is off the critical path of every item but a workgroup's first.
+  struct Meta { int b, chunk, len; int64_t slot; };
+  auto load_meta = [&](int item) {
+    const int pair = (item < items ? item : items - 1) / a.KH;
+    Meta mt;
+    mt.b = a.schedule[2 + 2 * pair];
+    mt.chunk = a.schedule[3 + 2 * pair];
+    mt.slot = a.slot_ids ? a.slot_ids[mt.b] : mt.b;
+    mt.len = a.positions[mt.b] + 1;
+    return mt;
+  };
+  Meta next_meta = load_meta(blockIdx.x);
   for (int item = blockIdx.x; item < items; item += gridDim.x) {
-  const int pair = item / a.KH, h = item % a.KH;
-  const int b = a.schedule[2 + 2 * pair], chunk = a.schedule[3 + 2 * pair];
-  const int64_t slot = a.slot_ids ? a.slot_ids[b] : b;
-  const int len = a.positions[b] + 1;
+  const Meta meta = next_meta;
+  next_meta = load_meta(item + gridDim.x);
+  const int h = item % a.KH;
+  const int b = meta.b, chunk = meta.chunk, len = meta.len;
+  const int64_t slot = meta.slot;
   const int start = chunk * kMfmaChunk;
 
   // A operand of S = Q.K^T: Q[head g][dims 4s..4s+3] for s = 0..15 (zero rows beyond the group)

@@ -31,9 +31,11 @@ __device__ __forceinline__ void philox(uint32_t c0, uint32_t c1, uint32_t c2, ui
   out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
 }
 // Standard Gumbel noise from a 32-bit word: u in [0,1) floored at 1e-30 (lfm25_sampling.py:21-27).
+// The two logarithms run on the hardware log2 unit (about 1 ulp): this is noise, and the full-precision library
+// routine made the sampler compute-bound (about a hundred instructions per logit).
 __device__ __forceinline__ float gumbel(uint32_t bits) {
   const float u = fmaxf((float)(bits >> 8) * (1.0f / 16777216.0f), 1.0e-30f);
-  return -logf(-logf(u));
+  return -__logf(-__logf(u));
 }
 __device__ __forceinline__ uint64_t row_key(int64_t seed, int64_t step) {
   return ((uint64_t)seed + (uint64_t)step * kGolden) & kMask63;
@@ -57,6 +59,9 @@ sample_partial_kernel(const T* logits, float* scratch, const int64_t* seeds, con
   float best = -INFINITY, tmax = -INFINITY;
   int best_i = 0x7fffffff;
   float vals[16];
+  const float inv_temp = 1.0f / fmaxf(temp, 1.0e-30f);
+  typedef T vec4 __attribute__((ext_vector_type(4)));
+  const bool vector_ok = (V & 3) == 0;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int64_t col0 = (int64_t)part * kTile + (i * 256 + threadIdx.x) * 4;
@@ -67,14 +72,23 @@ sample_partial_kernel(const T* logits, float* scratch, const int64_t* seeds, con
       philox((uint32_t)ctr, (uint32_t)(ctr >> 32), per_row ? 0u : (uint32_t)((row * V + col0) & 3), 0u, (uint32_t)key,
              (uint32_t)(key >> 32), rnd);
     }
+    float x4[4];
+    if (vector_ok && col0 < V) {
+      const vec4 v = *reinterpret_cast<const vec4*>(src + col0);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) x4[e] = Elem<T>::load(v[e]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) x4[e] = col0 + e < V ? Elem<T>::load(src[col0 + e]) : -INFINITY;
+    }
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int64_t col = col0 + e;
-      const float x = col < V ? Elem<T>::load(src[col]) : -INFINITY;
+      const float x = x4[e];
       vals[i * 4 + e] = x;
       tmax = fmaxf(tmax, x);
       float score = x;
-      if (temp > 0.f) score = x / fmaxf(temp, 1.0e-30f) + gumbel(rnd[e]);
+      if (temp > 0.f) score = x * inv_temp + gumbel(rnd[e]);
       if (col < V && (score > best || best_i == 0x7fffffff)) { best = score; best_i = (int)col; }
     }
   }
@@ -93,7 +107,7 @@ sample_partial_kernel(const T* logits, float* scratch, const int64_t* seeds, con
   const float shift = bmax == -INFINITY ? 0.f : bmax;
   float sum = 0.f;
 #pragma unroll
-  for (int i = 0; i < 16; ++i) sum += expf(vals[i] - shift);
+  for (int i = 0; i < 16; ++i) sum += __expf(vals[i] - shift);
   sum = wave_sum(sum);
   if (lane == 0) s_sum[wave] = sum;
   __syncthreads();
