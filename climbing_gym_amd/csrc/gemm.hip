@@ -21,7 +21,14 @@ namespace {
 constexpr int kStepBytes = 128;          // K bytes staged per step
 constexpr int kChunksPerRow = kStepBytes / 16;
 
-__device__ __forceinline__ int lds_slot(int row, int chunk) { return row * kChunksPerRow + (chunk ^ (row & 7)); }
+// Slot of a row's 16-byte chunk in a staged tile.  The XOR pattern is chosen per operand type from a sweep of
+// ds_read_b128 patterns on gfx950 (LDS reads peak at 256 B/clk): the e4m3 fragment read (16 rows x chunks 2g, 2g+1)
+// runs at 240 B/clk with row&7 ^ bit 3 of the row and at 128 B/clk with row&7 alone; the bf16 fragment read
+// (chunk g + 4*pass) is the other way round.  Staging writes (8 lanes per row) are indifferent (78 B/clk either way).
+template <int SW> __device__ __forceinline__ int lds_slot(int row, int chunk) {
+  const int x = SW == 1 ? ((row & 7) ^ ((row >> 3) & 1)) : (row & 7);
+  return row * kChunksPerRow + (chunk ^ x);
+}
 
 typedef int i32x8 __attribute__((ext_vector_type(8)));
 
@@ -33,8 +40,8 @@ template <> struct StepMfma<1> {
   // e4m3: lane group g owns chunks 2g, 2g+1 (32 bytes) -> one v_mfma_f32_16x16x128_f8f6f4 (unit scales)
   typedef i32x8 frag;
   static constexpr int PASSES = 1;
-  static __device__ __forceinline__ frag load(const i32x4* tile, int row, int lgrp, int) {
-    const i32x4 lo = tile[lds_slot(row, 2 * lgrp)], hi = tile[lds_slot(row, 2 * lgrp + 1)];
+  template <int SW> static __device__ __forceinline__ frag load(const i32x4* tile, int row, int lgrp, int) {
+    const i32x4 lo = tile[lds_slot<SW>(row, 2 * lgrp)], hi = tile[lds_slot<SW>(row, 2 * lgrp + 1)];
     return frag{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
   }
   static __device__ __forceinline__ f32x4 run(const frag& w, const frag& a, f32x4 acc) {
@@ -45,8 +52,8 @@ template <> struct StepMfma<2> {
   // bf16: two passes; in pass h lane group g owns chunk g + 4h (8 values) -> v_mfma_f32_16x16x32_bf16
   typedef i32x4 frag;
   static constexpr int PASSES = 2;
-  static __device__ __forceinline__ frag load(const i32x4* tile, int row, int lgrp, int pass) {
-    return tile[lds_slot(row, lgrp + 4 * pass)];
+  template <int SW> static __device__ __forceinline__ frag load(const i32x4* tile, int row, int lgrp, int pass) {
+    return tile[lds_slot<SW>(row, lgrp + 4 * pass)];
   }
   static __device__ __forceinline__ f32x4 run(const frag& w, const frag& a, f32x4 acc) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, w), __builtin_bit_cast(bf16x8, a), acc, 0, 0, 0);
@@ -59,7 +66,7 @@ __device__ __forceinline__ void store_out(void* out, int out_dtype, int64_t idx,
   else ((float*)out)[idx] = v;
 }
 
-template <int EB, int BM, int BN, int WM, int WN, bool KTAIL>
+template <int EB, int BM, int BN, int WM, int WN, int SW, bool KTAIL>
 __global__ void __launch_bounds__(WM * WN * 64)
 gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_t* __restrict__ A,
                const uint8_t* __restrict__ W, const float* __restrict__ a_scales, const float* __restrict__ w_scales,
@@ -133,13 +140,13 @@ gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_
 #pragma unroll
     for (int i = 0; i < A_PER; ++i) {
       const int idx = tid + i * NT;
-      if (A_CHUNKS % NT == 0 || idx < A_CHUNKS) lds[buf][lds_slot(idx / kChunksPerRow, idx % kChunksPerRow)] = ra[set][i];
+      if (A_CHUNKS % NT == 0 || idx < A_CHUNKS) lds[buf][lds_slot<SW>(idx / kChunksPerRow, idx % kChunksPerRow)] = ra[set][i];
     }
 #pragma unroll
     for (int i = 0; i < W_PER; ++i) {
       const int idx = tid + i * NT;
       if (W_CHUNKS % NT == 0 || idx < W_CHUNKS)
-        lds[buf][A_CHUNKS + lds_slot(idx / kChunksPerRow, idx % kChunksPerRow)] = rw[set][i];
+        lds[buf][A_CHUNKS + lds_slot<SW>(idx / kChunksPerRow, idx % kChunksPerRow)] = rw[set][i];
     }
   };
 
@@ -155,9 +162,9 @@ gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_
     for (int pass = 0; pass < StepMfma<EB>::PASSES; ++pass) {
       frag fa[MI], fw[NI];
 #pragma unroll
-      for (int i = 0; i < MI; ++i) fa[i] = StepMfma<EB>::load(&lds[buf][0], wm * TM + i * 16 + lrow, lgrp, pass);
+      for (int i = 0; i < MI; ++i) fa[i] = StepMfma<EB>::template load<SW>(&lds[buf][0], wm * TM + i * 16 + lrow, lgrp, pass);
 #pragma unroll
-      for (int j = 0; j < NI; ++j) fw[j] = StepMfma<EB>::load(&lds[buf][A_CHUNKS], wn * TN + j * 16 + lrow, lgrp, pass);
+      for (int j = 0; j < NI; ++j) fw[j] = StepMfma<EB>::template load<SW>(&lds[buf][A_CHUNKS], wn * TN + j * 16 + lrow, lgrp, pass);
 #pragma unroll
       for (int i = 0; i < MI; ++i)
 #pragma unroll
@@ -292,7 +299,7 @@ Plan default_plan(int64_t M, int64_t N, int64_t Kb) {
   return {tile, splits};
 }
 
-template <int EB, int BM, int BN, int WM, int WN>
+template <int EB, int BM, int BN, int WM, int WN, int SW>
 void launch_tile(void* out, float* partial, const uint8_t* A, const uint8_t* W, const float* as, const float* ws, int M,
                  int N, int64_t Kb, int splits, int out_dtype, bool keep_partials, hipStream_t s) {
   const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
@@ -300,10 +307,10 @@ void launch_tile(void* out, float* partial, const uint8_t* A, const uint8_t* W, 
   const int per = (int)((steps + splits - 1) / splits);
   const dim3 grid((tiles + 7) / 8 * 8, splits), block(WM * WN * 64);
   if (Kb % kStepBytes == 0)
-    hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN, false>), grid, block, 0, s, out, (splits > 1 || keep_partials) ? partial : nullptr, A, W,
+    hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN, SW, false>), grid, block, 0, s, out, (splits > 1 || keep_partials) ? partial : nullptr, A, W,
                        as, ws, M, N, Kb, per, out_dtype);
   else
-    hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN, true>), grid, block, 0, s, out, (splits > 1 || keep_partials) ? partial : nullptr, A, W,
+    hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN, SW, true>), grid, block, 0, s, out, (splits > 1 || keep_partials) ? partial : nullptr, A, W,
                        as, ws, M, N, Kb, per, out_dtype);
 }
 
@@ -335,7 +342,7 @@ int gemm_entry(const char* name, void* out, const void* a, const float* as, cons
   LFM2_REQUIRE(plan.splits == 1 || workspace != nullptr, "%s: split-K needs a workspace", name);
   LFM2_REQUIRE(reduce || workspace != nullptr, "%s: partial products need a destination", name);
 #define TILE_(ID, BM, BN, WM, WN) \
-  case ID: launch_tile<EB, BM, BN, WM, WN>(out, workspace, A, W, as, ws, (int)M, (int)N, Kb, plan.splits, out_dtype, !reduce, s); break
+  case ID: launch_tile<EB, BM, BN, WM, WN, EB == 1 ? 1 : 0>(out, workspace, A, W, as, ws, (int)M, (int)N, Kb, plan.splits, out_dtype, !reduce, s); break
   switch (plan.tile) {
     TILE_(0, 16, 64, 1, 4);
     TILE_(1, 32, 64, 2, 2);
