@@ -18,16 +18,17 @@
 
 namespace {
 
-constexpr int kStepBytes = 128;          // K bytes staged per step
-constexpr int kChunksPerRow = kStepBytes / 16;
+constexpr int kStepBytes = 128;          // K bytes one MFMA pass group consumes per row (and the default staging step)
 
 // Slot of a row's 16-byte chunk in a staged tile.  The XOR pattern is chosen per operand type from a sweep of
 // ds_read_b128 patterns on gfx950 (LDS reads peak at 256 B/clk): the e4m3 fragment read (16 rows x chunks 2g, 2g+1)
 // runs at 240 B/clk with row&7 ^ bit 3 of the row and at 128 B/clk with row&7 alone; the bf16 fragment read
 // (chunk g + 4*pass) is the other way round.  Staging writes (8 lanes per row) are indifferent (78 B/clk either way).
-template <int SW> __device__ __forceinline__ int lds_slot(int row, int chunk) {
-  const int x = SW == 1 ? ((row & 7) ^ ((row >> 3) & 1)) : (row & 7);
-  return row * kChunksPerRow + (chunk ^ x);
+// CPR = chunks per staged row (8 for 128-byte K steps, 16 for 256-byte steps, where rows are a full bank sweep apart
+// and the XOR must cover four chunk bits: row&15 reads at 241 B/clk, row&7 at 128).
+template <int SW, int CPR> __device__ __forceinline__ int lds_slot(int row, int chunk) {
+  const int x = CPR == 16 ? (row & 15) : SW == 1 ? ((row & 7) ^ ((row >> 3) & 1)) : (row & 7);
+  return row * CPR + (chunk ^ x);
 }
 
 typedef int i32x8 __attribute__((ext_vector_type(8)));
@@ -40,8 +41,8 @@ template <> struct StepMfma<1> {
   // e4m3: lane group g owns chunks 2g, 2g+1 (32 bytes) -> one v_mfma_f32_16x16x128_f8f6f4 (unit scales)
   typedef i32x8 frag;
   static constexpr int PASSES = 1;
-  template <int SW> static __device__ __forceinline__ frag load(const i32x4* tile, int row, int lgrp, int) {
-    const i32x4 lo = tile[lds_slot<SW>(row, 2 * lgrp)], hi = tile[lds_slot<SW>(row, 2 * lgrp + 1)];
+  template <int SW, int CPR> static __device__ __forceinline__ frag load(const i32x4* tile, int row, int lgrp, int, int sub) {
+    const i32x4 lo = tile[lds_slot<SW, CPR>(row, 8 * sub + 2 * lgrp)], hi = tile[lds_slot<SW, CPR>(row, 8 * sub + 2 * lgrp + 1)];
     return frag{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
   }
   static __device__ __forceinline__ f32x4 run(const frag& w, const frag& a, f32x4 acc) {
@@ -52,8 +53,8 @@ template <> struct StepMfma<2> {
   // bf16: two passes; in pass h lane group g owns chunk g + 4h (8 values) -> v_mfma_f32_16x16x32_bf16
   typedef i32x4 frag;
   static constexpr int PASSES = 2;
-  template <int SW> static __device__ __forceinline__ frag load(const i32x4* tile, int row, int lgrp, int pass) {
-    return tile[lds_slot<SW>(row, lgrp + 4 * pass)];
+  template <int SW, int CPR> static __device__ __forceinline__ frag load(const i32x4* tile, int row, int lgrp, int pass, int sub) {
+    return tile[lds_slot<SW, CPR>(row, 8 * sub + lgrp + 4 * pass)];
   }
   static __device__ __forceinline__ f32x4 run(const frag& w, const frag& a, f32x4 acc) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, w), __builtin_bit_cast(bf16x8, a), acc, 0, 0, 0);
@@ -66,13 +67,14 @@ __device__ __forceinline__ void store_out(void* out, int out_dtype, int64_t idx,
   else ((float*)out)[idx] = v;
 }
 
-template <int EB, int BM, int BN, int WM, int WN, int SW, bool KTAIL>
+template <int EB, int BM, int BN, int WM, int WN, int SW, int KS, bool KTAIL>
 __global__ void __launch_bounds__(WM * WN * 64)
 gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_t* __restrict__ A,
                const uint8_t* __restrict__ W, const float* __restrict__ a_scales, const float* __restrict__ w_scales,
                int M, int N, int64_t Kb, int steps_per_split, int out_dtype) {
   constexpr int NT = WM * WN * 64;
   constexpr int TM = BM / WM, TN = BN / WN, MI = TM / 16, NI = TN / 16;
+  constexpr int kChunksPerRow = KS / 16;  // KS = K bytes staged per step and row: 128, or 256 (two MFMA sub-steps per barrier)
   constexpr int A_CHUNKS = BM * kChunksPerRow, W_CHUNKS = BN * kChunksPerRow;
   constexpr int A_PER = (A_CHUNKS + NT - 1) / NT, W_PER = (W_CHUNKS + NT - 1) / NT;
   __shared__ i32x4 lds[2][A_CHUNKS + W_CHUNKS];
@@ -84,7 +86,7 @@ gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_
   if (lid >= tiles) return;
   const int m_base = (lid % mt) * BM, n_base = (lid / mt) * BN;
 
-  const int64_t total_steps = (Kb + kStepBytes - 1) / kStepBytes;
+  const int64_t total_steps = (Kb + KS - 1) / KS;
   const int64_t step0 = (int64_t)blockIdx.y * steps_per_split;
   int64_t nsteps = total_steps - step0;
   if (nsteps > steps_per_split) nsteps = steps_per_split;
@@ -100,7 +102,7 @@ gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_
   // no branch between issue and use the compiler keeps them in flight across the MFMAs of two K steps.
   auto fetch = [&](int64_t step, int set) {
     step = step < nsteps ? step : nsteps - 1;
-    const int64_t kb = (step0 + step) * kStepBytes;
+    const int64_t kb = (step0 + step) * KS;
 #pragma unroll
     for (int i = 0; i < A_PER; ++i) {
       int idx = tid + i * NT;
@@ -140,13 +142,13 @@ gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_
 #pragma unroll
     for (int i = 0; i < A_PER; ++i) {
       const int idx = tid + i * NT;
-      if (A_CHUNKS % NT == 0 || idx < A_CHUNKS) lds[buf][lds_slot<SW>(idx / kChunksPerRow, idx % kChunksPerRow)] = ra[set][i];
+      if (A_CHUNKS % NT == 0 || idx < A_CHUNKS) lds[buf][lds_slot<SW, kChunksPerRow>(idx / kChunksPerRow, idx % kChunksPerRow)] = ra[set][i];
     }
 #pragma unroll
     for (int i = 0; i < W_PER; ++i) {
       const int idx = tid + i * NT;
       if (W_CHUNKS % NT == 0 || idx < W_CHUNKS)
-        lds[buf][A_CHUNKS + lds_slot<SW>(idx / kChunksPerRow, idx % kChunksPerRow)] = rw[set][i];
+        lds[buf][A_CHUNKS + lds_slot<SW, kChunksPerRow>(idx / kChunksPerRow, idx % kChunksPerRow)] = rw[set][i];
     }
   };
 
@@ -159,16 +161,21 @@ gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_
   auto multiply = [&](int buf) {
     typedef typename StepMfma<EB>::frag frag;
 #pragma unroll
-    for (int pass = 0; pass < StepMfma<EB>::PASSES; ++pass) {
-      frag fa[MI], fw[NI];
+    for (int sub = 0; sub < KS / kStepBytes; ++sub) {
 #pragma unroll
-      for (int i = 0; i < MI; ++i) fa[i] = StepMfma<EB>::template load<SW>(&lds[buf][0], wm * TM + i * 16 + lrow, lgrp, pass);
+      for (int pass = 0; pass < StepMfma<EB>::PASSES; ++pass) {
+        frag fa[MI], fw[NI];
 #pragma unroll
-      for (int j = 0; j < NI; ++j) fw[j] = StepMfma<EB>::template load<SW>(&lds[buf][A_CHUNKS], wn * TN + j * 16 + lrow, lgrp, pass);
+        for (int i = 0; i < MI; ++i)
+          fa[i] = StepMfma<EB>::template load<SW, kChunksPerRow>(&lds[buf][0], wm * TM + i * 16 + lrow, lgrp, pass, sub);
 #pragma unroll
-      for (int i = 0; i < MI; ++i)
+        for (int j = 0; j < NI; ++j)
+          fw[j] = StepMfma<EB>::template load<SW, kChunksPerRow>(&lds[buf][A_CHUNKS], wn * TN + j * 16 + lrow, lgrp, pass, sub);
 #pragma unroll
-        for (int j = 0; j < NI; ++j) acc[i][j] = StepMfma<EB>::run(fw[j], fa[i], acc[i][j]);
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+          for (int j = 0; j < NI; ++j) acc[i][j] = StepMfma<EB>::run(fw[j], fa[i], acc[i][j]);
+      }
     }
   };
 
@@ -268,10 +275,12 @@ gemm_naive_kernel(void* out, const uint8_t* A, const uint8_t* W, const float* a_
   store_out(out, out_dtype, idx, t);
 }
 
-struct TileInfo { int bm, bn; };
-constexpr int kNumTiles = 9;
-constexpr TileInfo kTiles[kNumTiles] = {{16, 64}, {32, 64}, {64, 64}, {128, 64}, {128, 128}, {64, 128},
-                                        {128, 128}, {64, 128}, {128, 64}};
+struct TileInfo { int bm, bn, ks; };
+constexpr int kNumTiles = 12;
+constexpr TileInfo kTiles[kNumTiles] = {{16, 64, 128}, {32, 64, 128}, {64, 64, 128}, {128, 64, 128}, {128, 128, 128},
+                                        {64, 128, 128}, {128, 128, 128}, {64, 128, 128}, {128, 64, 128},
+                                        {16, 64, 256}, {32, 64, 256}, {64, 64, 256}};
+int64_t tile_steps(int tile, int64_t Kb) { return (Kb + kTiles[tile].ks - 1) / kTiles[tile].ks; }
 
 struct Plan { int tile, splits; };
 
@@ -287,6 +296,10 @@ Plan default_plan(int64_t M, int64_t N, int64_t Kb) {
   else if (count(2) >= 512) tile = 2;
   else if (count(1) >= 256 || M <= 64) tile = M <= 64 ? 2 : 1;
   else tile = 2;
+  // With at most about one and a half 32x64 workgroups per CU nothing overlaps a workgroup's serial chain of K
+  // steps (wait, LDS write, barrier, LDS read, MFMA), so halve the number of links: 256-byte K steps
+  // (7.2 us against 8.7 us at M=256, N=K=2048; with more workgroups per CU the smaller step wins).
+  if (tile == 1 && count(1) <= 384 && Kb >= 2048) tile = 10;
   const int64_t steps = (Kb + kStepBytes - 1) / kStepBytes;
   int splits = 1;
   // Long-K products whose tiles cannot fill the chip (the SwiGLU down projection at decode batch sizes): a workgroup's
@@ -299,18 +312,18 @@ Plan default_plan(int64_t M, int64_t N, int64_t Kb) {
   return {tile, splits};
 }
 
-template <int EB, int BM, int BN, int WM, int WN, int SW>
+template <int EB, int BM, int BN, int WM, int WN, int SW, int KS>
 void launch_tile(void* out, float* partial, const uint8_t* A, const uint8_t* W, const float* as, const float* ws, int M,
                  int N, int64_t Kb, int splits, int out_dtype, bool keep_partials, hipStream_t s) {
   const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-  const int64_t steps = (Kb + kStepBytes - 1) / kStepBytes;
+  const int64_t steps = (Kb + KS - 1) / KS;
   const int per = (int)((steps + splits - 1) / splits);
   const dim3 grid((tiles + 7) / 8 * 8, splits), block(WM * WN * 64);
-  if (Kb % kStepBytes == 0)
-    hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN, SW, false>), grid, block, 0, s, out, (splits > 1 || keep_partials) ? partial : nullptr, A, W,
+  if (Kb % KS == 0)
+    hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN, SW, KS, false>), grid, block, 0, s, out, (splits > 1 || keep_partials) ? partial : nullptr, A, W,
                        as, ws, M, N, Kb, per, out_dtype);
   else
-    hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN, SW, true>), grid, block, 0, s, out, (splits > 1 || keep_partials) ? partial : nullptr, A, W,
+    hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN, SW, KS, true>), grid, block, 0, s, out, (splits > 1 || keep_partials) ? partial : nullptr, A, W,
                        as, ws, M, N, Kb, per, out_dtype);
 }
 
@@ -335,24 +348,27 @@ int gemm_entry(const char* name, void* out, const void* a, const float* as, cons
     plan.tile = tile;
   }
   if (split_k > 0) plan.splits = split_k;
-  const int64_t steps = (Kb + kStepBytes - 1) / kStepBytes;
+  const int64_t steps = tile_steps(plan.tile, Kb);
   if (plan.splits > steps) plan.splits = (int)steps;
   // every split must own at least one step
   while (plan.splits > 1 && (steps + plan.splits - 1) / plan.splits * (plan.splits - 1) >= steps) --plan.splits;
   LFM2_REQUIRE(plan.splits == 1 || workspace != nullptr, "%s: split-K needs a workspace", name);
   LFM2_REQUIRE(reduce || workspace != nullptr, "%s: partial products need a destination", name);
-#define TILE_(ID, BM, BN, WM, WN) \
-  case ID: launch_tile<EB, BM, BN, WM, WN, EB == 1 ? 1 : 0>(out, workspace, A, W, as, ws, (int)M, (int)N, Kb, plan.splits, out_dtype, !reduce, s); break
+#define TILE_(ID, BM, BN, WM, WN, KS) \
+  case ID: launch_tile<EB, BM, BN, WM, WN, EB == 1 ? 1 : 0, KS>(out, workspace, A, W, as, ws, (int)M, (int)N, Kb, plan.splits, out_dtype, !reduce, s); break
   switch (plan.tile) {
-    TILE_(0, 16, 64, 1, 4);
-    TILE_(1, 32, 64, 2, 2);
-    TILE_(2, 64, 64, 2, 2);
-    TILE_(3, 128, 64, 2, 2);
-    TILE_(4, 128, 128, 2, 2);
-    TILE_(5, 64, 128, 2, 2);
-    TILE_(6, 128, 128, 2, 4);
-    TILE_(7, 64, 128, 2, 4);
-    TILE_(8, 128, 64, 4, 2);
+    TILE_(0, 16, 64, 1, 4, 128);
+    TILE_(1, 32, 64, 2, 2, 128);
+    TILE_(2, 64, 64, 2, 2, 128);
+    TILE_(3, 128, 64, 2, 2, 128);
+    TILE_(4, 128, 128, 2, 2, 128);
+    TILE_(5, 64, 128, 2, 2, 128);
+    TILE_(6, 128, 128, 2, 4, 128);
+    TILE_(7, 64, 128, 2, 4, 128);
+    TILE_(8, 128, 64, 4, 2, 128);
+    TILE_(9, 16, 64, 1, 4, 256);
+    TILE_(10, 32, 64, 2, 2, 256);
+    TILE_(11, 64, 64, 2, 2, 256);
   }
 #undef TILE_
   if (plan.splits > 1 && reduce)
@@ -374,7 +390,8 @@ extern "C" int lfm2_fp8_gemm(void* out, const uint8_t* a_q, const float* a_scale
 extern "C" int lfm2_fp8_gemm_partials(float* partials, const uint8_t* a_q, const uint8_t* w_q, int64_t M, int64_t N,
                                       int64_t K, int tile, int split_k, void* stream) {
   LFM2_REQUIRE(split_k >= 1 && split_k <= 16, "fp8_gemm_partials: split_k %d not in [1,16]", split_k);
-  const int64_t steps = (K + kStepBytes - 1) / kStepBytes;
+  LFM2_REQUIRE(tile < kNumTiles, "fp8_gemm_partials: tile index %d out of range", tile);
+  const int64_t steps = tile_steps(tile >= 0 ? tile : default_plan(M, N, K).tile, K);
   LFM2_REQUIRE(split_k <= steps && (steps + split_k - 1) / split_k * (split_k - 1) < steps,
                "fp8_gemm_partials: %d splits leave one without a K step", split_k);
   return gemm_entry<1>("fp8_gemm_partials", nullptr, a_q, nullptr, w_q, nullptr, partials, M, N, K, LFM2_DTYPE_F32, tile,
