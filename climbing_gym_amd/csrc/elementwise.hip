@@ -143,6 +143,13 @@ rms_norm_kernel(T* out, uint8_t* q, float* scales, T* summed, const T* x, const 
         for (int e = 0; e < N; ++e) ss += v[j][e] * v[j][e];
       }
     }
+    // the norm weights do not depend on the reduction: fetch them before it, so the kernel pays one memory round trip
+    float g[NV][N];
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int64_t i = (int64_t)(j * kThreads + threadIdx.x) * N;
+      if (i < H) load_vec<T>(w + i, g[j]);
+    }
     ss = block_sum<kWaves>(ss, red);
     const float rstd = 1.0f / sqrtf(ss / (float)H + eps);
     float amax = 0.f;
@@ -150,11 +157,9 @@ rms_norm_kernel(T* out, uint8_t* q, float* scales, T* summed, const T* x, const 
     for (int j = 0; j < NV; ++j) {
       const int64_t i = (int64_t)(j * kThreads + threadIdx.x) * N;
       if (i < H) {
-        float g[N];
-        load_vec<T>(w + i, g);
 #pragma unroll
         for (int e = 0; e < N; ++e) {
-          v[j][e] = round_to<T>(v[j][e] * rstd) * g[e];
+          v[j][e] = round_to<T>(v[j][e] * rstd) * g[j][e];
           if (FP8) { v[j][e] = round_to<T>(v[j][e]); amax = fmaxf(amax, fabsf(v[j][e])); }
         }
         if (!FP8) store_vec<T>(out + i, v[j]);
@@ -621,28 +626,35 @@ __global__ void __launch_bounds__(kThreads) prepare_qkv_wave_kernel(PrepArgs a) 
 #pragma unroll
   for (int i = 0; i < R; ++i) val[i] = on ? Elem<T>::load(src[lane + 64 * i]) : 0.f;
   if (u < a.QH + a.KH) {
+    // everything the head needs is requested before the reduction: norm weights, and the rotary factors behind the
+    // row's position
     const T* wgt = u < a.QH ? (const T*)a.qw : (const T*)a.kw;
+    int64_t pos = a.positions[row];
+    pos = pos < 0 ? 0 : (pos >= a.max_positions ? a.max_positions - 1 : pos);
+    float gw[R], c[R], sn[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      const int t = on ? (lane + 64 * i) % half : 0;
+      gw[i] = on ? Elem<T>::load(wgt[lane + 64 * i]) : 0.f;
+      c[i] = round_to<T>(a.cosT[pos * half + t]);
+      sn[i] = round_to<T>(a.sinT[pos * half + t]);
+    }
     float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < R; ++i) ss += val[i] * val[i];
     ss = wave_sum(ss);
     const float rstd = 1.0f / sqrtf(ss / (float)D + a.eps);
-    int64_t pos = a.positions[row];
-    pos = pos < 0 ? 0 : (pos >= a.max_positions ? a.max_positions - 1 : pos);
     float w[R];
 #pragma unroll
     for (int i = 0; i < R; ++i) {
       const float n = round_to<T>(val[i] * rstd);
-      w[i] = on ? round_to<T>(n * Elem<T>::load(wgt[lane + 64 * i])) : 0.f;
+      w[i] = on ? round_to<T>(n * gw[i]) : 0.f;
     }
 #pragma unroll
     for (int i = 0; i < R; ++i) {
       const int d = lane + 64 * i;
-      const int t = on ? d % half : 0;
-      const float c = round_to<T>(a.cosT[pos * half + t]);
-      const float sn = round_to<T>(a.sinT[pos * half + t]);
       const float partner = D >= 128 ? w[i ^ (D / 128)] : __shfl_xor(w[i], half, 64);
-      const float left = round_to<T>(w[i] * c), right = round_to<T>(partner * sn);
+      const float left = round_to<T>(w[i] * c[i]), right = round_to<T>(partner * sn[i]);
       val[i] = round_to<T>(d < half ? left - right : left + right);
     }
   }
