@@ -502,3 +502,28 @@ def test_score_completions_matches_teacher_forced_oracle():
             want.append(float(logits[0].log_softmax(-1)[t]))
             logits = oracle.append_tokens(cache, torch.tensor([0]), torch.tensor([t]))
         torch.testing.assert_close(torch.tensor(scores), torch.tensor(want), atol=2e-2, rtol=0)
+
+
+@torch.inference_mode()
+def test_tiny_model_greedy_tokens_against_the_committed_vectors():
+    """tests/golden/config1_greedy.json holds the fp32 CPU result of the CPU-runnable benchmark case.  The bf16 HIP
+    path, free running, must produce the same ids up to the first position where the recorded margin between the
+    two best tokens is below 2e-2 (the logits tolerance): before that point every id is pinned."""
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "config1_greedy.json")) as f:
+        golden = json.load(f)
+    engine, _, _, prompts = _config1()
+    assert [len(p) for p in prompts] == golden["prompt_lengths"] and [p[:4] for p in prompts] == golden["prompt_heads"]
+    engine.enable_cuda_graphs(max_graphs=1)
+    out = engine.generate(*_flat(prompts), repeats=1,
+                          sampling=LFM25SamplingConfig(temperature=0.0, max_new_tokens=64, ignore_eos=True))
+    mine = out.token_ids[:, 0].cpu().tolist()
+    pinned = 0
+    for row in range(4):
+        margins = golden["margin_to_second"][row]
+        horizon = next((i for i, m in enumerate(margins) if m < 2e-2), 64)
+        assert mine[row][:horizon] == golden["token_ids"][row][:horizon], f"row {row} differs before step {horizon}"
+        pinned += horizon
+    print(f"{pinned} of 256 greedy ids pinned by the golden vectors")
+    assert pinned >= 128

@@ -138,3 +138,25 @@ def test_capacity_rounding_known_answers():
     assert graph_capacity(22 + 20, 64, 256) == 64
     assert graph_capacity(30, 3, 256) == 128
     assert graph_capacity(250, 3, 256) == 256
+
+
+def test_oracle_reproduces_the_committed_config1_vectors():
+    """tests/golden/config1_greedy.json (written by tests/golden/make_config1.py, first tokens cross-checked against
+    Transformers there): the oracle must keep producing those 4 x 64 greedy ids, logprobs and margins."""
+    import json
+    import os
+    import sys
+    here = os.path.dirname(os.path.abspath(__file__))
+    sys.path.insert(0, os.path.join(here, "golden"))
+    import make_config1
+    with open(os.path.join(here, "golden", "config1_greedy.json")) as f:
+        golden = json.load(f)
+    cfg, state, prompts = make_config1.build()
+    assert [len(p) for p in prompts] == golden["prompt_lengths"] and [p[:4] for p in prompts] == golden["prompt_heads"]
+    oracle = OracleEngine(cfg, state, torch.float32, max_model_len=256)
+    with torch.inference_mode():
+        tokens, logprobs, trace = oracle.generate(prompts, 64, temperature=0.0, return_logits=True)
+    assert tokens.tolist() == golden["token_ids"]
+    torch.testing.assert_close(logprobs, torch.tensor(golden["logprobs"]), atol=2e-5, rtol=0)
+    best = torch.stack([t.max(-1).values for t in trace], 1)
+    torch.testing.assert_close(best, torch.tensor(golden["best_logit"]), atol=2e-4, rtol=0)
