@@ -24,6 +24,10 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 
 
+def fp8_requested(args):
+    return args.precision == "fp8"
+
+
 def parse_args():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
@@ -83,6 +87,59 @@ def time_decode_attention(engine, session, samples):
     kv_token = cfg.num_key_value_heads * cfg.head_dim * 2 * (1 if cache.fp8 else 2) + (cfg.num_key_value_heads * 2 * 4 if cache.fp8 else 0)
     bytes_per_call = tokens * kv_token + 2 * rows * cfg.num_attention_heads * cfg.head_dim * 2
     return total_ms / 1000 / launches, bytes_per_call, tokens
+
+
+def time_gemms(engine, rows=256, prefill_rows=4096, repeats=5):
+    """Secondary figures: the W8A8 projections at the decode batch size, cycling through the layers' weights so they
+    stream from HBM (GB/s of weight bytes; HBM-bound regime), and the fused gate+up projection at a prefill chunk of
+    4096 tokens (TFLOP/s against the 5.0 PFLOP/s dense fp8 MFMA peak).  HIP events on the launch stream."""
+    from climbing_gym_amd import ops
+    fp8 = engine._fp8()
+    layers = engine.weights.layers
+    groups = {"w13": [fp8.get(id(l.w13_weight)) for l in layers], "w2": [fp8.get(id(l.w2_weight)) for l in layers],
+              "qkv": [fp8.get(id(l.attention.qkv_weight)) for l in layers if l.attention is not None],
+              "conv_in": [fp8.get(id(l.conv.in_weight)) for l in layers if l.conv is not None],
+              "out": [fp8.get(id((l.attention or l.conv).out_weight)) for l in layers]}
+    stream = torch.cuda.current_stream()
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    out = {"decode_rows": rows, "decode": {}, "prefill_rows": prefill_rows}
+
+    def run(packs, m):
+        width = packs[0].values.size(1)
+        x = torch.randn(m, width, device="cuda", dtype=torch.bfloat16)
+        xq, xs = ops.quantize_rows(x)
+        def body():
+            for _ in range(repeats):
+                for p in packs:
+                    p.linear_quantized(xq, xs)
+        body()
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()   # captured and replayed as one graph: host launch cost stays out of the figure
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side), torch.cuda.graph(graph, stream=side):
+            body()
+        torch.cuda.synchronize()
+        graph.replay()
+        begin.record(stream)
+        graph.replay()
+        end.record(stream)
+        end.synchronize()
+        return begin.elapsed_time(end) / 1000 / (repeats * len(packs))
+    for name, packs in groups.items():
+        if any(p is None for p in packs) or not packs:
+            continue
+        n, k = packs[0].values.shape
+        sec = run(packs, rows)
+        out["decode"][name] = {"n": n, "k": k, "us": round(sec * 1e6, 2), "weight_GBps": round(n * k / sec / 1e9, 1),
+                               "TFLOPs": round(2 * rows * n * k / sec / 1e12, 1)}
+    packs = groups["w13"]
+    if packs and packs[0] is not None:
+        n, k = packs[0].values.shape
+        sec = run(packs[:4], prefill_rows)
+        tflops = 2 * prefill_rows * n * k / sec / 1e12
+        out["prefill"] = {"name": "w13", "n": n, "k": k, "us": round(sec * 1e6, 1), "TFLOPs": round(tflops, 1),
+                          "mfma_fp8_frac_of_5PF": round(tflops / 5000, 4)}
+    return out
 
 
 def calibration_copy():
@@ -165,6 +222,7 @@ def main():
         assert not finished, "no sequence may finish inside the timed region"
         attn_s, attn_bytes, ctx_tokens = time_decode_attention(engine, session, args.attn_samples)
         calibration_copy()
+        gemms = time_gemms(engine) if fp8_requested(args) else None
         kv_token = 6 * (attn_bytes - 2 * args.batch * 32 * 64 * 2) // max(ctx_tokens, 1)
     fp8 = args.precision == "fp8"
     weights = sum(w.numel() for w in set(engine.weights.linear_matrices())) * (1 if fp8 else 2)
@@ -181,7 +239,7 @@ def main():
                                f"concurrent sequences, prompts U[{args.prompt_low},{args.prompt_high}] tokens, temperature 1, "
                                f"max_model_len {args.max_model_len}, HIP-graph decode step",
                    "context_tokens": ctx_tokens, "prefill_tok_per_s": round(sum(map(len, prompts)) / prefill_s, 1),
-                   "step_algorithmic_bytes": step_bytes,
+                   "gemm": gemms, "step_algorithmic_bytes": step_bytes,
                    "step_hbm_fraction": round(step_bytes / (ms_per_step / 1000) / 1e9 / HBM_PEAK_GBS, 4)},
         "roofline": {"kernel": "decode_attn_mfma_kernel + decode_combine_kernel (one ragged GQA decode-attention call, e4m3 KV)"
                                if fp8 else "decode_attn_kernel + decode_combine_kernel (bf16 KV)",
