@@ -67,7 +67,7 @@ __device__ __forceinline__ void store_out(void* out, int out_dtype, int64_t idx,
   else ((float*)out)[idx] = v;
 }
 
-template <int EB, int BM, int BN, int WM, int WN, int SW, int KS, bool KTAIL>
+template <int EB, int BM, int BN, int WM, int WN, int SW, int KS, bool KTAIL, int ST = 0>
 __global__ void __launch_bounds__(WM * WN * 64)
 gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_t* __restrict__ A,
                const uint8_t* __restrict__ W, const float* __restrict__ a_scales, const float* __restrict__ w_scales,
@@ -77,7 +77,9 @@ gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_
   constexpr int kChunksPerRow = KS / 16;  // KS = K bytes staged per step and row: 128, or 256 (two MFMA sub-steps per barrier)
   constexpr int A_CHUNKS = BM * kChunksPerRow, W_CHUNKS = BN * kChunksPerRow;
   constexpr int A_PER = (A_CHUNKS + NT - 1) / NT, W_PER = (W_CHUNKS + NT - 1) / NT;
-  __shared__ i32x4 lds[2][A_CHUNKS + W_CHUNKS];
+  // ST = 0: tiles staged through registers into two LDS buffers; ST >= 2: a ring of ST LDS buffers filled by
+  // direct global->LDS loads (no staging registers, no ds_write and no wait between load and LDS store)
+  __shared__ i32x4 lds[ST > 0 ? ST : 2][A_CHUNKS + W_CHUNKS];
 
   // XCD-aware tile order: consecutive logical ids (same XCD, adjacent in time) share an N tile.
   const int mt = (M + BM - 1) / BM, nt = (N + BN - 1) / BN, tiles = mt * nt;
@@ -179,6 +181,55 @@ gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_
     }
   };
 
+  if constexpr (ST > 0) {
+    static_assert(!KTAIL, "direct-to-LDS loads cannot zero-fill a partial K step");
+    static_assert(A_CHUNKS % 64 == 0 && W_CHUNKS % 64 == 0, "a wave fills 64 consecutive slots per instruction");
+    // Slot s of a staged tile holds (row s / CPR, chunk (s % CPR) ^ swizzle(row)); the instruction writes lane l's
+    // 16 bytes to slot base + l, so each lane fetches the global chunk that belongs to its slot.
+    auto issue = [&](int64_t step, int buf) {
+      step = step < nsteps ? step : nsteps - 1;
+      const int64_t kb = (step0 + step) * KS;
+#pragma unroll
+      for (int i = 0; i < A_PER; ++i) {
+        const int slot = i * NT + tid;
+        if (A_CHUNKS % NT == 0 || slot < A_CHUNKS) {
+          const int row = slot / kChunksPerRow;
+          const int c = lds_slot<SW, kChunksPerRow>(row, slot % kChunksPerRow) - row * kChunksPerRow;
+          int gr = m_base + row;
+          gr = gr < M ? gr : M - 1;
+          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(A + (int64_t)gr * Kb + kb + c * 16),
+                                           (__attribute__((address_space(3))) void*)(&lds[buf][i * NT + wave * 64]), 16, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < W_PER; ++i) {
+        const int slot = i * NT + tid;
+        if (W_CHUNKS % NT == 0 || slot < W_CHUNKS) {
+          const int row = slot / kChunksPerRow;
+          const int c = lds_slot<SW, kChunksPerRow>(row, slot % kChunksPerRow) - row * kChunksPerRow;
+          int gr = n_base + row;
+          gr = gr < N ? gr : N - 1;
+          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(W + (int64_t)gr * Kb + kb + c * 16),
+                                           (__attribute__((address_space(3))) void*)(&lds[buf][A_CHUNKS + i * NT + wave * 64]), 16, 0, 0);
+        }
+      }
+    };
+    // loads complete in order: with ST-1 steps in flight, step s has landed once at most ST-2 steps' loads remain
+    constexpr int kPending = (ST - 2) * (A_PER + W_PER);
+    constexpr int kWait = (kPending & 0xF) | (0x7 << 4) | (0xF << 8) | ((kPending >> 4) << 14);  // vmcnt only
+#pragma unroll
+    for (int st = 0; st < ST - 1; ++st) issue(st, st);
+    int buf = 0, fill = ST - 1;
+    for (int64_t s = 0; s < nsteps; ++s) {
+      __builtin_amdgcn_s_waitcnt(kWait);
+      __builtin_amdgcn_s_barrier();  // (a bare barrier: __syncthreads would add a fence that drains the loads in flight)
+      // step s is in LDS for every wave, and every wave is done reading the buffer refilled next
+      issue(s + ST - 1, fill);
+      multiply(buf);
+      buf = buf + 1 == ST ? 0 : buf + 1;
+      fill = fill + 1 == ST ? 0 : fill + 1;
+    }
+  } else {
   if (nsteps > 0) {
     fetch(0, 0);
     fetch(1, 1);
@@ -202,6 +253,7 @@ gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_
       stash(0, 0);
       __syncthreads();
     }
+  }
   }
 
   // Epilogue: lane holds out[m = .. + lrow][n = .. + 4*lgrp + r], r = 0..3.
@@ -276,43 +328,38 @@ gemm_naive_kernel(void* out, const uint8_t* A, const uint8_t* W, const float* a_
 }
 
 struct TileInfo { int bm, bn, ks; };
-constexpr int kNumTiles = 12;
+constexpr int kNumTiles = 23;
 constexpr TileInfo kTiles[kNumTiles] = {{16, 64, 128}, {32, 64, 128}, {64, 64, 128}, {128, 64, 128}, {128, 128, 128},
                                         {64, 128, 128}, {128, 128, 128}, {64, 128, 128}, {128, 64, 128},
-                                        {16, 64, 256}, {32, 64, 256}, {64, 64, 256}};
+                                        {16, 64, 256}, {32, 64, 256}, {64, 64, 256},
+                                        {32, 64, 128}, {64, 64, 128}, {128, 128, 128}, {32, 64, 256},
+                                        {64, 64, 128}, {32, 64, 128}, {16, 64, 256}, {128, 64, 128}, {64, 128, 128},
+                                        {16, 64, 128}, {128, 64, 128}};
 int64_t tile_steps(int tile, int64_t Kb) { return (Kb + kTiles[tile].ks - 1) / kTiles[tile].ks; }
 
 struct Plan { int tile, splits; };
 
-// Default tile/split choice, from sweeps on MI355X at M = 256 (decode) and M = 4096 (prefill): the 8-wave 128x128
-// tile once it alone fills the 256 CUs, otherwise the largest smaller tile that gives every CU about two
-// workgroups; K is split (2 or 4 ways) only for long-K shapes that still leave CUs idle.
+// Default tile/split choice, from sweeps on MI355X at M = 256 (decode, weights streaming from HBM inside a HIP graph)
+// and M = 4096 (prefill).  Above 64 rows the direct-to-LDS ring variants win everywhere: the 8-wave 128x128 tile
+// once it alone fills the 256 CUs (1.3-2.0 PFLOP/s at M = 4096; 42 us for the 65536-row head at M = 256), otherwise
+// smaller tiles with deeper rings the fewer workgroups a CU gets (its K loop is then a serial chain that nothing
+// overlaps).  With K bytes not a multiple of the step these indices run their register-staged twins.
 Plan default_plan(int64_t M, int64_t N, int64_t Kb) {
   auto count = [&](int t) { return ((M + kTiles[t].bm - 1) / kTiles[t].bm) * ((N + kTiles[t].bn - 1) / kTiles[t].bn); };
+  const int64_t steps = (Kb + kStepBytes - 1) / kStepBytes;
   int tile;
   if (M <= 16) tile = 0;
   else if (M <= 32) tile = 1;
-  else if (count(6) >= 256) tile = 6;
-  else if (count(2) >= 512) tile = 2;
-  else if (count(1) >= 256 || M <= 64) tile = M <= 64 ? 2 : 1;
-  else tile = 2;
-  // With at most about one and a half 32x64 workgroups per CU nothing overlaps a workgroup's serial chain of K
-  // steps (wait, LDS write, barrier, LDS read, MFMA), so halve the number of links: 256-byte K steps
-  // (7.2 us against 8.7 us at M=256, N=K=2048; with more workgroups per CU the smaller step wins).
-  if (tile == 1 && count(1) <= 384 && Kb >= 2048) tile = 10;
-  const int64_t steps = (Kb + kStepBytes - 1) / kStepBytes;
-  int splits = 1;
-  // Long-K products whose tiles cannot fill the chip (the SwiGLU down projection at decode batch sizes): a workgroup's
-  // K loop is a serial chain of a few hundred ns per step, so four shorter chains on 64x64 tiles plus the reduce
-  // launch beat one long chain (13.3 us against 18.3 us at M=256, N=2048, K=5632 with weights streaming from HBM).
-  if (steps >= 32 && M > 64 && count(2) <= 256) {
-    tile = 2;
-    while (count(tile) * splits < 512 && splits < 4 && steps / (splits * 2) >= 8) splits *= 2;
-  }
-  return {tile, splits};
+  else if (M <= 64) tile = 2;
+  else if (count(6) >= 256) tile = 14;               // 128x128, ring of 2
+  else if (count(2) >= 512) tile = 13;               // 64x64, ring of 3
+  else if (count(1) > 384) tile = 15;                // 32x64, 256-byte steps, ring of 2
+  else if (count(1) > 256) tile = 16;                // 64x64, ring of 4
+  else tile = steps >= 32 ? 17 : 12;                 // 32x64, ring of 5 (long K) or 4
+  return {tile, 1};
 }
 
-template <int EB, int BM, int BN, int WM, int WN, int SW, int KS>
+template <int EB, int BM, int BN, int WM, int WN, int SW, int KS, int ST = 0>
 void launch_tile(void* out, float* partial, const uint8_t* A, const uint8_t* W, const float* as, const float* ws, int M,
                  int N, int64_t Kb, int splits, int out_dtype, bool keep_partials, hipStream_t s) {
   const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
@@ -320,7 +367,7 @@ void launch_tile(void* out, float* partial, const uint8_t* A, const uint8_t* W, 
   const int per = (int)((steps + splits - 1) / splits);
   const dim3 grid((tiles + 7) / 8 * 8, splits), block(WM * WN * 64);
   if (Kb % KS == 0)
-    hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN, SW, KS, false>), grid, block, 0, s, out, (splits > 1 || keep_partials) ? partial : nullptr, A, W,
+    hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN, SW, KS, false, ST>), grid, block, 0, s, out, (splits > 1 || keep_partials) ? partial : nullptr, A, W,
                        as, ws, M, N, Kb, per, out_dtype);
   else
     hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN, SW, KS, true>), grid, block, 0, s, out, (splits > 1 || keep_partials) ? partial : nullptr, A, W,
@@ -354,8 +401,8 @@ int gemm_entry(const char* name, void* out, const void* a, const float* as, cons
   while (plan.splits > 1 && (steps + plan.splits - 1) / plan.splits * (plan.splits - 1) >= steps) --plan.splits;
   LFM2_REQUIRE(plan.splits == 1 || workspace != nullptr, "%s: split-K needs a workspace", name);
   LFM2_REQUIRE(reduce || workspace != nullptr, "%s: partial products need a destination", name);
-#define TILE_(ID, BM, BN, WM, WN, KS) \
-  case ID: launch_tile<EB, BM, BN, WM, WN, EB == 1 ? 1 : 0, KS>(out, workspace, A, W, as, ws, (int)M, (int)N, Kb, plan.splits, out_dtype, !reduce, s); break
+#define TILE_(ID, BM, BN, WM, WN, KS, ...) \
+  case ID: launch_tile<EB, BM, BN, WM, WN, EB == 1 ? 1 : 0, KS, ##__VA_ARGS__>(out, workspace, A, W, as, ws, (int)M, (int)N, Kb, plan.splits, out_dtype, !reduce, s); break
   switch (plan.tile) {
     TILE_(0, 16, 64, 1, 4, 128);
     TILE_(1, 32, 64, 2, 2, 128);
@@ -369,6 +416,17 @@ int gemm_entry(const char* name, void* out, const void* a, const float* as, cons
     TILE_(9, 16, 64, 1, 4, 256);
     TILE_(10, 32, 64, 2, 2, 256);
     TILE_(11, 64, 64, 2, 2, 256);
+    TILE_(12, 32, 64, 2, 2, 128, 4);
+    TILE_(13, 64, 64, 2, 2, 128, 3);
+    TILE_(14, 128, 128, 2, 4, 128, 2);
+    TILE_(15, 32, 64, 2, 2, 256, 2);
+    TILE_(16, 64, 64, 2, 2, 128, 4);
+    TILE_(17, 32, 64, 2, 2, 128, 5);
+    TILE_(18, 16, 64, 1, 4, 256, 3);
+    TILE_(19, 128, 64, 4, 2, 128, 2);
+    TILE_(20, 64, 128, 2, 4, 128, 2);
+    TILE_(21, 16, 64, 1, 4, 128, 4);
+    TILE_(22, 128, 64, 2, 2, 128, 2);
   }
 #undef TILE_
   if (plan.splits > 1 && reduce)

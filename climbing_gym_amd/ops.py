@@ -238,17 +238,17 @@ class PackedFP8Weight:
 
     def linear_quantized(self, x, scales, *, dtype=torch.bfloat16, config=None, defer_reduce=False):
         """config = (tile index, split_k) overrides the default tile choice.  With `defer_reduce`, a product the
-        default plan splits along K comes back as a `SplitProduct` for `rms_norm_fp8` to reduce."""
+        plan (default or `config`) splits along K comes back as a `SplitProduct` for `rms_norm_fp8` to reduce."""
         batch, width = x.shape
         rows = self.values.size(0)
         if width != self.values.size(1):
             raise ValueError("FP8 activation and weight widths differ")
         tile, split_k = (-1, 0) if config is None else (int(config[0]), int(config[1]) if len(config) > 1 else 0)
-        if defer_reduce and config is None:
-            splits = query("lfm2_fp8_gemm_default_splits", batch, rows, width)
+        if defer_reduce:
+            splits = query("lfm2_fp8_gemm_default_splits", batch, rows, width) if split_k == 0 else split_k
             if splits > 1:
                 partials = torch.empty((splits, batch, rows), device=x.device, dtype=torch.float32)
-                call("lfm2_fp8_gemm_partials", partials, x, self.values, batch, rows, width, -1, splits)
+                call("lfm2_fp8_gemm_partials", partials, x, self.values, batch, rows, width, tile, splits)
                 return SplitProduct(partials, scales, self.scales, dtype)
         out = torch.empty((batch, rows), device=x.device, dtype=dtype)
         need = query("lfm2_fp8_gemm_workspace", batch, rows, width) if split_k == 0 else max(split_k, 1) * batch * rows
