@@ -6,19 +6,23 @@ Reference module -> module of this package:
   inference/lfm25_cuda_kernels.py, lfm25_fp8.py, lfm25_fp8_kv.py, lfm25_batching.py, lfm25_sampling.py -> ops.py
   inference/lfm25_session.py       -> session.py
   inference/text_stops.py          -> text_stops.py
+  inference/lfm25_async_engine.py  -> async_engine.py;  inference/config.py, types.py -> inference_config.py, types.py
 """
 from .config import LFM2Config, LFM25SamplingConfig
 
 __all__ = ["LFM2Config", "LFM25SamplingConfig", "LFM25Engine", "LFM25PackedWeights", "LFM25HybridCache",
            "LFM25PrefixBatch", "LFM25DecodeBatch", "LFM25StepOutput", "LFM25GenerationOutput", "LFM25HIPDecoder",
            "LFM25CUDADecoder", "LFM25GenerationSession", "LFM25ContinuationHandle", "LFM25SessionResult",
-           "flatten_token_batches"]
+           "flatten_token_batches", "LFM25AsyncInferenceEngine", "SamplingConfig", "InferenceEngineConfig",
+           "GenerationOutput", "GenerationResult"]
 
 _LAZY = {
     "LFM25Engine": "engine", "LFM25PrefixBatch": "engine", "LFM25DecodeBatch": "engine", "LFM25StepOutput": "engine",
     "LFM25GenerationOutput": "engine", "flatten_token_batches": "engine", "LFM25PackedWeights": "weights",
     "LFM25HybridCache": "cache", "LFM25HIPDecoder": "decoder", "LFM25CUDADecoder": "decoder",
     "LFM25GenerationSession": "session", "LFM25ContinuationHandle": "session", "LFM25SessionResult": "session",
+    "LFM25AsyncInferenceEngine": "async_engine", "SamplingConfig": "inference_config",
+    "InferenceEngineConfig": "inference_config", "GenerationOutput": "types", "GenerationResult": "types",
 }
 
 

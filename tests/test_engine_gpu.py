@@ -527,3 +527,53 @@ def test_tiny_model_greedy_tokens_against_the_committed_vectors():
         pinned += horizon
     print(f"{pinned} of 256 greedy ids pinned by the golden vectors")
     assert pinned >= 128
+
+
+class _ByteTokenizer:
+    """Latin-1 bytes as token ids: enough text plumbing for the adapter on a 257-entry vocabulary."""
+
+    def __len__(self):
+        return 256
+
+    def encode(self, text, add_special_tokens=False):
+        return list(text.encode("latin-1"))
+
+    def decode(self, ids, skip_special_tokens=False, clean_up_tokenization_spaces=False):
+        return bytes(int(i) % 256 for i in ids).decode("latin-1")
+
+
+@torch.inference_mode()
+def test_async_adapter_runs_batches_and_chains_on_the_hip_engine():
+    """generate_many gives what a direct engine.generate of the same prompts gives; a two-phase chain whose second
+    prompt extends the first completion resumes from the cache and continues the greedy sequence a single longer
+    request produces (lfm25_async_engine.py:235-409)."""
+    import asyncio
+    from climbing_gym_amd.async_engine import LFM25AsyncInferenceEngine
+    from climbing_gym_amd.inference_config import InferenceEngineConfig, SamplingConfig
+    engine, _, _ = _engine()
+    engine.enable_cuda_graphs(max_graphs=2)
+    adapter = LFM25AsyncInferenceEngine.from_components(engine=engine, tokenizer=_ByteTokenizer(),
+                                                        config=InferenceEngineConfig(model_path="", seed=3), max_batch_size=8)
+    greedy = SamplingConfig(temperature=0.0, max_tokens=12, logprobs=1, extra_params={"ignore_eos": True})
+    prompts = ["hello world", "abc", "the quick brown fox"]
+    results = asyncio.run(adapter.generate_many(prompts, sampling=greedy))
+    direct = engine.generate(*_flat([list(p.encode("latin-1")) for p in prompts]), repeats=1,
+                             sampling=LFM25SamplingConfig(temperature=0.0, max_new_tokens=12, ignore_eos=True))
+    for row, result in enumerate(results):
+        assert result.token_ids == tuple(direct.token_ids[row, 0].cpu().tolist())
+        assert result.outputs[0].finish_reason == "length" and len(result.completion_logprobs) == 12
+        assert result.text == _ByteTokenizer().decode(result.token_ids)
+
+    half = SamplingConfig(temperature=0.0, max_tokens=6, extra_params={"ignore_eos": True})
+
+    def on_result(index, result):
+        if result.request_id.endswith("phase-0"):
+            return (list(result.prompt_token_ids + result.token_ids), half)
+        return None
+    chains = asyncio.run(adapter.generate_chains([(p, half) for p in prompts], on_result=on_result, max_new_tokens=16))
+    for row, phases in enumerate(chains):
+        assert len(phases) == 2
+        assert phases[0].token_ids + phases[1].token_ids == results[row].token_ids
+    assert adapter.last_session_stats["admitted_requests"] == 3
+    adapter.close()
+    engine.disable_cuda_graphs()
