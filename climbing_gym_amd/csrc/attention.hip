@@ -292,6 +292,7 @@ __global__ void __launch_bounds__(256) decode_attn_mfma_kernel(DecodeArgs a) {
   __shared__ __bf16 lds_p[4][4][64];
   __shared__ float sm[4][4], sl[4][4], sacc[4][4][D];
   const int items = a.schedule[0] * a.KH;
+  if (items <= 0) return;
   // An item's row, chunk, length and slot sit behind three dependent loads; the next item's are fetched while the
   // current one is processed so that chain is off the critical path of every item but a workgroup's first.
   struct Meta { int b, chunk, len; int64_t slot; };
