@@ -8,6 +8,7 @@ looks at the `alive` flags only every `finish_check_interval` steps.
 """
 from __future__ import annotations
 
+import gc
 from collections import OrderedDict
 from dataclasses import dataclass, field
 
@@ -135,8 +136,17 @@ class LFM25HIPDecoder:
         current.wait_stream(stream)
         torch.cuda.synchronize(device)
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=stream):
-            step()
+        # torch.cuda.graph collects garbage before the capture begins; the cyclic collector must not run again until
+        # it ends: finalising an unreachable graph or stream of an earlier engine while this stream is capturing
+        # aborts the process
+        collector_was_on = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph, stream=stream):
+                step()
+        finally:
+            if collector_was_on:
+                gc.enable()
         current.wait_stream(stream)
         return graph
 
