@@ -1,4 +1,4 @@
-// On-GPU sampling and scheduler bookkeeping: greedy / Gumbel-max categorical sampling with raw
+// On-GPU sampling and scheduler bookkeeping: greedy / categorical sampling with raw
 // log-probabilities, temperature + top-k + nucleus sampling, the per-row record step of a
 // generation session (stop automaton, finish codes, RNG positions) and the slot gather/scatter
 // used by compact decode batches.  Nothing here synchronises with the host.
@@ -17,6 +17,7 @@ namespace {
 constexpr uint64_t kGolden = 0x9E3779B97F4A7C15ull;
 constexpr uint64_t kMask63 = 0x7FFFFFFFFFFFFFFFull;
 constexpr int kTile = 4096;
+constexpr int kNoIndex = 0x7fffffff;
 
 // Philox4x32-10 (Salmon et al. 2011): 128-bit counter, 64-bit key -> four 32-bit words.
 __device__ __forceinline__ void philox(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1,
@@ -42,113 +43,214 @@ __device__ __forceinline__ uint64_t row_key(int64_t seed, int64_t step) {
 }
 
 // ------------------------------------------------------------------------------------ full-support sampler
-// Pass 1: one workgroup per (row, 4096-column tile): best Gumbel score with its first index, and
-// the tile's (max, sum exp) of the raw logits.  scratch[(row*parts+part)*4 + {score,index,max,sum}].
+// Greedy rows take the first maximum.  Rows with a temperature draw from softmax(logits / T) by inverting the
+// cumulative distribution with ONE uniform number per row (Philox keyed by the row's seed and step): the same
+// categorical law as the reference's Gumbel-max (lfm25_sampling.py:9-58) without a random number, two logarithms and
+// ten rounds of 32-bit multiplies per logit, which made the sampler compute-bound (30 us at 256 x 65536; the logits
+// themselves stream in 8 us).  Exact draws were never comparable with the reference (its generator is Triton's);
+// the distribution and the determinism in (seed, step) are what the tests hold.
+//
+// Pass 1: one workgroup per (row, 4096-column tile): the tile's maximum, sum exp(x - max) of the raw logits (for
+// the log-probability) and of the tempered ones (the tile's probability mass).  About eight vector instructions per
+// logit: with 16.8 M logits a step the arithmetic, not the 33 MB of traffic, is what the pass costs, hence the
+// hardware exp2 with the scale folded into one multiply-add, and no second exponential at temperature 0 or 1.
+// scratch[(row*parts+part)*4 + {tempered sum, unused, max, raw sum}].
+constexpr float kLog2e = 1.4426950408889634f;
+struct TileStat { float max, sum, mass; };
+// Joins two partial softmax states (online normaliser, Milakov & Gimelshein 2018).
+__device__ __forceinline__ TileStat join(const TileStat& a, const TileStat& b, float inv_temp) {
+  TileStat r;
+  r.max = fmaxf(a.max, b.max);
+  const float da = a.max == r.max ? 0.f : a.max - r.max, db = b.max == r.max ? 0.f : b.max - r.max;  // no inf - inf
+  r.sum = a.sum * __expf(da) + b.sum * __expf(db);
+  r.mass = a.mass * __expf(da * inv_temp) + b.mass * __expf(db * inv_temp);
+  return r;
+}
+// 16 bytes of consecutive columns, one load when the row stride allows it; columns beyond V read as -inf.
 template <typename T>
-__global__ void __launch_bounds__(256)
-sample_partial_kernel(const T* logits, float* scratch, const int64_t* seeds, const int64_t* steps,
-                      const float* temperatures, int64_t seed, int64_t step, float temperature, int64_t V, int parts) {
-  __shared__ float s_score[4], s_max[4], s_sum[4];
-  __shared__ int s_index[4];
-  const int64_t row = blockIdx.y;
-  const int part = blockIdx.x;
-  const bool per_row = seeds != nullptr;
-  const float temp = per_row ? temperatures[row] : temperature;
-  const uint64_t key = per_row ? row_key(seeds[row], steps[row]) : row_key(seed, step);
-  const T* src = logits + row * V;
-  float best = -INFINITY, tmax = -INFINITY;
-  int best_i = 0x7fffffff;
-  float vals[16];
-  const float inv_temp = 1.0f / fmaxf(temp, 1.0e-30f);
-  typedef T vec4 __attribute__((ext_vector_type(4)));
-  const bool vector_ok = (V & 3) == 0;
+__device__ __forceinline__ void load_columns(const T* src, int64_t col0, int64_t V, bool vector_ok, float* out) {
+  constexpr int EPL = 16 / sizeof(T);
+  typedef T vec __attribute__((ext_vector_type(EPL)));
+  if (vector_ok && col0 < V) {
+    const vec v = *reinterpret_cast<const vec*>(src + col0);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int64_t col0 = (int64_t)part * kTile + (i * 256 + threadIdx.x) * 4;
-    uint32_t rnd[4] = {0, 0, 0, 0};
-    if (temp > 0.f && col0 < V) {
-      // per-row streams count columns; the shared stream counts flattened (row, column) like the reference
-      const uint64_t ctr = per_row ? (uint64_t)(col0 >> 2) : (uint64_t)((row * V + col0) >> 2);
-      philox((uint32_t)ctr, (uint32_t)(ctr >> 32), per_row ? 0u : (uint32_t)((row * V + col0) & 3), 0u, (uint32_t)key,
-             (uint32_t)(key >> 32), rnd);
-    }
-    float x4[4];
-    if (vector_ok && col0 < V) {
-      const vec4 v = *reinterpret_cast<const vec4*>(src + col0);
+    for (int e = 0; e < EPL; ++e) out[e] = Elem<T>::load(v[e]);
+  } else {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) x4[e] = Elem<T>::load(v[e]);
-    } else {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) x4[e] = col0 + e < V ? Elem<T>::load(src[col0 + e]) : -INFINITY;
-    }
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int64_t col = col0 + e;
-      const float x = x4[e];
-      vals[i * 4 + e] = x;
-      tmax = fmaxf(tmax, x);
-      float score = x;
-      if (temp > 0.f) score = x * inv_temp + gumbel(rnd[e]);
-      if (col < V && (score > best || best_i == 0x7fffffff)) { best = score; best_i = (int)col; }
-    }
-  }
-  // wave then block arg-max (ties -> lowest column) and max
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    const float ob = __shfl_xor(best, o, 64);
-    const int oi = __shfl_xor(best_i, o, 64);
-    if (oi != 0x7fffffff && (best_i == 0x7fffffff || ob > best || (ob == best && oi < best_i))) { best = ob; best_i = oi; }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, o, 64));
-  }
-  if (lane == 0) { s_score[wave] = best; s_index[wave] = best_i; s_max[wave] = tmax; }
-  __syncthreads();
-  float bmax = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
-  const float shift = bmax == -INFINITY ? 0.f : bmax;
-  float sum = 0.f;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) sum += __expf(vals[i] - shift);
-  sum = wave_sum(sum);
-  if (lane == 0) s_sum[wave] = sum;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    float b = s_score[0];
-    int bi = s_index[0];
-    for (int w = 1; w < 4; ++w)
-      if (s_index[w] != 0x7fffffff && (bi == 0x7fffffff || s_score[w] > b || (s_score[w] == b && s_index[w] < bi))) { b = s_score[w]; bi = s_index[w]; }
-    float* dst = scratch + (row * parts + part) * 4;
-    dst[0] = b; dst[1] = __int_as_float(bi); dst[2] = bmax; dst[3] = (s_sum[0] + s_sum[1]) + (s_sum[2] + s_sum[3]);
+    for (int e = 0; e < EPL; ++e) out[e] = col0 + e < V ? Elem<T>::load(src[col0 + e]) : -INFINITY;
   }
 }
 
-// Pass 2: merge the tiles of a row.
 template <typename T>
-__global__ void __launch_bounds__(64)
-sample_finish_kernel(const T* logits, const float* scratch, int64_t* tokens, float* logprobs, int64_t V, int parts) {
-  const int64_t row = blockIdx.x;
-  const float* src = scratch + row * parts * 4;
-  float best = -INFINITY, mx = -INFINITY;
-  int bi = 0x7fffffff;
-  for (int p = threadIdx.x; p < parts; p += 64) {
-    const float s = src[p * 4];
-    const int i = __float_as_int(src[p * 4 + 1]);
-    if (i != 0x7fffffff && (bi == 0x7fffffff || s > best || (s == best && i < bi))) { best = s; bi = i; }
-    mx = fmaxf(mx, src[p * 4 + 2]);
-  }
+__global__ void __launch_bounds__(256)
+sample_partial_kernel(const T* logits, float* scratch, const float* temperatures, float temperature, int64_t V, int parts) {
+  constexpr int EPL = 16 / sizeof(T), LOADS = 16 / EPL;
+  __shared__ TileStat s_stat[4];
+  const int64_t row = blockIdx.y;
+  const int part = blockIdx.x;
+  const float temp = temperatures ? temperatures[row] : temperature;
+  const float inv_temp = temp > 0.f ? 1.0f / temp : 0.f;
+  const T* src = logits + row * V;
+  const bool vector_ok = V % EPL == 0;
+  float vals[16];
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    const float ob = __shfl_xor(best, o, 64);
-    const int oi = __shfl_xor(bi, o, 64);
-    if (oi != 0x7fffffff && (bi == 0x7fffffff || ob > best || (ob == best && oi < bi))) { best = ob; bi = oi; }
-    mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+  for (int i = 0; i < LOADS; ++i)
+    load_columns(src, (int64_t)part * kTile + (i * 256 + threadIdx.x) * EPL, V, vector_ok, vals + i * EPL);
+  float top = vals[0];
+#pragma unroll
+  for (int i = 1; i < 16; ++i) top = fmaxf(top, vals[i]);
+  top = wave_max(top);
+  const float shift = top == -INFINITY ? 0.f : top;
+  TileStat mine{top, 0.f, 0.f};
+  const float bias = -shift * kLog2e;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) mine.sum += __builtin_amdgcn_exp2f(fmaf(vals[i], kLog2e, bias));
+  mine.sum = wave_sum(mine.sum);
+  if (inv_temp == 1.f || inv_temp == 0.f) {
+    mine.mass = mine.sum;   // greedy rows never read it
+  } else {
+    const float scale = kLog2e * inv_temp, tempered_bias = bias * inv_temp;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) mine.mass += __builtin_amdgcn_exp2f(fmaf(vals[i], scale, tempered_bias));
+    mine.mass = wave_sum(mine.mass);
   }
-  float total = 0.f;
-  for (int p = threadIdx.x; p < parts; p += 64) total += src[p * 4 + 3] * expf(src[p * 4 + 2] - mx);
-  total = wave_sum(total);
+  if ((threadIdx.x & 63) == 0) s_stat[threadIdx.x >> 6] = mine;
+  __syncthreads();
   if (threadIdx.x == 0) {
-    if (bi == 0x7fffffff) bi = 0;
-    tokens[row] = bi;
-    if (logprobs) logprobs[row] = Elem<T>::load(logits[row * V + bi]) - (mx + logf(total));
+    const TileStat t = join(join(s_stat[0], s_stat[1], inv_temp), join(s_stat[2], s_stat[3], inv_temp), inv_temp);
+    float4 packed;
+    packed.x = t.mass; packed.y = 0.f; packed.z = t.max; packed.w = t.sum;
+    *reinterpret_cast<float4*>(scratch + (row * parts + part) * 4) = packed;
+  }
+}
+
+// Pass 2, one workgroup per row: merge the tiles, then read one tile again.  Greedy rows take the first column
+// that holds the maximum, in the first tile that has it.  The others pick the tile and then the column where the
+// cumulative mass passes u * total (tiles and columns in index order; the last column with mass if rounding pushes
+// the target past the end).  At most 256 tiles (a vocabulary of 2^20).
+template <typename T>
+__global__ void __launch_bounds__(256)
+sample_finish_kernel(const T* logits, const float* scratch, int64_t* tokens, float* logprobs, const int64_t* seeds,
+                     const int64_t* steps, const float* temperatures, int64_t seed, int64_t step, float temperature,
+                     int64_t V, int parts) {
+  __shared__ TileStat s_stat[4];
+  __shared__ float s_tile_mass[256];
+  __shared__ float s_wave[4];
+  __shared__ float s_target;
+  __shared__ double s_uniform;
+  __shared__ int s_tile, s_pick;
+  const int64_t row = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const bool per_row = seeds != nullptr;
+  const float temp = per_row ? temperatures[row] : temperature;
+  const float inv_temp = temp > 0.f ? 1.0f / temp : 0.f;
+  TileStat own{-INFINITY, 0.f, 0.f};
+  if (threadIdx.x < parts) {
+    const float4 packed = *reinterpret_cast<const float4*>(scratch + (row * parts + threadIdx.x) * 4);
+    own.mass = packed.x; own.max = packed.z; own.sum = packed.w;
+  }
+  if (threadIdx.x == 255) {  // a thread with no tile of its own draws the row's uniform number meanwhile
+    const uint64_t key = per_row ? row_key(seeds[row], steps[row]) : row_key(seed, step);
+    uint32_t rnd[4];
+    // per-row streams use counter 0; the shared stream counts rows
+    philox(per_row ? 0u : (uint32_t)row, per_row ? 0u : (uint32_t)(row >> 32), 0u, 0u, (uint32_t)key, (uint32_t)(key >> 32), rnd);
+    s_uniform = (double)((((uint64_t)rnd[0] << 32) | rnd[1]) >> 11) * (1.0 / 9007199254740992.0);
+    s_pick = kNoIndex;
+  }
+  const float wave_top = wave_max(own.max);
+  if (lane == 0) s_wave[wave] = wave_top;
+  __syncthreads();
+  const float mx = fmaxf(fmaxf(s_wave[0], s_wave[1]), fmaxf(s_wave[2], s_wave[3]));
+  const float gap = own.max == mx ? 0.f : own.max - mx;
+  float total = own.sum * __expf(gap);
+  if (threadIdx.x < parts) s_tile_mass[threadIdx.x] = temp > 0.f ? own.mass * __expf(gap * inv_temp) : (own.max == mx ? 1.f : 0.f);
+  total = wave_sum(total);
+  if (lane == 0) s_stat[wave].sum = total;
+  __syncthreads();
+  total = (s_stat[0].sum + s_stat[1].sum) + (s_stat[2].sum + s_stat[3].sum);
+  if (threadIdx.x == 0) {
+    int tile = 0;
+    float inside = 0.f;
+    if (temp > 0.f) {
+      // 53 uniform bits and double sums across tiles: the resolution inside the chosen tile is then relative to
+      // that tile's mass, not to the whole row's
+      double z = 0.0;
+      for (int p = 0; p < parts; ++p) z += (double)s_tile_mass[p];
+      const double target = s_uniform * z;
+      double before = 0.0;
+      for (int p = 0; p < parts; ++p) {
+        const double m = (double)s_tile_mass[p];
+        if (m > 0.0) tile = p;                   // last tile with mass, in case rounding overshoots
+        if (target < before + m) break;
+        before += m;
+      }
+      inside = (float)(target - before);
+    } else {
+      while (tile < parts - 1 && s_tile_mass[tile] == 0.f) ++tile;   // first tile that holds the maximum
+    }
+    s_tile = tile;
+    s_target = inside;
+  }
+  __syncthreads();
+  const int tile = s_tile;
+  const float target = s_target;
+  // the tile again: each thread owns 16 consecutive columns, so column order = thread order
+  constexpr int EPL = 16 / sizeof(T), LOADS = 16 / EPL;
+  const int64_t col0 = (int64_t)tile * kTile + threadIdx.x * 16;
+  const bool vector_ok = V % EPL == 0;
+  float x[16];
+#pragma unroll
+  for (int i = 0; i < LOADS; ++i) load_columns(logits + row * V, col0 + i * EPL, V, vector_ok, x + i * EPL);
+  int pick = kNoIndex, last = -1;
+  if (temp > 0.f) {
+    float e[16], sum = 0.f;
+    const float scale = kLog2e * inv_temp, bias = -mx * scale;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      e[i] = __builtin_amdgcn_exp2f(fmaf(x[i], scale, bias));   // -inf beyond V and for masked columns: 0
+      sum += e[i];
+    }
+    // exclusive prefix of the threads' sums: wave scan, then the earlier waves' totals
+    float incl = sum;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const float v = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += v;
+    }
+    if (lane == 63) s_wave[wave] = incl;
+    __syncthreads();
+    float run = incl - sum;
+    for (int w = 0; w < wave; ++w) run += s_wave[w];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      if (e[i] > 0.f) {
+        last = (int)(col0 + i);
+        if (pick == kNoIndex && target < run + e[i]) pick = last;
+      }
+      run += e[i];
+    }
+  } else {
+#pragma unroll
+    for (int i = 15; i >= 0; --i)
+      if (x[i] == mx && col0 + i < V) pick = (int)(col0 + i);
+  }
+  if (pick != kNoIndex) atomicMin(&s_pick, pick);
+  __syncthreads();
+  if (s_pick == kNoIndex) {  // the target lies past the tile's recomputed mass: the last column with mass
+    __syncthreads();
+    if (threadIdx.x == 0) s_pick = -1;
+    __syncthreads();
+    if (last >= 0) atomicMax(&s_pick, last);
+    __syncthreads();
+  }
+  const int token = s_pick < 0 ? (int)((int64_t)tile * kTile) : s_pick;   // nothing comparable (NaN row): the tile's first column
+  // the thread that holds the chosen column writes the row's result
+  if (token >= col0 && token < col0 + 16) {
+    tokens[row] = token;
+    float chosen = x[0];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) chosen = token - col0 == i ? x[i] : chosen;
+    if (logprobs) logprobs[row] = chosen - (mx + logf(total));
   }
 }
 
@@ -450,13 +552,14 @@ extern "C" int lfm2_sample(int64_t* tokens, float* logprobs, const void* logits,
   LFM2_REQUIRE(temperature >= 0.f, "sample: negative temperature");
   LFM2_REQUIRE((seeds == nullptr) == (steps == nullptr) && (seeds == nullptr) == (temperatures == nullptr),
                "sample: seeds, steps and temperatures go together");
+  LFM2_REQUIRE(V <= 256ll * kTile, "sample: vocabulary above 1048576");
   const int parts = ceil_div(V, kTile);
   hipStream_t s = (hipStream_t)stream;
   DISPATCH_DTYPE(dtype, "sample",
-                 hipLaunchKernelGGL(sample_partial_kernel<T>, dim3(parts, B), dim3(256), 0, s, (const T*)logits, scratch, seeds,
-                                    steps, temperatures, seed, step, temperature, V, parts);
-                 hipLaunchKernelGGL(sample_finish_kernel<T>, dim3(B), dim3(64), 0, s, (const T*)logits, scratch, tokens,
-                                    logprobs, V, parts));
+                 hipLaunchKernelGGL(sample_partial_kernel<T>, dim3(parts, B), dim3(256), 0, s, (const T*)logits, scratch,
+                                    temperatures, temperature, V, parts);
+                 hipLaunchKernelGGL(sample_finish_kernel<T>, dim3(B), dim3(256), 0, s, (const T*)logits, scratch, tokens,
+                                    logprobs, seeds, steps, temperatures, seed, step, temperature, V, parts));
   LFM2_LAUNCH_CHECK();
 }
 

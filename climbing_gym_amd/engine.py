@@ -429,7 +429,7 @@ class LFM25Engine:
 
     # ------------------------------------------------------------------ sampling helpers
     def _sample(self, logits, sampling: LFM25SamplingConfig, *, step: int, seen_token_mask=None):
-        """Greedy, full-support Gumbel-max, or temperature/top-k/top-p on the device; log-probabilities are the raw
+        """Greedy, a full-support categorical draw, or temperature/top-k/top-p on the device; log-probabilities are the raw
         log-softmax of the draw (lfm25_engine.py:1574-1609).  A repetition penalty is applied to an fp32 copy first."""
         if seen_token_mask is not None and sampling.repetition_penalty != 1.0:
             lf = logits.float()

@@ -376,8 +376,10 @@ def _sample_scratch(batch: int, vocab: int, device):
 
 
 def sample_logits(logits: torch.Tensor, *, temperature: float, seed: int, step: int, return_logprobs: bool):
-    """lfm25_sampling.py:61-92: greedy (first maximum) or Gumbel-max over the full support; log-probabilities
-    are the raw log-softmax of the chosen token.  Deterministic in (seed, step)."""
+    """lfm25_sampling.py:61-92: greedy (first maximum) or a categorical draw from softmax(logits / T) over the
+    full support (one uniform number per row through the inverse cumulative distribution: the same law as the
+    reference's Gumbel-max); log-probabilities are the raw log-softmax of the chosen token.  Deterministic in
+    (seed, step)."""
     if logits.ndim != 2 or not logits.is_cuda or logits.dtype not in (torch.bfloat16, torch.float16, torch.float32):
         raise ValueError("sampling requires a 2D CUDA BF16/FP16/FP32 logits tensor")
     logits = logits.contiguous()

@@ -202,7 +202,8 @@ int lfm2_advance_positions(int32_t* lengths, const int32_t* positions, const int
 /* ---------------------------------------------------------------- sampling and bookkeeping */
 
 /* sample_logits / RowSampler.sample of lfm25_sampling.py:9-123: greedy (temperature 0: first
- * maximum) or Gumbel-max over the full support; logprobs are raw log-softmax of the pick.
+ * maximum) or a draw from softmax(logits / T) over the full support (inverse CDF, one uniform per row;
+ * the same law as the reference's Gumbel-max, V <= 2^20); logprobs are raw log-softmax of the pick.
  * Per-row arrays (seeds int64, steps int64, temperatures float) may be NULL, then the scalar
  * seed/step/temperature apply.  scratch: float[B*parts*4] with parts = ceil(V/4096). */
 int lfm2_sample(int64_t* tokens, float* logprobs, const void* logits, float* scratch, const int64_t* seeds,
