@@ -33,6 +33,8 @@ _SIGNATURES = {
     "lfm2_conv_prefill": "ppppppp" "llllip",
     "lfm2_fp8_gemm": "pppppp" "llliiip",
     "lfm2_bf16_gemm": "pppp" "llliip",
+    "lfm2_fp8_gemm_rows": "ppppppp" "lllliip",
+    "lfm2_bf16_gemm_rows": "ppppp" "llllip",
     "lfm2_store_kv_fp8": "ppppppppp" "lliilllllllllip",
     "lfm2_append_kv": "ppppppp" "liilllip",
     "lfm2_store_kv_packed": "ppppppppp" "liillliip",

@@ -61,6 +61,16 @@ template <> struct StepMfma<2> {
   }
 };
 
+// Optional placement of output rows: row m goes to out row slots[m] (m when slots is null); rows whose slot is
+// negative, not below `capacity` (the rows `out` holds), or whose `active` byte is 0 are not written.  This is the
+// scatter of lfm25_batching.py:25-32 done by the producing GEMM instead of by a copy of the logits.
+struct RowMap { const int32_t* slots; const uint8_t* active; int capacity; };
+__device__ __forceinline__ int mapped_row(const RowMap& rows, int m) {
+  if (rows.active && !rows.active[m]) return -1;
+  const int slot = rows.slots ? rows.slots[m] : m;
+  return slot < rows.capacity ? slot : -1;
+}
+
 __device__ __forceinline__ void store_out(void* out, int out_dtype, int64_t idx, float v) {
   if (out_dtype == LFM2_DTYPE_BF16) ((__bf16*)out)[idx] = (__bf16)v;
   else if (out_dtype == LFM2_DTYPE_F16) ((_Float16*)out)[idx] = (_Float16)v;
@@ -71,7 +81,7 @@ template <int EB, int BM, int BN, int WM, int WN, int SW, int KS, bool KTAIL, in
 __global__ void __launch_bounds__(WM * WN * 64)
 gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_t* __restrict__ A,
                const uint8_t* __restrict__ W, const float* __restrict__ a_scales, const float* __restrict__ w_scales,
-               int M, int N, int64_t Kb, int steps_per_split, int out_dtype) {
+               int M, int N, int64_t Kb, int steps_per_split, int out_dtype, RowMap rows) {
   constexpr int NT = WM * WN * 64;
   constexpr int TM = BM / WM, TN = BN / WN, MI = TM / 16, NI = TN / 16;
   constexpr int kChunksPerRow = KS / 16;  // KS = K bytes staged per step and row: 128, or 256 (two MFMA sub-steps per barrier)
@@ -214,8 +224,10 @@ gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_
         }
       }
     };
-    // loads complete in order: with ST-1 steps in flight, step s has landed once at most ST-2 steps' loads remain
-    constexpr int kPending = (ST - 2) * (A_PER + W_PER);
+    // loads complete in order: with ST-1 steps in flight, step s has landed once at most ST-2 steps' loads remain.
+    // Each wave counts its own loads, and when a tile has fewer chunks than threads the last waves issue fewer per
+    // step (only the full passes): the bound uses that smallest count, which is merely stricter for the others.
+    constexpr int kPending = (ST - 2) * (A_CHUNKS / NT + W_CHUNKS / NT);
     constexpr int kWait = (kPending & 0xF) | (0x7 << 4) | (0xF << 8) | ((kPending >> 4) << 14);  // vmcnt only
 #pragma unroll
     for (int st = 0; st < ST - 1; ++st) issue(st, st);
@@ -258,10 +270,10 @@ gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_
 
   // Epilogue: lane holds out[m = .. + lrow][n = .. + 4*lgrp + r], r = 0..3.
   const bool split = partial != nullptr;
-  auto finish = [&](f32x4 v, int m, int n, float sa) {  // scale (row then column) and store up to 4 columns
+  auto finish = [&](f32x4 v, int m_out, int n, float sa) {  // scale (row then column) and store up to 4 columns
     if (a_scales)
       for (int r = 0; r < 4; ++r) v[r] = (v[r] * sa) * (n + r < N ? w_scales[n + r] : 0.f);
-    const int64_t idx = (int64_t)m * N + n;
+    const int64_t idx = (int64_t)m_out * N + n;
     if (out_dtype == LFM2_DTYPE_BF16 && n + 3 < N && (N & 3) == 0) {
       bf16x4 o = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
       *reinterpret_cast<bf16x4*>((__bf16*)out + idx) = o;
@@ -273,6 +285,8 @@ gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_
   for (int i = 0; i < MI; ++i) {
     const int m = m_base + wm * TM + i * 16 + lrow;
     if (m >= M) continue;
+    const int m_out = split ? m : mapped_row(rows, m);
+    if (m_out < 0) continue;
     const float sa = (!split && a_scales) ? a_scales[m] : 1.0f;
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
@@ -283,7 +297,7 @@ gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_
         if (n + 3 < N && (N & 3) == 0) *reinterpret_cast<f32x4*>(dst) = acc[i][j];
         else for (int r = 0; r < 4 && n + r < N; ++r) dst[r] = acc[i][j][r];
       } else {
-        finish(acc[i][j], m, n, sa);
+        finish(acc[i][j], m_out, n, sa);
       }
     }
   }
@@ -308,10 +322,12 @@ reduce_split_kernel(void* out, const float* partial, const float* a_scales, cons
 template <int EB>
 __global__ void __launch_bounds__(256)
 gemm_naive_kernel(void* out, const uint8_t* A, const uint8_t* W, const float* a_scales, const float* w_scales, int64_t M,
-                  int64_t N, int64_t K, int out_dtype) {
+                  int64_t N, int64_t K, int out_dtype, RowMap rows) {
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= M * N) return;
   const int64_t m = idx / N, n = idx % N;
+  const int m_out = mapped_row(rows, (int)m);
+  if (m_out < 0) return;
   float t = 0.f;
   if (EB == 1) {
     const uint8_t *a = A + m * K, *w = W + n * K;
@@ -324,7 +340,7 @@ gemm_naive_kernel(void* out, const uint8_t* A, const uint8_t* W, const float* a_
     for (int64_t k = 0; k < K; ++k) t = fmaf((float)a[k], (float)w[k], t);
   }
   if (a_scales) t = (t * a_scales[m]) * w_scales[n];
-  store_out(out, out_dtype, idx, t);
+  store_out(out, out_dtype, (int64_t)m_out * N + n, t);
 }
 
 struct TileInfo { int bm, bn, ks; };
@@ -361,23 +377,23 @@ Plan default_plan(int64_t M, int64_t N, int64_t Kb) {
 
 template <int EB, int BM, int BN, int WM, int WN, int SW, int KS, int ST = 0>
 void launch_tile(void* out, float* partial, const uint8_t* A, const uint8_t* W, const float* as, const float* ws, int M,
-                 int N, int64_t Kb, int splits, int out_dtype, bool keep_partials, hipStream_t s) {
+                 int N, int64_t Kb, int splits, int out_dtype, bool keep_partials, RowMap rows, hipStream_t s) {
   const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   const int64_t steps = (Kb + KS - 1) / KS;
   const int per = (int)((steps + splits - 1) / splits);
   const dim3 grid((tiles + 7) / 8 * 8, splits), block(WM * WN * 64);
   if (Kb % KS == 0)
     hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN, SW, KS, false, ST>), grid, block, 0, s, out, (splits > 1 || keep_partials) ? partial : nullptr, A, W,
-                       as, ws, M, N, Kb, per, out_dtype);
+                       as, ws, M, N, Kb, per, out_dtype, rows);
   else
     hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN, SW, KS, true>), grid, block, 0, s, out, (splits > 1 || keep_partials) ? partial : nullptr, A, W,
-                       as, ws, M, N, Kb, per, out_dtype);
+                       as, ws, M, N, Kb, per, out_dtype, rows);
 }
 
 template <int EB>
 int gemm_entry(const char* name, void* out, const void* a, const float* as, const void* w, const float* ws,
                float* workspace, int64_t M, int64_t N, int64_t K, int out_dtype, int tile, int split_k, void* stream,
-               bool reduce = true) {
+               bool reduce = true, RowMap rows = {nullptr, nullptr, 0x7fffffff}) {
   LFM2_REQUIRE(M > 0 && N > 0 && K > 0, "%s: empty shape", name);
   LFM2_REQUIRE(M < (1 << 30) && N < (1 << 30), "%s: M or N too large", name);
   LFM2_REQUIRE(out_dtype >= LFM2_DTYPE_BF16 && out_dtype <= LFM2_DTYPE_F32, "%s: bad output dtype", name);
@@ -386,7 +402,7 @@ int gemm_entry(const char* name, void* out, const void* a, const float* as, cons
   const int64_t Kb = K * EB;
   if (Kb % 16 != 0 || ((uintptr_t)a | (uintptr_t)w) % 16 != 0) {
     LFM2_REQUIRE(reduce, "%s: partial products need K bytes and pointers aligned to 16", name);
-    hipLaunchKernelGGL(gemm_naive_kernel<EB>, dim3(ceil_div(M * N, 256)), dim3(256), 0, s, out, A, W, as, ws, M, N, K, out_dtype);
+    hipLaunchKernelGGL(gemm_naive_kernel<EB>, dim3(ceil_div(M * N, 256)), dim3(256), 0, s, out, A, W, as, ws, M, N, K, out_dtype, rows);
     LFM2_LAUNCH_CHECK();
   }
   Plan plan = default_plan(M, N, Kb);
@@ -395,6 +411,7 @@ int gemm_entry(const char* name, void* out, const void* a, const float* as, cons
     plan.tile = tile;
   }
   if (split_k > 0) plan.splits = split_k;
+  LFM2_REQUIRE(plan.splits == 1 || (!rows.slots && !rows.active), "%s: placed output rows do not combine with split-K", name);
   const int64_t steps = tile_steps(plan.tile, Kb);
   if (plan.splits > steps) plan.splits = (int)steps;
   // every split must own at least one step
@@ -402,7 +419,7 @@ int gemm_entry(const char* name, void* out, const void* a, const float* as, cons
   LFM2_REQUIRE(plan.splits == 1 || workspace != nullptr, "%s: split-K needs a workspace", name);
   LFM2_REQUIRE(reduce || workspace != nullptr, "%s: partial products need a destination", name);
 #define TILE_(ID, BM, BN, WM, WN, KS, ...) \
-  case ID: launch_tile<EB, BM, BN, WM, WN, EB == 1 ? 1 : 0, KS, ##__VA_ARGS__>(out, workspace, A, W, as, ws, (int)M, (int)N, Kb, plan.splits, out_dtype, !reduce, s); break
+  case ID: launch_tile<EB, BM, BN, WM, WN, EB == 1 ? 1 : 0, KS, ##__VA_ARGS__>(out, workspace, A, W, as, ws, (int)M, (int)N, Kb, plan.splits, out_dtype, !reduce, rows, s); break
   switch (plan.tile) {
     TILE_(0, 16, 64, 1, 4, 128);
     TILE_(1, 32, 64, 2, 2, 128);
@@ -469,6 +486,26 @@ extern "C" int lfm2_bf16_gemm(void* out, const void* x, const void* w, float* wo
                               int tile, int split_k, void* stream) {
   LFM2_REQUIRE(split_k <= 16, "bf16_gemm: split_k above 16");
   return gemm_entry<2>("bf16_gemm", out, x, nullptr, w, nullptr, workspace, M, N, K, LFM2_DTYPE_BF16, tile, split_k, stream);
+}
+
+extern "C" int lfm2_fp8_gemm_rows(void* out, const uint8_t* a_q, const float* a_scales, const uint8_t* w_q,
+                                  const float* w_scales, const int32_t* out_rows, const uint8_t* row_active,
+                                  int64_t out_capacity, int64_t M, int64_t N, int64_t K, int out_dtype, int tile,
+                                  void* stream) {
+  LFM2_REQUIRE(a_scales && w_scales, "fp8_gemm_rows: scales are required");
+  LFM2_REQUIRE(out_capacity > 0 && out_capacity < (1ll << 31), "fp8_gemm_rows: bad output capacity");
+  LFM2_REQUIRE(out_rows || M <= out_capacity, "fp8_gemm_rows: more rows than the output holds");
+  return gemm_entry<1>("fp8_gemm_rows", out, a_q, a_scales, w_q, w_scales, nullptr, M, N, K, out_dtype, tile, 1, stream, true,
+                       RowMap{out_rows, row_active, (int)out_capacity});
+}
+
+extern "C" int lfm2_bf16_gemm_rows(void* out, const void* x, const void* w, const int32_t* out_rows,
+                                   const uint8_t* row_active, int64_t out_capacity, int64_t M, int64_t N, int64_t K, int tile,
+                                   void* stream) {
+  LFM2_REQUIRE(out_capacity > 0 && out_capacity < (1ll << 31), "bf16_gemm_rows: bad output capacity");
+  LFM2_REQUIRE(out_rows || M <= out_capacity, "bf16_gemm_rows: more rows than the output holds");
+  return gemm_entry<2>("bf16_gemm_rows", out, x, nullptr, w, nullptr, nullptr, M, N, K, LFM2_DTYPE_BF16, tile, 1, stream, true,
+                       RowMap{out_rows, row_active, (int)out_capacity});
 }
 
 extern "C" int64_t lfm2_bf16_gemm_workspace(int64_t M, int64_t N, int64_t K) {

@@ -116,8 +116,9 @@ class LFM25HIPDecoder:
         self.fp8_weights.clear()
 
     # ------------------------------------------------------------------ capture
-    def _forward(self, cache, tokens, active=None, *, slot_ids=None, positions=None):
-        return self.engine._decode_forward(cache, tokens, active, slot_ids=slot_ids, positions=positions, fp8=self.fp8_weights)
+    def _forward(self, cache, tokens, active=None, *, slot_ids=None, positions=None, logits_out=None):
+        return self.engine._decode_forward(cache, tokens, active, slot_ids=slot_ids, positions=positions, fp8=self.fp8_weights,
+                                           logits_out=logits_out)
 
     def _capture(self, step, before_warmup=None):
         """Two warm-up launches, then record `step` into a HIP graph on the decoder's capture stream."""
@@ -171,12 +172,9 @@ class LFM25HIPDecoder:
         holder = {}
 
         def step():
-            logits = self._forward(cache, tokens, active)
-            if saved is not None and active is not None:
-                ops.scatter_logits(saved, logits, None, active)
-            elif saved is not None:
-                saved.copy_(logits)  # uncaptured steps allocate fresh logits each time; keep one stable buffer
-            holder["logits"] = saved if saved is not None else logits
+            # masked steps write only the live rows of `saved`; uncaptured steps write all of it, so that one stable
+            # buffer holds the logits either way
+            holder["logits"] = self._forward(cache, tokens, active, logits_out=saved)
 
         graph = self._capture(step, before_warmup=cache.seq_lens.zero_)
         entry = _DecodeGraph(cache, tokens, holder["logits"] if self.capture else saved, graph, active)
@@ -197,8 +195,7 @@ class LFM25HIPDecoder:
 
         def step():
             ops.gather_inputs(tokens, positions, active, entry.input_tokens, entry.cache.seq_lens, entry.active, slots)
-            logits = self._forward(entry.cache, tokens, active, slot_ids=slots, positions=positions)
-            ops.scatter_logits(entry.logits, logits, slots, active)
+            self._forward(entry.cache, tokens, active, slot_ids=slots, positions=positions, logits_out=entry.logits)
 
         graph = self._capture(step)
         return CompactDecodeGraph(graph, slots, (tokens, positions, active))

@@ -221,16 +221,17 @@ class LFM25Engine:
     def _fp8(self):
         return self._cuda_decoder.fp8_weights if self._cuda_decoder is not None else {}
 
-    def _norm_linear(self, x, norm_weight, residual, weight, fp8):
-        """residual-add + RMSNorm feeding a projection; W8A8 when the projection has an e4m3 copy."""
+    def _norm_linear(self, x, norm_weight, residual, weight, fp8, place=None):
+        """residual-add + RMSNorm feeding a projection; W8A8 when the projection has an e4m3 copy.  `place`
+        (an `ops.RowPlacement`) sends the product's rows into an existing buffer."""
         packed = fp8.get(id(weight))
         if packed is not None:
             q, scales, residual = ops.rms_norm_fp8(x, norm_weight, self.config.norm_eps, residual)
-            return packed.linear_quantized(q, scales, dtype=self.dtype), residual
+            return packed.linear_quantized(q, scales, dtype=self.dtype, place=place), residual
         if isinstance(x, ops.SplitProduct):
             x = x.materialize()
         normed, residual = ops.rms_norm(x, norm_weight, self.config.norm_eps, residual)
-        return ops.linear(normed, weight), residual
+        return ops.linear(normed, weight, place=place), residual
 
     def _linear(self, x, weight, fp8):
         """Out projection of an operator; `x` is a tensor or, from a fused producer, (e4m3 rows, scales)."""
@@ -263,14 +264,25 @@ class LFM25Engine:
                 hidden = ops.linear(ops.swiglu(gate_up), layer.w2_weight)
         return hidden, residual
 
-    def _head(self, hidden, residual, fp8):
-        logits, _ = self._norm_linear(hidden, self.weights.embedding_norm_weight, residual, self.weights.lm_head_weight, fp8)
+    def _head(self, hidden, residual, fp8, place=None):
+        logits, _ = self._norm_linear(hidden, self.weights.embedding_norm_weight, residual, self.weights.lm_head_weight, fp8,
+                                      place if self.dtype == torch.bfloat16 or id(self.weights.lm_head_weight) in fp8 else None)
+        if place is not None and logits is not place.out:   # a product the placing GEMM does not cover (fp16/fp32 head)
+            if place.active is None and place.slots is None:
+                place.out[:logits.size(0)].copy_(logits)
+            else:
+                active = place.active if place.active is not None else torch.ones(logits.size(0), device=logits.device, dtype=torch.bool)
+                ops.scatter_logits(place.out, logits, place.slots, active)
+            return place.out
         return logits
 
     # ------------------------------------------------------------------ decode step (one token per row)
-    def _decode_forward(self, cache: LFM25HybridCache, tokens, active=None, *, slot_ids=None, positions=None, fp8=None):
+    def _decode_forward(self, cache: LFM25HybridCache, tokens, active=None, *, slot_ids=None, positions=None, fp8=None,
+                        logits_out=None):
         """One token for every row (lfm25_cuda.py:128-192).  Rows index cache slots directly, or through `slot_ids`
-        (then `positions` are the rows' lengths and -1 marks padding)."""
+        (then `positions` are the rows' lengths and -1 marks padding).  With `logits_out` ([slots, vocab]) the head
+        projection writes the live rows' logits there (row -> its slot) and the other rows keep theirs: the
+        `_scatter_logits` step of lfm25_batching.py:99-101 without a copy."""
         cfg = self.config
         fp8 = self._fp8() if fp8 is None else fp8
         positions = cache.seq_lens if positions is None else positions
@@ -301,7 +313,8 @@ class LFM25Engine:
             return ops.conv_update(bcx, op.conv_weight, state, active, slot_ids)
 
         hidden, residual = self._backbone(tokens, attention_op, conv_op, fp8, defer_reduce=True)
-        logits = self._head(hidden, residual, fp8)
+        place = None if logits_out is None else ops.RowPlacement(logits_out, slot_ids, active)
+        logits = self._head(hidden, residual, fp8, place)
         ops.advance_positions(cache.seq_lens, positions, slot_ids, active)
         return logits
 

@@ -9,6 +9,7 @@ into a HIP graph.
 from __future__ import annotations
 
 from dataclasses import dataclass
+from typing import Optional
 
 import torch
 
@@ -199,16 +200,44 @@ def conv_prefill(bcx, weight, state, cu_seqlens, seq_of_token, slots):
 
 
 # ----------------------------------------------------------------------------------- GEMMs
-def linear(x: torch.Tensor, weight: torch.Tensor, *, tile: int = -1, split_k: int = 0) -> torch.Tensor:
+@dataclass
+class RowPlacement:
+    """Where a product's rows go: row m is written to `out[slots[m]]` (`out[m]` without slots) when `active[m]`
+    (always without a mask) and the slot is in range; the other rows of `out` keep their contents.  This is
+    `_scatter_logits` of lfm25_batching.py:25-32 done by the producing GEMM."""
+    out: torch.Tensor
+    slots: Optional[torch.Tensor] = None
+    active: Optional[torch.Tensor] = None
+
+    def check(self, rows: int, columns: int, dtype) -> None:
+        out = self.out
+        if out.ndim != 2 or out.size(1) != columns or out.dtype != dtype or not out.is_contiguous():
+            raise ValueError("placed rows need a contiguous [slots, columns] destination of the product's dtype")
+        if self.slots is None and rows > out.size(0):
+            raise ValueError("more product rows than destination rows")
+        if self.slots is not None and (self.slots.dtype != torch.int32 or self.slots.numel() != rows):
+            raise ValueError("slots must be int32, one per product row")
+        if self.active is not None and (self.active.dtype not in (torch.bool, torch.uint8) or self.active.numel() != rows):
+            raise ValueError("active must be a bool mask, one per product row")
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, *, tile: int = -1, split_k: int = 0,
+           place: Optional[RowPlacement] = None) -> torch.Tensor:
     """lfm25_cuda_kernels.py:19-29: y = x W^T.  bf16 runs the MFMA kernel of this package; other dtypes
-    (only used by tests of the fp32 plumbing) go to the vendor GEMM."""
+    (only used by tests of the fp32 plumbing) go to the vendor GEMM.  With `place`, rows land in `place.out`."""
     if x.dtype != torch.bfloat16:
+        if place is not None:
+            raise ValueError("placed rows need a bf16 product")
         return torch.nn.functional.linear(x, weight)
     _check(x, weight)
     m, k = _rows(x), x.size(-1)
     n = weight.size(0)
     if weight.size(1) != k:
         raise ValueError("activation and weight widths differ")
+    if place is not None:
+        place.check(m, n, x.dtype)
+        call("lfm2_bf16_gemm_rows", place.out, x, weight, place.slots, place.active, place.out.size(0), m, n, k, tile)
+        return place.out
     out = torch.empty((*x.shape[:-1], n), device=x.device, dtype=x.dtype)
     need = query("lfm2_bf16_gemm_workspace", m, n, k) if split_k == 0 else max(split_k, 1) * m * n
     ws = torch.empty(need, device=x.device, dtype=torch.float32) if need and split_k != 1 else None
@@ -236,14 +265,20 @@ class PackedFP8Weight:
         values, scales = quantize_rows(x)
         return self.linear_quantized(values, scales, dtype=x.dtype, config=config)
 
-    def linear_quantized(self, x, scales, *, dtype=torch.bfloat16, config=None, defer_reduce=False):
+    def linear_quantized(self, x, scales, *, dtype=torch.bfloat16, config=None, defer_reduce=False, place=None):
         """config = (tile index, split_k) overrides the default tile choice.  With `defer_reduce`, a product the
-        plan (default or `config`) splits along K comes back as a `SplitProduct` for `rms_norm_fp8` to reduce."""
+        plan (default or `config`) splits along K comes back as a `SplitProduct` for `rms_norm_fp8` to reduce.
+        With `place` (a `RowPlacement`) the rows land in `place.out`."""
         batch, width = x.shape
         rows = self.values.size(0)
         if width != self.values.size(1):
             raise ValueError("FP8 activation and weight widths differ")
         tile, split_k = (-1, 0) if config is None else (int(config[0]), int(config[1]) if len(config) > 1 else 0)
+        if place is not None:
+            place.check(batch, rows, dtype)
+            call("lfm2_fp8_gemm_rows", place.out, x, scales, self.values, self.scales, place.slots, place.active,
+                 place.out.size(0), batch, rows, width, _code(dtype), tile)
+            return place.out
         if defer_reduce:
             splits = query("lfm2_fp8_gemm_default_splits", batch, rows, width) if split_k == 0 else split_k
             if splits > 1:

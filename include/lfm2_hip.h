@@ -123,6 +123,17 @@ int lfm2_bf16_gemm(void* out, const void* x, const void* w, float* workspace, in
                    int tile, int split_k, void* stream);
 int64_t lfm2_bf16_gemm_workspace(int64_t M, int64_t N, int64_t K);
 
+/* The two products with placed output rows: row m of the product is written to out row out_rows[m] (m itself when
+ * out_rows is NULL) unless that index is negative or >= out_capacity, or row_active[m] is 0 (row_active may be
+ * NULL); other rows of out keep their contents.  This is the head projection followed by _scatter_logits of
+ * lfm25_batching.py:25-32 (lfm25_cuda.py:190-192, lfm25_batching.py:99-101) in one launch, without the copy of
+ * the logits.  Never split along K. */
+int lfm2_fp8_gemm_rows(void* out, const uint8_t* a_q, const float* a_scales, const uint8_t* w_q, const float* w_scales,
+                       const int32_t* out_rows, const uint8_t* row_active, int64_t out_capacity, int64_t M, int64_t N,
+                       int64_t K, int out_dtype, int tile, void* stream);
+int lfm2_bf16_gemm_rows(void* out, const void* x, const void* w, const int32_t* out_rows, const uint8_t* row_active,
+                        int64_t out_capacity, int64_t M, int64_t N, int64_t K, int tile, void* stream);
+
 /* ---------------------------------------------------------------- KV cache and attention */
 
 /* store_kv of lfm25_fp8_kv.py:28-69.  k,v [B,T,KH,D] with element strides (ks0,ks1,ks2) / (vs0,..);

@@ -199,6 +199,51 @@ def test_bf16_linear_matches_fp32_matmul_of_the_same_operands(ops, m, k, n):
         torch.testing.assert_close(got.float().cpu(), expected, atol=2e-3, rtol=2 ** -7)
 
 
+@pytest.mark.parametrize("fp8", [True, False])
+@pytest.mark.parametrize("m,k,n", [(48, 512, 1000), (200, 2048, 4096), (7, 100, 72)])
+@torch.inference_mode()
+def test_placed_rows_equal_the_product_followed_by_scatter_logits(ops, fp8, m, k, n):
+    """The placing GEMMs against the plain product + `scatter_logits` (lfm25_batching.py:25-32): bit-identical live
+    rows, untouched rows elsewhere; padding slots (-1), inactive rows and out-of-range slots are skipped.  K = 100 takes the
+    any-shape kernel."""
+    torch.manual_seed(m + n)
+    x, w = torch.randn(m, k, device=DEV).bfloat16(), (torch.randn(n, k, device=DEV) * 0.05).bfloat16()
+    capacity = m + 9
+    slots = torch.randperm(capacity, device=DEV)[:m].to(torch.int32)
+    slots[1] = -1
+    slots[m - 1] = capacity + 3                      # beyond the destination: dropped, never written
+    active = torch.rand(m, device=DEV) > 0.3
+    active[0] = True
+    packed = ops.PackedFP8Weight.from_weight(w) if fp8 else None
+    q, scales = ops.quantize_rows(x) if fp8 else (None, None)
+
+    def product(place=None, tile=-1):
+        if fp8:
+            return packed.linear_quantized(q, scales, dtype=torch.bfloat16, config=(tile, 0), place=place)
+        return ops.linear(x, w, tile=tile, place=place)
+
+    for tile in (-1, 0, 2, 6, 12, 14, 15, 17):
+        if not fp8 and tile >= 9:
+            continue
+        plain = product(tile=tile)
+        for use_slots, use_mask in [(True, True), (True, False), (False, True), (False, False)]:
+            saved = torch.full((capacity, n), 7.0, device=DEV, dtype=torch.bfloat16)
+            expected = saved.clone()
+            rows = torch.arange(m, device=DEV)
+            target = slots.long() if use_slots else rows
+            keep = (target >= 0) & (target < capacity)
+            if use_mask:
+                keep &= active
+            expected[target[keep]] = plain[keep]
+            out = product(ops.RowPlacement(saved, slots if use_slots else None, active if use_mask else None), tile)
+            assert out is saved
+            assert torch.equal(saved.view(torch.int16), expected.view(torch.int16)), (tile, use_slots, use_mask)
+    with pytest.raises(ValueError):
+        product(ops.RowPlacement(torch.zeros(m - 1, n, device=DEV, dtype=torch.bfloat16)))
+    with pytest.raises(ValueError):
+        product(ops.RowPlacement(torch.zeros(capacity, n, device=DEV, dtype=torch.float16), slots))
+
+
 def _cache_tensors(batch, capacity, heads, dim, layout):
     if layout == "HND":
         k = torch.zeros(batch, heads, capacity, dim, device=DEV, dtype=torch.float8_e4m3fn).transpose(1, 2)
