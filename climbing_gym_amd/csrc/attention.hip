@@ -254,8 +254,10 @@ __global__ void __launch_bounds__(256) decode_attn_kernel(DecodeArgs a) {
 //   S = Q.K^T : sixteen v_mfma_f32_4x4x4_16B_bf16 (16 independent 4x4x4 blocks per instruction).  Block b
 //               multiplies Q[4 heads][4 dims] by K[tokens 4b..4b+3][4 dims], so lane l owns token l of the tile:
 //               it loads that token's 64-byte row with four 16-byte loads and ends with S[0..3][token l].
-//   softmax   : running maxima are wave-uniform and only raised (with a rescale) when some lane exceeds them,
-//               so per-lane partial sums of l and O can simply be added at the end.
+//   softmax   : running maxima are wave-uniform and only raised (with a rescale) when some lane exceeds them by
+//               more than kMaxSlack (so p <= 2^kMaxSlack, harmless in fp32 and bf16: the softmax is invariant to
+//               the reference point), so per-lane partial sums of l and O can simply be added at the end and the
+//               wave-wide maximum is needed on a wave's first tile and rarely afterwards.
 //   O += P.V  : lane (g16, q, i) loads V[token 4*g16+i (+16u)][dims 16q..16q+15]; every dword is a 4x4 byte block
 //               over the quad (4 tokens x 4 dims) which two DPP quad permutes + two v_perm transpose in
 //               registers, giving the B operand V[4 tokens][dim]; P comes back from LDS as the A operand.
@@ -265,6 +267,7 @@ __global__ void __launch_bounds__(256) decode_attn_kernel(DecodeArgs a) {
 // e4m3 -> bf16 conversion is v_cvt_scalef32_pk_bf16_fp8 (two values per instruction, scale 1).
 constexpr int kMfmaChunk = 1024;  // history tokens per workgroup (4 waves x 256)
 constexpr int kMfmaWaveTok = kMfmaChunk / 4;
+constexpr float kMaxSlack = 8.0f;  // log2 units
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 
@@ -373,7 +376,7 @@ __global__ void __launch_bounds__(256) decode_attn_mfma_kernel(DecodeArgs a) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       s[i] = valid ? s[i] * kscale : -1.0e30f;
-      raise |= s[i] > m[i];
+      raise |= s[i] > m[i] + kMaxSlack;
     }
     if (__any(raise)) {
 #pragma unroll
@@ -409,8 +412,7 @@ __global__ void __launch_bounds__(256) decode_attn_mfma_kernel(DecodeArgs a) {
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
       float v = acc[w][i];
-      v += __shfl_xor(v, 16, 64);
-      v += __shfl_xor(v, 32, 64);
+      v = add_lane_xor32(add_lane_xor16(v));
       acc[w][i] = v;
     }
   }
@@ -651,8 +653,7 @@ prefill_attn_kernel(T* __restrict__ out, const T* __restrict__ q, const T* __res
         st[j][i] = ok ? st[j][i] * scale_log2e : -1.0e30f;
         mx = fmaxf(mx, st[j][i]);
       }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    mx = max_lane_xor32(max_lane_xor16(mx));
     const float mnew = fmaxf(m, mx);
     const float alpha = exp2f(m - mnew);
     float rs = 0.f;
@@ -665,8 +666,7 @@ prefill_attn_kernel(T* __restrict__ out, const T* __restrict__ q, const T* __res
         rs += p;
         pf[j >> 1][(j & 1) * 4 + i] = (T)p;
       }
-    rs += __shfl_xor(rs, 16, 64);
-    rs += __shfl_xor(rs, 32, 64);
+    rs = add_lane_xor32(add_lane_xor16(rs));
     l = fmaf(l, alpha, rs);
     m = mnew;
 #pragma unroll

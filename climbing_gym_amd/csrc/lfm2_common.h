@@ -60,40 +60,30 @@ template <typename T> __device__ __forceinline__ float round_to(float v) { retur
 template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
 }
-__device__ __forceinline__ float wave_sum(float v) {
-  v += dpp_move<0xB1>(v);    // quad_perm [1,0,3,2]
-  v += dpp_move<0x4E>(v);    // quad_perm [2,3,0,1]
-  v += dpp_move<0x141>(v);   // row_half_mirror
-  v += dpp_move<0x140>(v);   // row_mirror
-  {
-    const unsigned x = __builtin_bit_cast(unsigned, v);
-    const auto r = __builtin_amdgcn_permlane16_swap(x, x, false, false);
-    v = __builtin_bit_cast(float, (unsigned)r[0]) + __builtin_bit_cast(float, (unsigned)r[1]);
-  }
-  {
-    const unsigned x = __builtin_bit_cast(unsigned, v);
-    const auto r = __builtin_amdgcn_permlane32_swap(x, x, false, false);
-    v = __builtin_bit_cast(float, (unsigned)r[0]) + __builtin_bit_cast(float, (unsigned)r[1]);
-  }
-  return v;
+// v combined with the value of the same lane position in the neighbouring row of 16 lanes (lane ^ 16), or in the
+// other half of the wave (lane ^ 32).  The swap returns {own | partner, partner | own} by row parity: a commutative
+// combination of the two is the same on both sides.
+struct AddOp { static __device__ __forceinline__ float apply(float a, float b) { return a + b; } };
+struct MaxOp { static __device__ __forceinline__ float apply(float a, float b) { return fmaxf(a, b); } };
+template <typename Op, bool HALVES> __device__ __forceinline__ float combine_swapped(float v) {
+  const unsigned x = __builtin_bit_cast(unsigned, v);
+  const auto r = HALVES ? __builtin_amdgcn_permlane32_swap(x, x, false, false) : __builtin_amdgcn_permlane16_swap(x, x, false, false);
+  return Op::apply(__builtin_bit_cast(float, (unsigned)r[0]), __builtin_bit_cast(float, (unsigned)r[1]));
 }
-__device__ __forceinline__ float wave_max(float v) {
-  v = fmaxf(v, dpp_move<0xB1>(v));
-  v = fmaxf(v, dpp_move<0x4E>(v));
-  v = fmaxf(v, dpp_move<0x141>(v));
-  v = fmaxf(v, dpp_move<0x140>(v));
-  {
-    const unsigned x = __builtin_bit_cast(unsigned, v);
-    const auto r = __builtin_amdgcn_permlane16_swap(x, x, false, false);
-    v = fmaxf(__builtin_bit_cast(float, (unsigned)r[0]), __builtin_bit_cast(float, (unsigned)r[1]));
-  }
-  {
-    const unsigned x = __builtin_bit_cast(unsigned, v);
-    const auto r = __builtin_amdgcn_permlane32_swap(x, x, false, false);
-    v = fmaxf(__builtin_bit_cast(float, (unsigned)r[0]), __builtin_bit_cast(float, (unsigned)r[1]));
-  }
-  return v;
+__device__ __forceinline__ float add_lane_xor16(float v) { return combine_swapped<AddOp, false>(v); }
+__device__ __forceinline__ float add_lane_xor32(float v) { return combine_swapped<AddOp, true>(v); }
+__device__ __forceinline__ float max_lane_xor16(float v) { return combine_swapped<MaxOp, false>(v); }
+__device__ __forceinline__ float max_lane_xor32(float v) { return combine_swapped<MaxOp, true>(v); }
+template <typename Op> __device__ __forceinline__ float wave_all(float v) {
+  v = Op::apply(v, dpp_move<0xB1>(v));    // quad_perm [1,0,3,2]
+  v = Op::apply(v, dpp_move<0x4E>(v));    // quad_perm [2,3,0,1]
+  v = Op::apply(v, dpp_move<0x141>(v));   // row_half_mirror
+  v = Op::apply(v, dpp_move<0x140>(v));   // row_mirror
+  v = combine_swapped<Op, false>(v);
+  return combine_swapped<Op, true>(v);
 }
+__device__ __forceinline__ float wave_sum(float v) { return wave_all<AddOp>(v); }
+__device__ __forceinline__ float wave_max(float v) { return wave_all<MaxOp>(v); }
 // Block-wide reductions through a small LDS array; every thread gets the result.
 template <int WAVES> __device__ __forceinline__ float block_sum(float v, float* scratch) {
   v = wave_sum(v);
