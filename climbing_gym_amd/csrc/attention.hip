@@ -88,6 +88,10 @@ constexpr int kChunk = 512;        // history tokens per workgroup
 constexpr int kWaveTok = kChunk / 4;
 constexpr int kGB = 4;             // query heads per workgroup (one GQA group, padded)
 
+// Schedule layout (int32): [0] number of (row, chunk) pairs; from kSchedRows on one 16-byte record per row (index of
+// the pair of its first full chunk, index of the pair of its partial chunk, its length or 0 when it sits out, 0);
+// then one 16-byte record per pair (row, chunk, length, slot).
+constexpr int kSchedRows = 4;
 struct DecodeArgs {
   void* out;
   const void *q, *kc, *vc;
@@ -95,11 +99,33 @@ struct DecodeArgs {
   const int32_t *positions, *slot_ids, *block_table;
   const uint8_t* active;
   float *ws_acc, *ws_m, *ws_l;
-  const int32_t* schedule;  // [0] = number of (row, chunk) items, then the pairs
+  const int32_t* schedule;  // work list of the scheduled kernel (layout above); null for the generic kernel
   int64_t max_blocks, c0, c1, c2;
-  int page, QH, KH, D, G, nchunks, chunk;
+  int page, QH, KH, D, G, nchunks, chunk, B;
   float scale_log2e;
 };
+
+// Row of the partial-result arrays that holds chunk c of (row b, query head qh).  The generic kernel's rows are dense,
+// [b][qh][chunk]; the scheduled kernel's are [pair][qh], so that one item's heads are one contiguous block.
+struct RowPairs { int full_first, partial, nfull, len; };
+// The row's length (0: inactive, padding or empty) and, for the scheduled kernel, where its partial results are:
+// one load of the row's record there, the rows' own arrays otherwise.
+__device__ __forceinline__ RowPairs row_pairs(const DecodeArgs& a, int b) {
+  RowPairs r{0, 0, 0, 0};
+  if (a.schedule) {
+    const i32x4 rec = *reinterpret_cast<const i32x4*>(a.schedule + kSchedRows + 4 * b);
+    r.full_first = rec[0]; r.partial = rec[1]; r.len = rec[2]; r.nfull = rec[2] / a.chunk;
+    return r;
+  }
+  r.len = a.positions[b] + 1;
+  if (a.active && !a.active[b]) r.len = 0;
+  if (a.slot_ids && a.slot_ids[b] < 0) r.len = 0;
+  return r;
+}
+__device__ __forceinline__ int64_t partial_row(const DecodeArgs& a, const RowPairs& r, int b, int qh, int c) {
+  if (!a.schedule) return ((int64_t)b * a.QH + qh) * a.nchunks + c;
+  return (int64_t)(c < r.nfull ? r.full_first + c : r.partial) * a.QH + qh;
+}
 
 template <bool FP8> struct KvLoad;
 template <> struct KvLoad<true> {  // 16 e4m3 codes
@@ -265,8 +291,7 @@ __global__ void __launch_bounds__(256) decode_attn_kernel(DecodeArgs a) {
 //               are added once per wave.
 //
 // e4m3 -> bf16 conversion is v_cvt_scalef32_pk_bf16_fp8 (two values per instruction, scale 1).
-constexpr int kMfmaChunk = 1024;  // history tokens per workgroup (4 waves x 256)
-constexpr int kMfmaWaveTok = kMfmaChunk / 4;
+constexpr int kMfmaChunk = 256;  // history tokens per item (one wave)
 constexpr float kMaxSlack = 8.0f;  // log2 units
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -285,92 +310,150 @@ __device__ __forceinline__ int quad_transpose_bytes(int x, int lane) {
   return __builtin_amdgcn_perm(u, y, (lane & 2) ? 0x03020706 : 0x05040100);
 }
 
-// The grid is persistent: workgroups stride over the (row, chunk, KV head) items of a schedule that a tiny kernel
-// builds from the rows' current lengths, so a ragged batch in a large-capacity cache launches no empty workgroups.
-template <bool PAGED>
-__global__ void __launch_bounds__(256) decode_attn_mfma_kernel(DecodeArgs a) {
-  constexpr int D = 64;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int g = lane & 3, vq = (lane >> 2) & 3, g16 = lane >> 4;
-  __shared__ __bf16 lds_p[4][4][64];
-  __shared__ float sm[4][4], sl[4][4], sacc[4][4][D];
-  const int items = a.schedule[0] * a.KH;
-  if (items <= 0) return;
-  // An item's row, chunk, length and slot sit behind three dependent loads; the next item's are fetched while the
-  // current one is processed so that chain is off the critical path of every item but a workgroup's first.
-  struct Meta { int b, chunk, len; int64_t slot; };
-  auto load_meta = [&](int item) {
-    const int pair = (item < items ? item : items - 1) / a.KH;
-    Meta mt;
-    mt.b = a.schedule[2 + 2 * pair];
-    mt.chunk = a.schedule[3 + 2 * pair];
-    mt.slot = a.slot_ids ? a.slot_ids[mt.b] : mt.b;
-    mt.len = a.positions[mt.b] + 1;
-    return mt;
-  };
-  Meta next_meta = load_meta(blockIdx.x);
-  for (int item = blockIdx.x; item < items; item += gridDim.x) {
-  const Meta meta = next_meta;
-  next_meta = load_meta(item + gridDim.x);
-  const int h = item % a.KH;
-  const int b = meta.b, chunk = meta.chunk, len = meta.len;
-  const int64_t slot = meta.slot;
-  const int start = chunk * kMfmaChunk;
+// The grid is persistent and its unit is the wave: every wave works on its own through (row, chunk, KV head) items of
+// a schedule that a tiny kernel builds from the rows' current lengths, and writes its item's partial result itself.
+// A ragged batch in a large-capacity cache therefore launches no empty work, and no wave ever waits at a barrier
+// for a neighbour with a longer piece of history.
+//
+// What the kernel can draw from memory is bounded by the bytes its waves have in flight, so a wave treats its items
+// as one stream of 64-token tiles and always has the next tile of the stream on its way while it multiplies the
+// current one, across item boundaries too:
+//   * a wave's items are its own index plus multiples of the number of waves; the schedule lists the items by
+//     decreasing length (in tiles), so every wave gets the same work to within a tile or two without a work queue
+//     (a counter's returned value would sit in a register that no wait protects across a whole item);
+//   * an item's 16-byte record (row, chunk, length, slot) is read through the scalar cache one item ahead;
+//   * the next item's first tile goes into the spare tile registers while the current item's last tile is
+//     multiplied, and with every tile come eight bytes per lane of the queries of the item it belongs to, which
+//     the wave puts into LDS when it starts that item (the query operands are read from there for every tile
+//     rather than held in 32 registers).
+// Loads are never issued under a condition (a branch around loads makes every later wait a wait for all of them),
+// and nothing is loaded straight into LDS (with such a load in flight the compiler waits for all loads at once).
+struct ItemRecord { int b, chunk, len, slot; };
 
-  // A operand of S = Q.K^T: Q[head g][dims 4s..4s+3] for s = 0..15 (zero rows beyond the group)
-  s16x4 qop[16];
-  {
-    const bool ok = g < a.G;
-    const __bf16* src = (const __bf16*)a.q + ((int64_t)b * a.QH + h * a.G + (ok ? g : 0)) * D;
-#pragma unroll
-    for (int c = 0; c < 8; ++c) {
-      i32x4 w = {0, 0, 0, 0};
-      if (ok) w = *reinterpret_cast<const i32x4*>(src + 8 * c);
-      const i32x2 lo = {w[0], w[1]}, hi = {w[2], w[3]};
-      qop[2 * c] = __builtin_bit_cast(s16x4, lo);
-      qop[2 * c + 1] = __builtin_bit_cast(s16x4, hi);
-    }
-  }
-  auto token_offset = [&](int t) -> int64_t {
+template <bool PAGED>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) decode_attn_mfma_kernel(DecodeArgs a) {
+  constexpr int D = 64;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // item state lives in scalar registers
+  const int g = lane & 3, vq = (lane >> 2) & 3, g16 = lane >> 4;
+  __shared__ __bf16 lds_p[4][4][64];   // one P tile per wave; nothing in LDS is shared between waves
+  __shared__ __attribute__((aligned(16))) float lds_o[4][4][4 * D + 4];   // per wave: the four token groups' O[head][dim] (+4: banks)
+  __shared__ __attribute__((aligned(16))) __bf16 lds_q[4][4][D];          // per wave: the item's query rows
+  const int32_t* const records = a.schedule + kSchedRows + 4 * a.B;
+  const int items = a.schedule[0] * a.KH;
+  const int first = blockIdx.x * 4 + wave, nwaves = gridDim.x * 4;
+  if (first >= items) return;
+
+  // ---- the pieces of the pipeline
+  // An item's record comes through the scalar cache (nothing writes the records while this kernel runs, so they are
+  // read as constant memory): scalar loads have their own counter and do not queue behind the tile loads.
+  auto read_record = [&](int idx) {
+    const int pair = (idx < items ? idx : items - 1) / a.KH;
+    const uint64_t address = (uint64_t)(records + 4 * (int64_t)pair);   // the same in every lane; say so to the compiler
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)address), hi = __builtin_amdgcn_readfirstlane((uint32_t)(address >> 32));
+    return *reinterpret_cast<const __attribute__((address_space(4))) i32x4*>(((uint64_t)hi << 32) | lo);
+  };
+  auto token_offset = [&](int b, int64_t slot, int h, int t) -> int64_t {
     if (PAGED) {
       const int64_t blk = a.block_table[(int64_t)b * a.max_blocks + t / a.page];
       return blk * a.c0 + (int64_t)(t % a.page) * a.c1 + (int64_t)h * a.c2;
     }
     return slot * a.c0 + (int64_t)t * a.c1 + (int64_t)h * a.c2;
   };
-
-  float m[4], l[4];
-  f32x4 acc[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) { m[i] = -1.0e30f; l[i] = 0.f; acc[i] = f32x4{0.f, 0.f, 0.f, 0.f}; }
-
-  const int wbeg = start + wave * kMfmaWaveTok;
-  int wend = wbeg + kMfmaWaveTok;
-  wend = wend < len ? wend : len;
   const uint8_t* kbase = (const uint8_t*)a.kc;
   const uint8_t* vbase = (const uint8_t*)a.vc;
-  for (int T = wbeg; T < wend; T += 64) {
-    // ---- loads: this lane's K row, its scales, and its four V slices
-    const int tk = T + lane;
-    const bool valid = tk < wend;
-    const int64_t koff = token_offset(valid ? tk : wend - 1);
-    i32x4 kreg[4], vreg[4];
+  struct Tile { i32x4 k[4], v[4]; float sk, sv; i32x2 q; };
+  // this lane's K row, its scales, and its four V slices of the tile at T (tokens clamped to the item's last)
+  auto fetch = [&](int b, int64_t slot, int h, int T, int wend, Tile& t) {
+    int tk = T + lane;
+    tk = tk < wend ? tk : wend - 1;
+    const int64_t koff = token_offset(b, slot, h, tk);
 #pragma unroll
-    for (int c = 0; c < 4; ++c) kreg[c] = *reinterpret_cast<const i32x4*>(kbase + koff + 16 * c);
-    const float sk = a.ks[koff / D], sv = a.vs[koff / D];
+    for (int c = 0; c < 4; ++c) t.k[c] = *reinterpret_cast<const i32x4*>(kbase + koff + 16 * c);
+    t.sk = a.ks[koff / D];
+    t.sv = a.vs[koff / D];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       int tv = T + 16 * u + 4 * g16 + g;
       tv = tv < wend ? tv : wend - 1;
-      vreg[u] = *reinterpret_cast<const i32x4*>(vbase + token_offset(tv) + 16 * vq);
+      t.v[u] = *reinterpret_cast<const i32x4*>(vbase + token_offset(b, slot, h, tv) + 16 * vq);
     }
-    // ---- S[0..3][token lane]
+    // this lane's share of the item's queries: head g (clamped into the tensor), dims 4 (lane / 4) .. + 3
+    int row = h * a.G + g;
+    row = row < a.QH ? row : a.QH - 1;
+    t.q = *reinterpret_cast<const i32x2*>((const __bf16*)a.q + ((int64_t)b * a.QH + row) * D + 4 * (lane >> 2));
+  };
+  const uint32_t q_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) __bf16*)&lds_q[wave][g][0];
+  const uint32_t p_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) __bf16*)&lds_p[wave][g][4 * g16];
+
+  // ---- prologue: the first item, the second item's record, the first tile
+  int idx = first, idx_next = first + nwaves;
+  int b, chunk, len, h;
+  int64_t slot;
+  {
+    const i32x4 rec = read_record(idx);
+    b = rec[0]; chunk = rec[1]; len = rec[2]; slot = rec[3]; h = idx % a.KH;
+  }
+  i32x4 rec_next = read_record(idx_next);
+  int wbeg = chunk * kMfmaChunk;
+  int wend = wbeg + kMfmaChunk;
+  wend = wend < len ? wend : len;
+  Tile tile, ahead;
+  fetch(b, slot, h, wbeg, wend, tile);
+
+  float m[4], l[4];
+  f32x4 acc[4];
+  int T = wbeg;
+  // One tile of the stream: `cur` holds it, the tile after it is fetched into `nxt`.  Returns false after the
+  // wave's last item.  (Two calls with the tiles swapped make the loop body, so no tile is ever copied: a copy of
+  // registers that a load is still filling would wait for the load.)
+  auto step = [&](Tile& cur, Tile& nxt) __attribute__((always_inline)) -> bool {
+    if (T == wbeg) {   // ---- item start: the queries that came with this tile
+      *reinterpret_cast<i32x2*>(&lds_q[wave][g][4 * (lane >> 2)]) = cur.q;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { m[i] = -1.0e30f; l[i] = 0.f; acc[i] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+    }
+    // ---- the next tile of the stream: this item's, or the first of the next item (its record was asked for one
+    // item ago); without a next item, this item's last tile again
+    const bool last = T + 64 >= wend;
+    int nb = b, nlen = len, nh = h, nwbeg = wbeg, nwend = wend;
+    int64_t nslot = slot;
+    const bool have_next = last && idx_next < items;
+    if (have_next) {
+      nb = rec_next[0]; nlen = rec_next[2]; nslot = rec_next[3]; nh = idx_next % a.KH;
+      nwbeg = rec_next[1] * kMfmaChunk;
+      nwend = nwbeg + kMfmaChunk;
+      nwend = nwend < nlen ? nwend : nlen;
+    }
+    const int fT = last ? nwbeg : T + 64;
+    fetch(nb, nslot, nh, fT, nwend, nxt);
+
+    const bool valid = T + lane < wend;
+    const float sk = cur.sk, sv = cur.sv;
+    // ---- S[0..3][token lane].  A operand: Q[head g][dims 4s..4s+3] for s = 0..15, read from LDS for every tile
+    // rather than held in 32 registers (rows beyond the group hold a neighbouring head's queries: their results are
+    // computed and never stored).
     f32x4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int c = 0; c < 4; ++c)
+    for (int half = 0; half < 2; ++half) {   // two reads of 64 bytes: half the registers of one of 128
+      i32x4 qraw[4];
+      asm volatile(
+          "ds_read_b128 %0, %4\n\t"
+          "ds_read_b128 %1, %4 offset:16\n\t"
+          "ds_read_b128 %2, %4 offset:32\n\t"
+          "ds_read_b128 %3, %4 offset:48\n\t"
+          "s_waitcnt lgkmcnt(0)"
+          : "=&v"(qraw[0]), "=&v"(qraw[1]), "=&v"(qraw[2]), "=&v"(qraw[3])
+          : "v"(q_lds + half * 64)
+          : "memory");
 #pragma unroll
-      for (int w = 0; w < 4; ++w)
-        s = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(qop[4 * c + w], e4m3x4_to_bf16x4(kreg[c][w]), s, 0, 0, 0);
+      for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const i32x4 q4 = qraw[2 * c + (w >> 1)];
+          const i32x2 q2 = {q4[2 * (w & 1)], q4[2 * (w & 1) + 1]};
+          s = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, q2), e4m3x4_to_bf16x4(cur.k[2 * half + c][w]), s, 0, 0, 0);
+        }
+    }
     const float kscale = a.scale_log2e * sk;
     bool raise = false;
 #pragma unroll
@@ -396,88 +479,179 @@ __global__ void __launch_bounds__(256) decode_attn_mfma_kernel(DecodeArgs a) {
       lds_p[wave][i][lane] = (__bf16)(p * sv);
     }
     // ---- O[0..3][dims 16*vq + 4w + g] += P . V over this lane group's tokens
+    i32x2 praw[4];
+    asm volatile(
+        "ds_read_b64 %0, %4\n\t"
+        "ds_read_b64 %1, %4 offset:32\n\t"
+        "ds_read_b64 %2, %4 offset:64\n\t"
+        "ds_read_b64 %3, %4 offset:96\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&v"(praw[0]), "=&v"(praw[1]), "=&v"(praw[2]), "=&v"(praw[3])
+        : "v"(p_lds)
+        : "memory");
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      const i32x2 praw = *reinterpret_cast<const i32x2*>(&lds_p[wave][g][16 * u + 4 * g16]);
-      const s16x4 pop = __builtin_bit_cast(s16x4, praw);
+      const s16x4 pop = __builtin_bit_cast(s16x4, praw[u]);
 #pragma unroll
       for (int w = 0; w < 4; ++w)
-        acc[w] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(pop, e4m3x4_to_bf16x4(quad_transpose_bytes(vreg[u][w], lane)), acc[w], 0, 0, 0);
+        acc[w] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(pop, e4m3x4_to_bf16x4(quad_transpose_bytes(cur.v[u][w], lane)), acc[w], 0, 0, 0);
     }
-  }
-  // ---- wave totals: l over all lanes, O over the four token groups
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    l[i] = wave_sum(l[i]);
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      float v = acc[w][i];
-      v = add_lane_xor32(add_lane_xor16(v));
-      acc[w][i] = v;
-    }
-  }
-  if (g16 == 0) {
+    T += 64;
+    if (!last) return true;
+
+    // ---- item end.  Wave totals: l over all lanes; O over the four token groups through LDS, which also turns the
+    // MFMA layout (lane = 4 dims apart) into rows: lane L ends with O[head L/16][dims 4(L%16)..+3] and the item's
+    // heads leave as one contiguous block of 16 bytes per lane
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
+      l[i] = wave_sum(l[i]);
 #pragma unroll
-      for (int w = 0; w < 4; ++w) sacc[wave][i][16 * vq + 4 * w + g] = acc[w][i];
+      for (int w = 0; w < 4; ++w) lds_o[wave][g16][i * D + 16 * vq + 4 * w + g] = acc[w][i];
     }
-    if (lane == 0) {
+    {
+      const int i = lane >> 4, d4 = 4 * (lane & 15);
+      f32x4 o = *reinterpret_cast<const f32x4*>(&lds_o[wave][0][i * D + d4]);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) { sm[wave][i] = m[i]; sl[wave][i] = l[i]; }
-    }
-  }
-  __syncthreads();
-  {
-    const int gi = threadIdx.x >> 6, d = threadIdx.x & 63;  // 4 heads x 64 dims = 256 threads
-    if (gi < a.G) {
-      float mm = sm[0][gi];
-#pragma unroll
-      for (int w = 1; w < 4; ++w) mm = fmaxf(mm, sm[w][gi]);
-      float lt = 0.f, ot = 0.f;
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        const float f = __builtin_amdgcn_exp2f(sm[w][gi] - mm);
-        lt = fmaf(sl[w][gi], f, lt);
-        ot = fmaf(sacc[w][gi][d], f, ot);
+      for (int t = 1; t < 4; ++t) {
+        const f32x4 part_o = *reinterpret_cast<const f32x4*>(&lds_o[wave][t][i * D + d4]);
+        o[0] += part_o[0]; o[1] += part_o[1]; o[2] += part_o[2]; o[3] += part_o[3];
       }
-      const int64_t prow = ((int64_t)b * a.QH + h * a.G + gi) * a.nchunks + chunk;
-      a.ws_acc[prow * D + d] = ot;
-      if (d == 0) { a.ws_m[prow] = mm; a.ws_l[prow] = lt; }
+      const int64_t prow = (int64_t)(idx / a.KH) * a.QH + h * a.G;
+      if (i < a.G) *reinterpret_cast<f32x4*>(a.ws_acc + (prow + i) * D + d4) = o;
+      if (lane == 0) {   // the heads' maxima and sums: wave-uniform, sixteen bytes each for a full group
+        if (a.G == 4) {
+          *reinterpret_cast<f32x4*>(a.ws_m + prow) = f32x4{m[0], m[1], m[2], m[3]};
+          *reinterpret_cast<f32x4*>(a.ws_l + prow) = f32x4{l[0], l[1], l[2], l[3]};
+        } else {
+          a.ws_m[prow] = m[0]; a.ws_l[prow] = l[0];
+          if (a.G > 1) { a.ws_m[prow + 1] = m[1]; a.ws_l[prow + 1] = l[1]; }
+          if (a.G > 2) { a.ws_m[prow + 2] = m[2]; a.ws_l[prow + 2] = l[2]; }
+        }
+      }
     }
-  }
-  __syncthreads();  // the LDS tiles are reused by the next item
-  }
+    // Reads and writes share one counter and complete out of order with respect to each other, so with a store in
+    // flight every wait for a load becomes a wait for everything.  Let the stores finish here, where the only
+    // loads in flight are the next item's first tile and queries, which are needed next anyway.
+    __builtin_amdgcn_s_waitcnt(0 | (0x7 << 4) | (0xF << 8));
+    // ---- step to the next item; ask for the record of the one after it
+    if (!have_next) return false;
+    idx = idx_next;
+    b = nb; len = nlen; slot = nslot; h = nh; wbeg = nwbeg; wend = nwend;
+    T = wbeg;
+    idx_next = idx + nwaves;
+    rec_next = read_record(idx_next);
+    return true;
+  };
+  while (step(tile, ahead) && step(ahead, tile)) {}
 }
 
 // One workgroup turns the rows' lengths into the item list of the persistent kernel: row b contributes
-// ceil((positions[b]+1) / chunk) items unless it is inactive or padding.
+// ceil((positions[b]+1) / chunk) items unless it is inactive or padding.  Items are listed by decreasing length in
+// 64-token tiles: all full chunks first, then the rows' last, partial chunks of 4, 3, 2 and 1 tiles.  Waves take the
+// items round robin, so the r-th items of all waves are (nearly) equally long and every wave gets the same work.
+// One counting sweep over the rows gives the classes' sizes, a second one places the rows: in each, a thread's rank
+// within its class comes from a wave scan and the waves' totals.
+constexpr int kSchedClasses = 5;   // full chunks, then partial chunks of 4, 3, 2, 1 tiles (chunk = 256)
 __global__ void __launch_bounds__(1024)
 decode_schedule_kernel(int32_t* schedule, const int32_t* positions, const uint8_t* active, const int32_t* slot_ids, int B,
                        int chunk) {
-  __shared__ int scan[1024];
-  __shared__ int carry;
-  if (threadIdx.x == 0) carry = 0;
+  __shared__ int wave_total[kSchedClasses][16];
+  __shared__ int class_base[kSchedClasses + 1];   // where each class starts; running, during the second sweep
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int pairs_at = kSchedRows + 4 * B;
+  const int tiles_per_chunk = chunk / 64;
+  auto row_length = [&](int b) {
+    int len = 0;
+    if (b < B && (!active || active[b]) && (!slot_ids || slot_ids[b] >= 0)) len = positions[b] + 1;
+    return len > 0 ? len : 0;
+  };
+  auto classify = [&](int len, int* n) {   // how many items of each class the row contributes
+#pragma unroll
+    for (int k = 0; k < kSchedClasses; ++k) n[k] = 0;
+    n[0] = len / chunk;
+    const int rest_tiles = (len % chunk + 63) / 64;
+    if (rest_tiles > 0) {
+      const int k = tiles_per_chunk + 1 - rest_tiles;   // 1 .. tiles_per_chunk
+#pragma unroll
+      for (int c = 1; c < kSchedClasses; ++c) n[c] = c == (k < kSchedClasses ? k : kSchedClasses - 1);
+    }
+  };
+  // sweep 1: class sizes
+  int mine[kSchedClasses] = {0, 0, 0, 0, 0};
+  for (int base = 0; base < B; base += 1024) {
+    int n[kSchedClasses];
+    classify(row_length(base + threadIdx.x), n);
+#pragma unroll
+    for (int k = 0; k < kSchedClasses; ++k) mine[k] += n[k];
+  }
+#pragma unroll
+  for (int k = 0; k < kSchedClasses; ++k) {
+    int v = mine[k];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    if (lane == 0) wave_total[k][wave] = v;
+  }
   __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0;
+    for (int k = 0; k < kSchedClasses; ++k) {
+      class_base[k] = at;
+      for (int w = 0; w < 16; ++w) at += wave_total[k][w];
+    }
+    class_base[kSchedClasses] = at;
+    schedule[0] = at;
+  }
+  __syncthreads();
+  // sweep 2: places
   for (int base = 0; base < B; base += 1024) {
     const int b = base + threadIdx.x;
-    int n = 0;
-    if (b < B && (!active || active[b]) && (!slot_ids || slot_ids[b] >= 0)) n = (positions[b] + chunk) / chunk;
-    scan[threadIdx.x] = n;
-    __syncthreads();
-    for (int o = 1; o < 1024; o <<= 1) {
-      const int v = threadIdx.x >= o ? scan[threadIdx.x - o] : 0;
-      __syncthreads();
-      scan[threadIdx.x] += v;
-      __syncthreads();
+    const int len = row_length(b);
+    int n[kSchedClasses], before[kSchedClasses];
+    classify(len, n);
+#pragma unroll
+    for (int k = 0; k < kSchedClasses; ++k) {   // inclusive scan over the wave
+      int v = n[k];
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const int up = __shfl_up(v, o, 64);
+        if (lane >= o) v += up;
+      }
+      before[k] = v - n[k];
+      if (lane == 63) wave_total[k][wave] = v;
     }
-    const int first = carry + scan[threadIdx.x] - n;
-    for (int c = 0; c < n; ++c) { schedule[2 + 2 * (first + c)] = b; schedule[3 + 2 * (first + c)] = c; }
     __syncthreads();
-    if (threadIdx.x == 1023) carry += scan[1023];
+    int first[kSchedClasses];
+#pragma unroll
+    for (int k = 0; k < kSchedClasses; ++k) {
+      int at = class_base[k] + before[k];
+      for (int w = 0; w < wave; ++w) at += wave_total[k][w];
+      first[k] = at;
+    }
+    if (b < B) {
+      const int full = n[0];
+      int partial = 0;
+#pragma unroll
+      for (int k = 1; k < kSchedClasses; ++k) if (n[k]) partial = first[k];
+      int32_t* row = schedule + kSchedRows + 4 * b;
+      row[0] = first[0]; row[1] = partial; row[2] = len; row[3] = 0;
+      const int slot = slot_ids ? slot_ids[b] : b;
+      for (int c = 0; c < full; ++c) {   // the record the attention kernel reads: row, chunk, length, slot
+        int32_t* rec = schedule + pairs_at + 4 * (first[0] + c);
+        rec[0] = b; rec[1] = c; rec[2] = len; rec[3] = slot;
+      }
+      if (len % chunk) {
+        int32_t* rec = schedule + pairs_at + 4 * partial;
+        rec[0] = b; rec[1] = full; rec[2] = len; rec[3] = slot;
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x < kSchedClasses) {
+      int add = 0;
+      for (int w = 0; w < 16; ++w) add += wave_total[threadIdx.x][w];
+      class_base[threadIdx.x] += add;
+    }
     __syncthreads();
   }
-  if (threadIdx.x == 0) { schedule[0] = carry; schedule[1] = chunk; }
 }
 
 // Merge the chunk partials of one (row, query head); inactive or empty rows give zeros.
@@ -485,40 +659,38 @@ template <typename T>
 __global__ void __launch_bounds__(64) decode_combine_kernel(DecodeArgs a) {
   const int b = blockIdx.x, qh = blockIdx.y;
   T* out = (T*)a.out + ((int64_t)b * a.QH + qh) * a.D;
-  int len = a.positions[b] + 1;
-  if (a.active && !a.active[b]) len = 0;
-  if (a.slot_ids && a.slot_ids[b] < 0) len = 0;
+  const RowPairs rp = row_pairs(a, b);
+  const int len = rp.len;
   if (len <= 0) {
     for (int d = threadIdx.x; d < a.D; d += 64) out[d] = Elem<T>::store(0.f);
     return;
   }
   const int n = (len + a.chunk - 1) / a.chunk;
-  const int64_t prow = ((int64_t)b * a.QH + qh) * a.nchunks;
+  auto prow = [&](int c) { return partial_row(a, rp, b, qh, c); };
   float mm = -1.0e30f;
-  for (int c = 0; c < n; ++c) mm = fmaxf(mm, a.ws_m[prow + c]);
+  for (int c = 0; c < n; ++c) mm = fmaxf(mm, a.ws_m[prow(c)]);
   float lt = 0.f;
-  for (int c = 0; c < n; ++c) lt = fmaf(a.ws_l[prow + c], exp2f(a.ws_m[prow + c] - mm), lt);
+  for (int c = 0; c < n; ++c) lt = fmaf(a.ws_l[prow(c)], exp2f(a.ws_m[prow(c)] - mm), lt);
   const float inv = 1.0f / fmaxf(lt, 1.0e-20f);
   for (int d = threadIdx.x; d < a.D; d += 64) {
     float o = 0.f;
-    for (int c = 0; c < n; ++c) o = fmaf(a.ws_acc[(prow + c) * a.D + d], exp2f(a.ws_m[prow + c] - mm), o);
+    for (int c = 0; c < n; ++c) o = fmaf(a.ws_acc[prow(c) * a.D + d], exp2f(a.ws_m[prow(c)] - mm), o);
     out[d] = Elem<T>::store(o * inv);
   }
 }
 
 // The same merge for a whole row (all query heads) followed by the row's e4m3 quantisation, for callers whose next
 // step is an FP8 projection: values are rounded to the model dtype first, exactly as the two separate launches do.
-// Sixteen waves per row, wave w owning query heads w, w+16, ...; with NC > 0 the chunk loops are fully unrolled over
-// NC predicated iterations so that all of a lane's partial loads are in flight together (the partials were written
-// by other XCDs and come from beyond the local L2, so each dependent round costs a full memory latency).
+// Sixteen waves per row, wave w owning query heads w, w+16, ...; the chunk loops run in blocks of NC predicated
+// iterations so that a block's partial loads are in flight together (the partials were written by other XCDs and
+// come from beyond the local L2, so each dependent round costs a full memory latency).
 template <typename T, int NC>
 __global__ void __launch_bounds__(1024) decode_combine_fp8_kernel(DecodeArgs a, uint8_t* q_out, float* q_scales) {
   constexpr int kMaxPerLane = 4, kWavesPerRow = 16;
   __shared__ float red[kWavesPerRow];
   const int b = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  int len = a.positions[b] + 1;
-  if (a.active && !a.active[b]) len = 0;
-  if (a.slot_ids && a.slot_ids[b] < 0) len = 0;
+  const RowPairs rp = row_pairs(a, b);
+  const int len = rp.len;
   const int n = len > 0 ? (len + a.chunk - 1) / a.chunk : 0;
   const int per_head = (a.D + 63) / 64;
   float y[kMaxPerLane];
@@ -528,25 +700,41 @@ __global__ void __launch_bounds__(1024) decode_combine_fp8_kernel(DecodeArgs a, 
     const int qh = wave + kWavesPerRow * (i / per_head), d = lane + 64 * (i % per_head);
     y[i] = 0.f;
     if (qh < a.QH && d < a.D && n > 0) {
-      const int64_t prow = ((int64_t)b * a.QH + qh) * a.nchunks;
+      auto prow = [&](int c) { return partial_row(a, rp, b, qh, c); };
       float mm = -1.0e30f, lt = 0.f, o = 0.f;
-      if constexpr (NC > 0) {
-        float m[NC], l[NC], acc[NC];
+      // chunks in blocks of NC whose loads are all in flight together; the sums run in chunk order, exactly as
+      // the plain combine's loops do
+      float m[NC], l[NC], acc[NC];
+      auto load_block = [&](int c0, bool all) {
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
-          const int cc = c < n ? c : 0;
-          m[c] = a.ws_m[prow + cc]; l[c] = a.ws_l[prow + cc]; acc[c] = a.ws_acc[(prow + cc) * a.D + d];
+          const int cc = c0 + c < n ? c0 + c : 0;
+          const int64_t row = prow(cc);
+          m[c] = a.ws_m[row];
+          if (all) { l[c] = a.ws_l[row]; acc[c] = a.ws_acc[row * a.D + d]; }
         }
+      };
+      auto add_block = [&](int c0) {
 #pragma unroll
-        for (int c = 0; c < NC; ++c) if (c < n) mm = fmaxf(mm, m[c]);
+        for (int c = 0; c < NC; ++c)
+          if (c0 + c < n) {
+            const float f = exp2f(m[c] - mm);
+            lt = fmaf(l[c], f, lt);
+            o = fmaf(acc[c], f, o);
+          }
+      };
+      load_block(0, true);
 #pragma unroll
-        for (int c = 0; c < NC; ++c) if (c < n) lt = fmaf(l[c], exp2f(m[c] - mm), lt);
-#pragma unroll
-        for (int c = 0; c < NC; ++c) if (c < n) o = fmaf(acc[c], exp2f(m[c] - mm), o);
+      for (int c = 0; c < NC; ++c) if (c < n) mm = fmaxf(mm, m[c]);
+      if (n <= NC) {
+        add_block(0);
       } else {
-        for (int c = 0; c < n; ++c) mm = fmaxf(mm, a.ws_m[prow + c]);
-        for (int c = 0; c < n; ++c) lt = fmaf(a.ws_l[prow + c], exp2f(a.ws_m[prow + c] - mm), lt);
-        for (int c = 0; c < n; ++c) o = fmaf(a.ws_acc[(prow + c) * a.D + d], exp2f(a.ws_m[prow + c] - mm), o);
+        for (int c = NC; c < n; ++c) mm = fmaxf(mm, a.ws_m[prow(c)]);
+        add_block(0);
+        for (int c0 = NC; c0 < n; c0 += NC) {
+          load_block(c0, true);
+          add_block(c0);
+        }
       }
       y[i] = round_to<T>(o * (1.0f / fmaxf(lt, 1.0e-20f)));
       amax = fmaxf(amax, fabsf(y[i]));
@@ -565,8 +753,7 @@ __global__ void __launch_bounds__(1024) decode_combine_fp8_kernel(DecodeArgs a, 
 
 template <typename T>
 void launch_combine_fp8(const DecodeArgs& a, int64_t B, uint8_t* out_q, float* out_scales, hipStream_t s) {
-  if (a.nchunks <= 8) hipLaunchKernelGGL((decode_combine_fp8_kernel<T, 8>), dim3(B), dim3(1024), 0, s, a, out_q, out_scales);
-  else hipLaunchKernelGGL((decode_combine_fp8_kernel<T, 0>), dim3(B), dim3(1024), 0, s, a, out_q, out_scales);
+  hipLaunchKernelGGL((decode_combine_fp8_kernel<T, 12>), dim3(B), dim3(1024), 0, s, a, out_q, out_scales);
 }
 
 // ===================================================================================== prefill attention
@@ -768,12 +955,13 @@ extern "C" int lfm2_store_kv_packed(const void* k, const void* v, void* k_cache,
   LFM2_LAUNCH_CHECK();
 }
 
+constexpr int kMinChunk = kMfmaChunk < kChunk ? kMfmaChunk : kChunk;
 static int64_t schedule_ints(int64_t B, int64_t capacity) {
-  return 2 + 2 * B * ((capacity + kMfmaChunk - 1) / kMfmaChunk);
+  return kSchedRows + 4 * B + 4 * B * ((capacity + kMfmaChunk - 1) / kMfmaChunk);
 }
 
 extern "C" int64_t lfm2_decode_attention_workspace(int64_t B, int QH, int D, int64_t capacity) {
-  const int64_t nch = (capacity + kChunk - 1) / kChunk;  // the smaller chunk of the two kernels bounds both
+  const int64_t nch = (capacity + kMinChunk - 1) / kMinChunk;  // the smaller chunk of the two kernels bounds both
   return B * QH * nch * (D + 2) + schedule_ints(B, capacity);
 }
 
@@ -818,18 +1006,18 @@ extern "C" int lfm2_decode_attention(void* out, const void* q, const void* k_cac
   a.ws_l = a.ws_m + B * QH * nch;
   a.schedule = nullptr;
   a.max_blocks = max_blocks; a.c0 = c0; a.c1 = c1; a.c2 = c2;
-  a.page = page; a.QH = QH; a.KH = KH; a.D = D; a.G = G; a.nchunks = nch; a.chunk = chunk;
+  a.page = page; a.QH = QH; a.KH = KH; a.D = D; a.G = G; a.nchunks = nch; a.chunk = chunk; a.B = (int)B;
   a.scale_log2e = scale * LFM2_LOG2E;
   hipStream_t s = (hipStream_t)stream;
   if (mfma) {
     if (schedule == nullptr) {  // no shared schedule from the caller: build one in the tail of the workspace
-      int32_t* own = reinterpret_cast<int32_t*>(workspace + B * QH * ((capacity + kChunk - 1) / kChunk) * (D + 2));
+      int32_t* own = reinterpret_cast<int32_t*>(workspace + B * QH * ((capacity + kMinChunk - 1) / kMinChunk) * (D + 2));
       hipLaunchKernelGGL(decode_schedule_kernel, dim3(1), dim3(1024), 0, s, own, positions, active, slot_ids, (int)B, kMfmaChunk);
       schedule = own;
     }
     a.schedule = schedule;
-    // 3 workgroups per CU is what the kernel's register use allows on the 256 CUs; never more than the worst case
-    int64_t blocks = (int64_t)B * nch * KH;
+    // 4 workgroups per CU is what the kernel's register budget (128) allows on the 256 CUs; never more than the worst case
+    int64_t blocks = ((int64_t)B * nch * KH + 3) / 4;
     blocks = blocks < 768 ? blocks : 768;
     const dim3 mgrid((unsigned)blocks);
     if (block_table) hipLaunchKernelGGL(decode_attn_mfma_kernel<true>, mgrid, dim3(256), 0, s, a);

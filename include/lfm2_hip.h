@@ -175,9 +175,9 @@ int lfm2_decode_attention(void* out, const void* q, const void* k_cache, const v
                           void* stream);
 int64_t lfm2_decode_attention_workspace(int64_t B, int QH, int D, int64_t capacity);
 
-/* Work list of the persistent decode-attention kernel: one (row, 1024-token chunk) item per chunk of every active
- * row's history.  It depends only on positions/active/slot_ids, so the attention layers of one decode step can
- * share it (pass it as `schedule`; NULL makes lfm2_decode_attention build its own in the workspace).
+/* Work list of the persistent decode-attention kernel: one (row, 256-token chunk) item per chunk of every active
+ * row's history, longest first.  It depends only on positions/active/slot_ids, so the attention layers of one
+ * decode step can share it (pass it as `schedule`; NULL makes lfm2_decode_attention build its own in the workspace).
  * schedule: int32[lfm2_decode_schedule_size(B, capacity)].  No counterpart in the reference, whose Triton grid is
  * (rows, KV heads, splits) with a fixed split count (lfm25_fp8_kv.py:145-150). */
 int lfm2_decode_schedule(int32_t* schedule, const int32_t* positions, const uint8_t* active, const int32_t* slot_ids,
