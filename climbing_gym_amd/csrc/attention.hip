@@ -366,16 +366,38 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))
   auto fetch = [&](int b, int64_t slot, int h, int T, int wend, Tile& t) {
     int tk = T + lane;
     tk = tk < wend ? tk : wend - 1;
-    const int64_t koff = token_offset(b, slot, h, tk);
+    if (PAGED) {
+      const int64_t koff = token_offset(b, slot, h, tk);
 #pragma unroll
-    for (int c = 0; c < 4; ++c) t.k[c] = *reinterpret_cast<const i32x4*>(kbase + koff + 16 * c);
-    t.sk = a.ks[koff / D];
-    t.sv = a.vs[koff / D];
+      for (int c = 0; c < 4; ++c) t.k[c] = *reinterpret_cast<const i32x4*>(kbase + koff + 16 * c);
+      t.sk = a.ks[koff / D];
+      t.sv = a.vs[koff / D];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      int tv = T + 16 * u + 4 * g16 + g;
-      tv = tv < wend ? tv : wend - 1;
-      t.v[u] = *reinterpret_cast<const i32x4*>(vbase + token_offset(b, slot, h, tv) + 16 * vq);
+      for (int u = 0; u < 4; ++u) {
+        int tv = T + 16 * u + 4 * g16 + g;
+        tv = tv < wend ? tv : wend - 1;
+        t.v[u] = *reinterpret_cast<const i32x4*>(vbase + token_offset(b, slot, h, tv) + 16 * vq);
+      }
+    } else {
+      // the item's base is the same in every lane (scalar registers); a lane adds a 32-bit offset (the host checks
+      // that a slot's history spans less than 2 GiB and that the strides are whole scale rows)
+      const int64_t item_base = slot * a.c0 + (int64_t)h * a.c2;
+      const uint8_t* kitem = kbase + item_base;
+      const uint8_t* vitem = vbase + item_base;
+      const uint32_t koff = (uint32_t)tk * (uint32_t)a.c1;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) t.k[c] = *reinterpret_cast<const i32x4*>(kitem + koff + 16 * c);
+      const float* ks_item = a.ks + item_base / D;
+      const float* vs_item = a.vs + item_base / D;
+      const uint32_t soff = (uint32_t)tk * (uint32_t)(a.c1 / D);
+      t.sk = ks_item[soff];
+      t.sv = vs_item[soff];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        int tv = T + 16 * u + 4 * g16 + g;
+        tv = tv < wend ? tv : wend - 1;
+        t.v[u] = *reinterpret_cast<const i32x4*>(vitem + (uint32_t)tv * (uint32_t)a.c1 + 16 * vq);
+      }
     }
     // this lane's share of the item's queries: head g (clamped into the tensor), dims 4 (lane / 4) .. + 3
     int row = h * a.G + g;
@@ -445,6 +467,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))
           : "=&v"(qraw[0]), "=&v"(qraw[1]), "=&v"(qraw[2]), "=&v"(qraw[3])
           : "v"(q_lds + half * 64)
           : "memory");
+      // keep the conversions of the tile's registers below these reads: the wait for the tile then comes after the
+      // LDS round trip instead of in front of it
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int c = 0; c < 2; ++c)
 #pragma unroll
@@ -995,7 +1020,8 @@ extern "C" int lfm2_decode_attention(void* out, const void* q, const void* k_cac
   const int align = kv_fp8 ? 16 : 8;
   LFM2_REQUIRE(c0 % align == 0 && c1 % align == 0 && c2 % align == 0, "decode_attention: cache strides must be multiples of %d elements", align);
   const int G = QH / KH;
-  const bool mfma = kv_fp8 && D == 64 && G <= 4 && dtype == LFM2_DTYPE_BF16;
+  const bool mfma = kv_fp8 && D == 64 && G <= 4 && dtype == LFM2_DTYPE_BF16 &&
+                    (block_table || (c0 % 64 == 0 && c1 % 64 == 0 && c2 % 64 == 0 && capacity * c1 < (1ll << 31)));
   const int chunk = mfma ? kMfmaChunk : kChunk;
   const int nch = (int)((capacity + chunk - 1) / chunk);
   DecodeArgs a;
