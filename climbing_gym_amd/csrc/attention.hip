@@ -331,12 +331,12 @@ __device__ __forceinline__ int quad_transpose_bytes(int x, int lane) {
 struct ItemRecord { int b, chunk, len, slot; };
 
 template <bool PAGED>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) decode_attn_mfma_kernel(DecodeArgs a) {
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) decode_attn_mfma_kernel(DecodeArgs a) {
   constexpr int D = 64;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // item state lives in scalar registers
   const int g = lane & 3, vq = (lane >> 2) & 3, g16 = lane >> 4;
   __shared__ __bf16 lds_p[4][4][64];   // one P tile per wave; nothing in LDS is shared between waves
-  __shared__ __attribute__((aligned(16))) float lds_o[4][4][4 * D + 4];   // per wave: the four token groups' O[head][dim] (+4: banks)
+  __shared__ __attribute__((aligned(16))) uint8_t lds_v[4][64][D];        // per wave: the tile's V rows, for the transposing read
   __shared__ __attribute__((aligned(16))) __bf16 lds_q[4][4][D];          // per wave: the item's query rows
   const int32_t* const records = a.schedule + kSchedRows + 4 * a.B;
   const int items = a.schedule[0] * a.KH;
@@ -404,8 +404,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))
     row = row < a.QH ? row : a.QH - 1;
     t.q = *reinterpret_cast<const i32x2*>((const __bf16*)a.q + ((int64_t)b * a.QH + row) * D + 4 * (lane >> 2));
   };
-  const uint32_t q_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) __bf16*)&lds_q[wave][g][0];
-  const uint32_t p_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) __bf16*)&lds_p[wave][g][4 * g16];
+  // Operand B of O += P.V needs, per lane, consecutive tokens of one dim, and V rows hold consecutive dims of one
+  // token.  The tile's rows go to LDS as they are and come back through ds_read_b64_tr_b8: within 16 lanes, lane s
+  // receives byte s % 8 of the eight 8-byte pieces that lanes 2j + s / 8 (j = 0..7) point at.  With lane p pointing
+  // at row p / 2, bytes 8 (p % 2) .. + 7 of a 16-dim column block, lane s gets 8 tokens of dim s: lane L of the
+  // wave owns dim L for the whole tile and the item.
+  const int s16 = lane & 15;
+  const uint8_t* v_piece = &lds_v[wave][s16 >> 1][16 * g16 + 8 * (s16 & 1)];
 
   // ---- prologue: the first item, the second item's record, the first tile
   int idx = first, idx_next = first + nwaves;
@@ -423,7 +428,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))
   fetch(b, slot, h, wbeg, wend, tile);
 
   float m[4], l[4];
-  f32x4 acc[4];
+  f32x4 acc;   // O[head 0..3][dim lane]
   int T = wbeg;
   // One tile of the stream: `cur` holds it, the tile after it is fetched into `nxt`.  Returns false after the
   // wave's last item.  (Two calls with the tiles swapped make the loop body, so no tile is ever copied: a copy of
@@ -432,10 +437,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))
     if (T == wbeg) {   // ---- item start: the queries that came with this tile
       *reinterpret_cast<i32x2*>(&lds_q[wave][g][4 * (lane >> 2)]) = cur.q;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) { m[i] = -1.0e30f; l[i] = 0.f; acc[i] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+      for (int i = 0; i < 4; ++i) { m[i] = -1.0e30f; l[i] = 0.f; }
+      acc = f32x4{0.f, 0.f, 0.f, 0.f};
     }
     // ---- the next tile of the stream: this item's, or the first of the next item (its record was asked for one
-    // item ago); without a next item, this item's last tile again
+    // item ago); without a next item, the current tile again (a cache hit)
     const bool last = T + 64 >= wend;
     int nb = b, nlen = len, nh = h, nwbeg = wbeg, nwend = wend;
     int64_t nslot = slot;
@@ -446,7 +452,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))
       nwend = nwbeg + kMfmaChunk;
       nwend = nwend < nlen ? nwend : nlen;
     }
-    const int fT = last ? nwbeg : T + 64;
+    const int fT = last ? (have_next ? nwbeg : T) : T + 64;
     fetch(nb, nslot, nh, fT, nwend, nxt);
 
     const bool valid = T + lane < wend;
@@ -456,29 +462,18 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))
     // computed and never stored).
     f32x4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int half = 0; half < 2; ++half) {   // two reads of 64 bytes: half the registers of one of 128
-      i32x4 qraw[4];
-      asm volatile(
-          "ds_read_b128 %0, %4\n\t"
-          "ds_read_b128 %1, %4 offset:16\n\t"
-          "ds_read_b128 %2, %4 offset:32\n\t"
-          "ds_read_b128 %3, %4 offset:48\n\t"
-          "s_waitcnt lgkmcnt(0)"
-          : "=&v"(qraw[0]), "=&v"(qraw[1]), "=&v"(qraw[2]), "=&v"(qraw[3])
-          : "v"(q_lds + half * 64)
-          : "memory");
-      // keep the conversions of the tile's registers below these reads: the wait for the tile then comes after the
-      // LDS round trip instead of in front of it
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int c = 0; c < 2; ++c)
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          const i32x4 q4 = qraw[2 * c + (w >> 1)];
-          const i32x2 q2 = {q4[2 * (w & 1)], q4[2 * (w & 1) + 1]};
-          s = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, q2), e4m3x4_to_bf16x4(cur.k[2 * half + c][w]), s, 0, 0, 0);
-        }
+    for (int c = 0; c < 4; ++c) {
+      const i32x4 q4 = *reinterpret_cast<const i32x4*>(&lds_q[wave][g][16 * c]);       // dims 16c .. 16c+7
+      const i32x4 q5 = *reinterpret_cast<const i32x4*>(&lds_q[wave][g][16 * c + 8]);   // dims 16c+8 .. 16c+15
+      const i32x2 qa = {q4[0], q4[1]}, qb = {q4[2], q4[3]}, qc = {q5[0], q5[1]}, qd = {q5[2], q5[3]};
+      s = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, qa), e4m3x4_to_bf16x4(cur.k[c][0]), s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, qb), e4m3x4_to_bf16x4(cur.k[c][1]), s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, qc), e4m3x4_to_bf16x4(cur.k[c][2]), s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, qd), e4m3x4_to_bf16x4(cur.k[c][3]), s, 0, 0, 0);
     }
+    // the tile's V rows to LDS, as they arrived (row = token, 16 bytes per lane)
+#pragma unroll
+    for (int u = 0; u < 4; ++u) *reinterpret_cast<i32x4*>(&lds_v[wave][16 * u + 4 * g16 + g][16 * vq]) = cur.v[u];
     const float kscale = a.scale_log2e * sk;
     bool raise = false;
 #pragma unroll
@@ -493,8 +488,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))
         const float alpha = __builtin_amdgcn_exp2f(m[i] - mnew);
         m[i] = mnew;
         l[i] *= alpha;
-#pragma unroll
-        for (int w = 0; w < 4; ++w) acc[w][i] *= alpha;
+        acc[i] *= alpha;
       }
     }
 #pragma unroll
@@ -503,61 +497,40 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))
       l[i] += p;
       lds_p[wave][i][lane] = (__bf16)(p * sv);
     }
-    // ---- O[0..3][dims 16*vq + 4w + g] += P . V over this lane group's tokens
-    i32x2 praw[4];
-    asm volatile(
-        "ds_read_b64 %0, %4\n\t"
-        "ds_read_b64 %1, %4 offset:32\n\t"
-        "ds_read_b64 %2, %4 offset:64\n\t"
-        "ds_read_b64 %3, %4 offset:96\n\t"
-        "s_waitcnt lgkmcnt(0)"
-        : "=&v"(praw[0]), "=&v"(praw[1]), "=&v"(praw[2]), "=&v"(praw[3])
-        : "v"(p_lds)
-        : "memory");
+    // ---- O[0..3][dim lane] += P . V, eight tokens per transposing read
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const s16x4 pop = __builtin_bit_cast(s16x4, praw[u]);
+    for (int tb = 0; tb < 8; ++tb) {
+      const i32x2 vt = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+          (__attribute__((address_space(3))) i32x2*)(v_piece + tb * 8 * D));
 #pragma unroll
-      for (int w = 0; w < 4; ++w)
-        acc[w] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(pop, e4m3x4_to_bf16x4(quad_transpose_bytes(cur.v[u][w], lane)), acc[w], 0, 0, 0);
+      for (int half = 0; half < 2; ++half) {
+        const i32x2 praw = *reinterpret_cast<const i32x2*>(&lds_p[wave][g][8 * tb + 4 * half]);
+        acc = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, praw), e4m3x4_to_bf16x4(vt[half]), acc, 0, 0, 0);
+      }
     }
     T += 64;
     if (!last) return true;
 
-    // ---- item end.  Wave totals: l over all lanes; O over the four token groups through LDS, which also turns the
-    // MFMA layout (lane = 4 dims apart) into rows: lane L ends with O[head L/16][dims 4(L%16)..+3] and the item's
-    // heads leave as one contiguous block of 16 bytes per lane
+    // ---- item end.  Wave totals of l; lane L holds O[head 0..3][dim L], so a head's row leaves as 256 contiguous bytes
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      l[i] = wave_sum(l[i]);
-#pragma unroll
-      for (int w = 0; w < 4; ++w) lds_o[wave][g16][i * D + 16 * vq + 4 * w + g] = acc[w][i];
-    }
+    for (int i = 0; i < 4; ++i) l[i] = wave_sum(l[i]);
+    // The partial results leave through hand-written stores.  Reads and writes share one counter and complete out
+    // of order with respect to each other, so with a store it knows of in flight the compiler turns every wait for
+    // a load into a wait for everything, which would stop the stream at each item.  Unknown to it, a pending store
+    // only makes a counted wait stricter: loads still complete in order among themselves.
     {
-      const int i = lane >> 4, d4 = 4 * (lane & 15);
-      f32x4 o = *reinterpret_cast<const f32x4*>(&lds_o[wave][0][i * D + d4]);
-#pragma unroll
-      for (int t = 1; t < 4; ++t) {
-        const f32x4 part_o = *reinterpret_cast<const f32x4*>(&lds_o[wave][t][i * D + d4]);
-        o[0] += part_o[0]; o[1] += part_o[1]; o[2] += part_o[2]; o[3] += part_o[3];
-      }
       const int64_t prow = (int64_t)(idx / a.KH) * a.QH + h * a.G;
-      if (i < a.G) *reinterpret_cast<f32x4*>(a.ws_acc + (prow + i) * D + d4) = o;
-      if (lane == 0) {   // the heads' maxima and sums: wave-uniform, sixteen bytes each for a full group
-        if (a.G == 4) {
-          *reinterpret_cast<f32x4*>(a.ws_m + prow) = f32x4{m[0], m[1], m[2], m[3]};
-          *reinterpret_cast<f32x4*>(a.ws_l + prow) = f32x4{l[0], l[1], l[2], l[3]};
-        } else {
-          a.ws_m[prow] = m[0]; a.ws_l[prow] = l[0];
-          if (a.G > 1) { a.ws_m[prow + 1] = m[1]; a.ws_l[prow + 1] = l[1]; }
-          if (a.G > 2) { a.ws_m[prow + 2] = m[2]; a.ws_l[prow + 2] = l[2]; }
-        }
+      float* dst = a.ws_acc + prow * D + lane;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (i < a.G) asm volatile("global_store_dword %0, %1, off" : : "v"(dst + i * D), "v"(acc[i]) : "memory");
+      if (lane < a.G) {   // the heads' maxima and sums are the same in every lane: lane i stores head i's
+        const float mv = lane == 0 ? m[0] : lane == 1 ? m[1] : lane == 2 ? m[2] : m[3];
+        const float lv = lane == 0 ? l[0] : lane == 1 ? l[1] : lane == 2 ? l[2] : l[3];
+        asm volatile("global_store_dword %0, %1, off" : : "v"(a.ws_m + prow + lane), "v"(mv) : "memory");
+        asm volatile("global_store_dword %0, %1, off" : : "v"(a.ws_l + prow + lane), "v"(lv) : "memory");
       }
     }
-    // Reads and writes share one counter and complete out of order with respect to each other, so with a store in
-    // flight every wait for a load becomes a wait for everything.  Let the stores finish here, where the only
-    // loads in flight are the next item's first tile and queries, which are needed next anyway.
-    __builtin_amdgcn_s_waitcnt(0 | (0x7 << 4) | (0xF << 8));
     // ---- step to the next item; ask for the record of the one after it
     if (!have_next) return false;
     idx = idx_next;
@@ -1042,7 +1015,8 @@ extern "C" int lfm2_decode_attention(void* out, const void* q, const void* k_cac
       schedule = own;
     }
     a.schedule = schedule;
-    // 4 workgroups per CU is what the kernel's register budget (128) allows on the 256 CUs; never more than the worst case
+    // 3 workgroups per CU (the register budget of 128 would allow 4, but with a handful of items per wave more
+    // waves only make the shares of work more unequal); never more than the worst case
     int64_t blocks = ((int64_t)B * nch * KH + 3) / 4;
     blocks = blocks < 768 ? blocks : 768;
     const dim3 mgrid((unsigned)blocks);
