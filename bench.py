@@ -68,20 +68,26 @@ def time_decode_attention(engine, session, samples):
     positions = (cache.seq_lens - 1).clamp_min(0).contiguous()
     active = torch.ones(rows, device="cuda", dtype=torch.bool)
     schedule = ops.decode_schedule(positions, active, capacity=cache.max_seq_len) if cache.fp8 else None
+    # the decode step's form of the call: rows come back e4m3-quantised when the out projection is W8A8
+    attention_ops = [l.attention for l in engine.weights.layers if l.attention is not None]
+    quantized = bool(cache.fp8 and attention_ops and id(attention_ops[0].out_weight) in engine._fp8()
+                     and -(-cfg.num_attention_heads // 16) * -(-cfg.head_dim // 64) <= 4)
     stream = torch.cuda.current_stream()
-    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     total_ms, launches = 0.0, 0
     for layer in range(cache.k_cache.size(0)):
         args = (q, cache.k_cache[layer], cache.v_cache[layer],
                 None if cache.k_scales is None else cache.k_scales[layer],
                 None if cache.v_scales is None else cache.v_scales[layer], positions)
-        ops.attend(*args, active=active, scale=engine._scaling, schedule=schedule)  # warm
-        begin.record(stream)
-        for _ in range(samples):
-            ops.attend(*args, active=active, scale=engine._scaling, schedule=schedule)
-        end.record(stream)
-        end.synchronize()
-        total_ms += begin.elapsed_time(end)
+        ops.attend(*args, active=active, scale=engine._scaling, schedule=schedule, quantized=quantized)  # warm
+        # one pair of events per call: a marker between two calls also keeps the next call's first waves from
+        # starting under the tail of this one, which a kernel trace would count twice
+        marks = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(samples)]
+        for begin, end in marks:
+            begin.record(stream)
+            ops.attend(*args, active=active, scale=engine._scaling, schedule=schedule, quantized=quantized)
+            end.record(stream)
+        marks[-1][1].synchronize()
+        total_ms += sum(begin.elapsed_time(end) for begin, end in marks)
         launches += samples
     tokens = int((positions.long() + 1).sum())
     kv_token = cfg.num_key_value_heads * cfg.head_dim * 2 * (1 if cache.fp8 else 2) + (cfg.num_key_value_heads * 2 * 4 if cache.fp8 else 0)
@@ -241,7 +247,7 @@ def main():
                    "context_tokens": ctx_tokens, "prefill_tok_per_s": round(sum(map(len, prompts)) / prefill_s, 1),
                    "gemm": gemms, "step_algorithmic_bytes": step_bytes,
                    "step_hbm_fraction": round(step_bytes / (ms_per_step / 1000) / 1e9 / HBM_PEAK_GBS, 4)},
-        "roofline": {"kernel": "decode_attn_mfma_kernel + decode_combine_kernel (one ragged GQA decode-attention call, e4m3 KV)"
+        "roofline": {"kernel": "decode_attn_mfma_kernel + decode_combine_fp8_kernel (one ragged GQA decode-attention call, e4m3 KV, rows quantised for the W8A8 out projection as in the decode step)"
                                if fp8 else "decode_attn_kernel + decode_combine_kernel (bf16 KV)",
                      "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(args, attn_bytes),
