@@ -29,8 +29,14 @@ extern "C" int lfm2_abi_version(void) { return 1; }
     default: LFM2_FAIL(LFM2_ERR_ARGUMENT, "unknown dtype %d", dtype);      \
   }
 
+#ifndef ROW_THREADS
+#define ROW_THREADS 512
+#endif
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / 64;
+// The per-row kernels (RMSNorm, row quantisation): threads per row
+constexpr int kRowThreads = ROW_THREADS;
+constexpr int kRowWaves = kRowThreads / 64;
 
 template <typename T> struct Vec {
   static constexpr int N = 16 / sizeof(T);
@@ -101,10 +107,10 @@ struct SplitInput {
 };
 
 template <typename T, int NV, bool ADD, bool FP8>
-__global__ void __launch_bounds__(kThreads)
+__global__ void __launch_bounds__(kRowThreads)
 rms_norm_kernel(T* out, uint8_t* q, float* scales, T* summed, const T* x, const T* w, const T* res, int64_t H,
                 float eps, SplitInput split) {
-  __shared__ float red[kWaves];
+  __shared__ float red[kRowWaves];
   const int64_t row = blockIdx.x;
   constexpr int N = Vec<T>::N;
   x += row * H;
@@ -116,7 +122,7 @@ rms_norm_kernel(T* out, uint8_t* q, float* scales, T* summed, const T* x, const 
     float ss = 0.f;
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
-      const int64_t i = (int64_t)(j * kThreads + threadIdx.x) * N;
+      const int64_t i = (int64_t)(j * kRowThreads + threadIdx.x) * N;
       if (i < H) {
         if (split.partial) {
           const float sa = split.a_scales[row];
@@ -147,15 +153,15 @@ rms_norm_kernel(T* out, uint8_t* q, float* scales, T* summed, const T* x, const 
     float g[NV][N];
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
-      const int64_t i = (int64_t)(j * kThreads + threadIdx.x) * N;
+      const int64_t i = (int64_t)(j * kRowThreads + threadIdx.x) * N;
       if (i < H) load_vec<T>(w + i, g[j]);
     }
-    ss = block_sum<kWaves>(ss, red);
+    ss = block_sum<kRowWaves>(ss, red);
     const float rstd = 1.0f / sqrtf(ss / (float)H + eps);
     float amax = 0.f;
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
-      const int64_t i = (int64_t)(j * kThreads + threadIdx.x) * N;
+      const int64_t i = (int64_t)(j * kRowThreads + threadIdx.x) * N;
       if (i < H) {
 #pragma unroll
         for (int e = 0; e < N; ++e) {
@@ -166,12 +172,12 @@ rms_norm_kernel(T* out, uint8_t* q, float* scales, T* summed, const T* x, const 
       }
     }
     if (FP8) {
-      amax = block_max<kWaves>(amax, red);
+      amax = block_max<kRowWaves>(amax, red);
       const float scale = fmaxf(amax / LFM2_E4M3_MAX, 1.0e-12f);
       if (threadIdx.x == 0) scales[row] = scale;
 #pragma unroll
       for (int j = 0; j < NV; ++j) {
-        const int64_t i = (int64_t)(j * kThreads + threadIdx.x) * N;
+        const int64_t i = (int64_t)(j * kRowThreads + threadIdx.x) * N;
         if (i < H) store_e4m3<N>(q + i, v[j], scale);
       }
     }
@@ -182,26 +188,26 @@ rms_norm_kernel(T* out, uint8_t* q, float* scales, T* summed, const T* x, const 
       return a;
     };
     float ss = 0.f;
-    for (int64_t i = threadIdx.x; i < H; i += kThreads) {
+    for (int64_t i = threadIdx.x; i < H; i += kRowThreads) {
       const float a = value(i);
       if (ADD) summed[i] = Elem<T>::store(a);
       ss += a * a;
     }
-    ss = block_sum<kWaves>(ss, red);
+    ss = block_sum<kRowWaves>(ss, red);
     const float rstd = 1.0f / sqrtf(ss / (float)H + eps);
     auto normed = [&](int64_t i) {
       float n = round_to<T>(value(i) * rstd) * Elem<T>::load(w[i]);
       return FP8 ? round_to<T>(n) : n;
     };
     if (!FP8) {
-      for (int64_t i = threadIdx.x; i < H; i += kThreads) out[i] = Elem<T>::store(normed(i));
+      for (int64_t i = threadIdx.x; i < H; i += kRowThreads) out[i] = Elem<T>::store(normed(i));
     } else {
       float amax = 0.f;
-      for (int64_t i = threadIdx.x; i < H; i += kThreads) amax = fmaxf(amax, fabsf(normed(i)));
-      amax = block_max<kWaves>(amax, red);
+      for (int64_t i = threadIdx.x; i < H; i += kRowThreads) amax = fmaxf(amax, fabsf(normed(i)));
+      amax = block_max<kRowWaves>(amax, red);
       const float scale = fmaxf(amax / LFM2_E4M3_MAX, 1.0e-12f);
       if (threadIdx.x == 0) scales[row] = scale;
-      for (int64_t i = threadIdx.x; i < H; i += kThreads) q[i] = to_e4m3(normed(i) / scale);
+      for (int64_t i = threadIdx.x; i < H; i += kRowThreads) q[i] = to_e4m3(normed(i) / scale);
     }
   }
 }
@@ -211,7 +217,7 @@ template <typename T> static int pick_nv(int64_t width) {
   constexpr int N = 16 / sizeof(T);
   if (width % N != 0) return 0;
   for (int nv = 1; nv <= 16; nv *= 2)
-    if ((int64_t)nv * kThreads * N >= width) return nv;
+    if ((int64_t)nv * kRowThreads * N >= width) return nv;
   return 0;
 }
 
@@ -231,7 +237,7 @@ static void launch_rms(void* out, uint8_t* q, float* scales, void* summed, const
                        SplitInput split = SplitInput{nullptr, nullptr, nullptr, 0, 0}) {
   const int nv = pick_nv<T>(H);
 #define RMS_(NVV)                                                                                            \
-  hipLaunchKernelGGL((rms_norm_kernel<T, NVV, ADD, FP8>), dim3(M), dim3(kThreads), 0, s, (T*)out, q, scales, \
+  hipLaunchKernelGGL((rms_norm_kernel<T, NVV, ADD, FP8>), dim3(M), dim3(kRowThreads), 0, s, (T*)out, q, scales, \
                      (T*)summed, (const T*)x, (const T*)w, (const T*)res, H, eps, split)
   LAUNCH_NV(nv, RMS_(1), RMS_(2), RMS_(4), RMS_(8), RMS_(16), RMS_(0));
 #undef RMS_
@@ -264,7 +270,7 @@ extern "C" int lfm2_rms_norm_fp8_split(uint8_t* q, float* scales, void* summed, 
   LFM2_REQUIRE(partial && a_scales && w_scales && splits >= 1, "rms_norm_fp8_split: partial products and both scale vectors are required");
   LFM2_REQUIRE(residual == nullptr || summed != nullptr, "rms_norm_fp8_split: residual given without a summed output");
   const int vec = dtype == LFM2_DTYPE_F32 ? 4 : 8;
-  LFM2_REQUIRE(H % vec == 0 && H <= (int64_t)16 * kThreads * vec, "rms_norm_fp8_split: width %ld is not a multiple of %d or too wide", (long)H, vec);
+  LFM2_REQUIRE(H % vec == 0 && H <= (int64_t)16 * kRowThreads * vec, "rms_norm_fp8_split: width %ld is not a multiple of %d or too wide", (long)H, vec);
   const SplitInput split{partial, a_scales, w_scales, M * H, splits};
   hipStream_t s = (hipStream_t)stream;
   DISPATCH_DTYPE(dtype, if (residual) launch_rms<T, true, true>(nullptr, q, scales, summed, nullptr, weight, residual, M, H, eps, s, split);
@@ -310,8 +316,8 @@ extern "C" int lfm2_swiglu(void* out, const void* x, int64_t M, int64_t I, int d
 
 // SWIGLU = false gives plain row quantisation of x[M,K].
 template <typename T, int NV, bool SWIGLU>
-__global__ void __launch_bounds__(kThreads) quantize_kernel(uint8_t* q, float* scales, const T* x, int64_t K) {
-  __shared__ float red[kWaves];
+__global__ void __launch_bounds__(kRowThreads) quantize_kernel(uint8_t* q, float* scales, const T* x, int64_t K) {
+  __shared__ float red[kRowWaves];
   const int64_t row = blockIdx.x;
   constexpr int N = Vec<T>::N;
   const T* a = x + row * (SWIGLU ? 2 * K : K);
@@ -322,7 +328,7 @@ __global__ void __launch_bounds__(kThreads) quantize_kernel(uint8_t* q, float* s
     float v[NV][N];
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
-      const int64_t i = (int64_t)(j * kThreads + threadIdx.x) * N;
+      const int64_t i = (int64_t)(j * kRowThreads + threadIdx.x) * N;
       if (i < K) {
         load_vec<T>(a + i, v[j]);
         if (SWIGLU) {
@@ -335,12 +341,12 @@ __global__ void __launch_bounds__(kThreads) quantize_kernel(uint8_t* q, float* s
         for (int e = 0; e < N; ++e) amax = fmaxf(amax, fabsf(v[j][e]));
       }
     }
-    amax = block_max<kWaves>(amax, red);
+    amax = block_max<kRowWaves>(amax, red);
     const float scale = fmaxf(amax / LFM2_E4M3_MAX, 1.0e-12f);
     if (threadIdx.x == 0) scales[row] = scale;
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
-      const int64_t i = (int64_t)(j * kThreads + threadIdx.x) * N;
+      const int64_t i = (int64_t)(j * kRowThreads + threadIdx.x) * N;
       if (i < K) store_e4m3<N>(q + i, v[j], scale);
     }
   } else {
@@ -348,11 +354,11 @@ __global__ void __launch_bounds__(kThreads) quantize_kernel(uint8_t* q, float* s
       float g = Elem<T>::load(a[i]);
       return SWIGLU ? round_to<T>(round_to<T>(silu_f(g)) * Elem<T>::load(b[i])) : g;
     };
-    for (int64_t i = threadIdx.x; i < K; i += kThreads) amax = fmaxf(amax, fabsf(value(i)));
-    amax = block_max<kWaves>(amax, red);
+    for (int64_t i = threadIdx.x; i < K; i += kRowThreads) amax = fmaxf(amax, fabsf(value(i)));
+    amax = block_max<kRowWaves>(amax, red);
     const float scale = fmaxf(amax / LFM2_E4M3_MAX, 1.0e-12f);
     if (threadIdx.x == 0) scales[row] = scale;
-    for (int64_t i = threadIdx.x; i < K; i += kThreads) q[i] = to_e4m3(value(i) / scale);
+    for (int64_t i = threadIdx.x; i < K; i += kRowThreads) q[i] = to_e4m3(value(i) / scale);
   }
 }
 
@@ -360,7 +366,7 @@ template <typename T, bool SWIGLU>
 static void launch_quantize(uint8_t* q, float* scales, const void* x, int64_t M, int64_t K, hipStream_t s) {
   const int nv = pick_nv<T>(K);
 #define Q_(NVV) \
-  hipLaunchKernelGGL((quantize_kernel<T, NVV, SWIGLU>), dim3(M), dim3(kThreads), 0, s, q, scales, (const T*)x, K)
+  hipLaunchKernelGGL((quantize_kernel<T, NVV, SWIGLU>), dim3(M), dim3(kRowThreads), 0, s, q, scales, (const T*)x, K)
   LAUNCH_NV(nv, Q_(1), Q_(2), Q_(4), Q_(8), Q_(16), Q_(0));
 #undef Q_
 }
