@@ -183,6 +183,13 @@ class LFM25Engine:
             self._cuda_decoder.clear()
         self._cuda_decoder = None
 
+    def compile_decode(self, *, mode: str = "reduce-overhead", fullgraph: bool = False) -> None:
+        """The reference compiles its eager decode step with a tracing compiler here (lfm25_engine.py:972-978).  This
+        engine has no such step to compile: the same request turns on HIP-graph capture of the kernel sequence."""
+        del mode, fullgraph
+        if self._cuda_decoder is None:
+            self.enable_cuda_graphs()
+
     def release_inference_buffers(self) -> None:
         decoder = self._cuda_decoder
         if decoder is None:
