@@ -331,6 +331,82 @@ def test_decode_matches_independent_fp32_softmax_with_ragged_lengths_and_inactiv
     assert torch.count_nonzero(moved[3]) == 0
 
 
+@torch.inference_mode()
+def test_work_list_lists_every_chunk_once_longest_first(ops):
+    """Layout of the decode-attention work list: pair count; a record per row (first full pair, partial pair,
+    length or 0 for rows that sit out); a record per pair (row, chunk, length, slot), full 256-token chunks first,
+    then partial chunks of 4, 3, 2, 1 tiles.  1500 rows: more than one block of the device scan."""
+    torch.manual_seed(3)
+    rows, chunk = 1500, 256
+    lengths = torch.randint(1, 3000, (rows,))
+    lengths[:8] = torch.tensor([1, 64, 65, 256, 257, 512, 2999, 255])
+    active = torch.rand(rows) > 0.1
+    slots = torch.randperm(rows).to(torch.int32)
+    slots[torch.rand(rows) < 0.05] = -1
+    schedule = ops.decode_schedule((lengths - 1).to(torch.int32).to(DEV), active.to(DEV), slots.to(DEV), capacity=3072).cpu()
+    live = active & (slots >= 0)
+    eff = torch.where(live, lengths, torch.zeros_like(lengths))
+    pairs = int((eff + chunk - 1).div(chunk, rounding_mode="floor").sum())
+    assert int(schedule[0]) == pairs
+    row_rec = schedule[4:4 + 4 * rows].view(rows, 4)
+    pair_rec = schedule[4 + 4 * rows:4 + 4 * rows + 4 * pairs].view(pairs, 4)
+    assert torch.equal(row_rec[:, 2].long(), eff)
+    # every (row, chunk) exactly once, with the row's length and slot
+    seen = set()
+    for r, c, n, slot in pair_rec.tolist():
+        assert live[r] and n == int(lengths[r]) and slot == int(slots[r]) and 0 <= c * chunk < n
+        assert (r, c) not in seen
+        seen.add((r, c))
+    assert len(seen) == pairs
+    # order: tiles per item never increase
+    tiles = [min(chunk, n - c * chunk + 0) for r, c, n, s in pair_rec.tolist()]
+    tiles = [(t + 63) // 64 for t in tiles]
+    assert tiles == sorted(tiles, reverse=True)
+    # the rows' records point at their pairs
+    for r in torch.nonzero(live).flatten().tolist()[:200]:
+        n = int(lengths[r])
+        for c in range(n // chunk):
+            assert pair_rec[int(row_rec[r, 0]) + c].tolist()[:2] == [r, c]
+        if n % chunk:
+            assert pair_rec[int(row_rec[r, 1])].tolist()[:2] == [r, n // chunk]
+
+
+@pytest.mark.parametrize("quantized", [False, True])
+@torch.inference_mode()
+def test_decode_over_more_rows_than_one_scan_block(ops, quantized):
+    """1100 rows (the device scan of the work list handles 1024 per block) with lengths across the chunk and tile
+    boundaries, inactive rows and slot indirection, against the oracle on sampled rows."""
+    torch.manual_seed(17)
+    rows, capacity, heads, groups, dim = 1100, 600, 8, 4, 64
+    k = torch.randn(rows, capacity, heads, dim).bfloat16()
+    v = torch.randn_like(k)
+    q = torch.randn(rows, 1, heads * groups, dim).bfloat16()
+    lengths = torch.randint(1, capacity + 1, (rows,))
+    lengths[:6] = torch.tensor([1, 64, 256, 257, 512, 600])
+    active = torch.rand(rows) > 0.1
+    slots = torch.randperm(rows).to(torch.int32)
+    kc, vc, ks, vs = _cache_tensors(rows, capacity, heads, dim, "HND")
+    ops.store_kv(k.to(DEV), v.to(DEV), kc, vc, ks, vs)
+    hist = (kc.cpu(), vc.cpu(), ks.cpu(), vs.cpu())
+    positions = (lengths[slots.long()] - 1).to(torch.int32)     # row i reads slot slots[i]
+    out = ops.attend(q.to(DEV), kc, vc, ks, vs, positions.to(DEV), active=active.to(DEV), slot_ids=slots.to(DEV),
+                     quantized=quantized)
+    if quantized:
+        codes, scales = out
+        result = (codes.float() * scales[:, None]).view(rows, heads * groups, dim).cpu()
+    else:
+        result = out[:, 0].float().cpu()
+    for row in [0, 1, 2, 3, 4, 5, 511, 1023, 1024, 1025, 1099]:
+        if not active[row]:
+            assert torch.count_nonzero(result[row]) == 0
+            continue
+        slot = int(slots[row])
+        expected = O.k_attend(q[row, 0], hist[0][slot], hist[1][slot], int(lengths[slot]), dim ** -0.5, hist[2][slot], hist[3][slot])
+        tolerance = dict(atol=0.05, rtol=0.07) if quantized else dict(atol=0.012, rtol=0.025)   # e4m3 rows: 1/16 relative steps
+        torch.testing.assert_close(result[row], expected, **tolerance)
+    assert torch.count_nonzero(result[~active]) == 0
+
+
 @pytest.mark.parametrize("fp8", [True, False])
 @torch.inference_mode()
 def test_paged_slot_mapped_history_equals_dense_history(ops, fp8):
