@@ -247,8 +247,8 @@ def main():
                    "context_tokens": ctx_tokens, "prefill_tok_per_s": round(sum(map(len, prompts)) / prefill_s, 1),
                    "gemm": gemms, "step_algorithmic_bytes": step_bytes,
                    "step_hbm_fraction": round(step_bytes / (ms_per_step / 1000) / 1e9 / HBM_PEAK_GBS, 4)},
-        "roofline": {"kernel": "decode_attn_mfma_kernel + decode_combine_fp8_kernel (one ragged GQA decode-attention call, e4m3 KV, rows quantised for the W8A8 out projection as in the decode step)"
-                               if fp8 else "decode_attn_kernel + decode_combine_kernel (bf16 KV)",
+        "roofline": {"kernel": "decode_attn_mfma_kernel + decode_combine_row_kernel (one ragged GQA decode-attention call, e4m3 KV, rows quantised for the W8A8 out projection as in the decode step)"
+                               if fp8 else "decode_attn_mfma_kernel + decode_combine_row_kernel (one ragged GQA decode-attention call, bf16 KV)",
                      "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(args, attn_bytes),
                      "avg_launch_us": round(attn_s * 1e6, 2), "algorithmic_bytes_per_launch": attn_bytes},

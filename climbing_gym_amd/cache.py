@@ -2,10 +2,10 @@
 
 Layout in HBM (one allocation per tensor, all layers of a kind together):
 
-  bf16 KV : k, v          [attn layers, slots, capacity, KV heads, D]
-  e4m3 KV : k, v bytes    [attn layers, slots, KV heads, capacity, D]   (each head's history is
-            scales fp32   [attn layers, slots, KV heads, capacity]       contiguous: 64 B / token)
-            exposed through [.., capacity, KV heads, ..] views so both layouts index alike
+  bf16 KV : k, v          [attn layers, slots, KV heads, capacity, D]   (each head's history is contiguous:
+  e4m3 KV : k, v bytes    [attn layers, slots, KV heads, capacity, D]    128 or 64 B / token, so the decode
+            scales fp32   [attn layers, slots, KV heads, capacity]       kernel streams whole DRAM pages)
+            exposed through [.., capacity, KV heads, ..] views, the index order of the reference's cache
   conv    : state         [conv layers, slots, H, 3]   (index 2 = newest tap)
   seq_lens: int32 [slots]
 """
@@ -37,7 +37,7 @@ class LFM25HybridCache:
             make = lambda: torch.zeros((*shape, head_dim), device=device, dtype=torch.float8_e4m3fn).permute(0, 1, 3, 2, 4)
             scale = lambda: torch.zeros(shape, device=device, dtype=torch.float32).permute(0, 1, 3, 2)
             return cls(make(), make(), conv, lens, scale(), scale())
-        make = lambda: torch.zeros((attn_layers, slots, capacity, kv_heads, head_dim), device=device, dtype=dtype)
+        make = lambda: torch.zeros((attn_layers, slots, kv_heads, capacity, head_dim), device=device, dtype=dtype).permute(0, 1, 3, 2, 4)
         return cls(make(), make(), conv, lens)
 
     def rows(self, start: int, end: int) -> "LFM25HybridCache":

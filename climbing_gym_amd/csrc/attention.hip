@@ -330,13 +330,15 @@ __device__ __forceinline__ int quad_transpose_bytes(int x, int lane) {
 // and nothing is loaded straight into LDS (with such a load in flight the compiler waits for all loads at once).
 struct ItemRecord { int b, chunk, len, slot; };
 
-template <bool PAGED>
+template <bool PAGED, bool FP8>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) decode_attn_mfma_kernel(DecodeArgs a) {
   constexpr int D = 64;
+  constexpr int TT = FP8 ? 64 : 32;   // tokens per tile: 4 KiB of K rows and 4 KiB of V rows either way
+  constexpr int ES = FP8 ? 1 : 2;     // bytes per element of the history
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // item state lives in scalar registers
   const int g = lane & 3, vq = (lane >> 2) & 3, g16 = lane >> 4;
   __shared__ __bf16 lds_p[4][4][64];   // one P tile per wave; nothing in LDS is shared between waves
-  __shared__ __attribute__((aligned(16))) uint8_t lds_v[4][64][D];        // per wave: the tile's V rows, for the transposing read
+  __shared__ __attribute__((aligned(16))) uint8_t lds_v[4][TT][D * ES];   // per wave: the tile's V rows, for the transposing read
   __shared__ __attribute__((aligned(16))) __bf16 lds_q[4][4][D];          // per wave: the item's query rows
   const int32_t* const records = a.schedule + kSchedRows + 4 * a.B;
   const int items = a.schedule[0] * a.KH;
@@ -362,43 +364,55 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
   const uint8_t* kbase = (const uint8_t*)a.kc;
   const uint8_t* vbase = (const uint8_t*)a.vc;
   struct Tile { i32x4 k[4], v[4]; float sk, sv; i32x2 q; };
-  // this lane's K row, its scales, and its four V slices of the tile at T (tokens clamped to the item's last)
+  // this lane's K row, its scales, and its four V slices of the tile at T (tokens clamped to the item's last).
+  // e4m3 history: lane L owns token L of 64 (a 64-byte row) and the V slices of tokens 16u + L / 16 * 4 + L % 4.
+  // 16-bit history: lane L owns dims 32 (L / 32) .. + 31 of token L % 32 (64 bytes of a 128-byte row) and 16 bytes
+  // of the V rows of tokens 8u + L / 8.
+  const int tl = FP8 ? lane : (lane & 31);              // this lane's token within a tile
+  const int krow_byte = FP8 ? 0 : 64 * (lane >> 5);     // where its share of a K row starts
+  const int vtok = FP8 ? 4 * g16 + g : (lane >> 3), vstep = FP8 ? 16 : 8, vbyte = FP8 ? 16 * vq : 16 * (lane & 7);
   auto fetch = [&](int b, int64_t slot, int h, int T, int wend, Tile& t) {
-    int tk = T + lane;
+    int tk = T + tl;
     tk = tk < wend ? tk : wend - 1;
     if (PAGED) {
       const int64_t koff = token_offset(b, slot, h, tk);
 #pragma unroll
-      for (int c = 0; c < 4; ++c) t.k[c] = *reinterpret_cast<const i32x4*>(kbase + koff + 16 * c);
-      t.sk = a.ks[koff / D];
-      t.sv = a.vs[koff / D];
+      for (int c = 0; c < 4; ++c) t.k[c] = *reinterpret_cast<const i32x4*>(kbase + koff * ES + krow_byte + 16 * c);
+      if constexpr (FP8) {
+        t.sk = a.ks[koff / D];
+        t.sv = a.vs[koff / D];
+      }
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        int tv = T + 16 * u + 4 * g16 + g;
+        int tv = T + vstep * u + vtok;
         tv = tv < wend ? tv : wend - 1;
-        t.v[u] = *reinterpret_cast<const i32x4*>(vbase + token_offset(b, slot, h, tv) + 16 * vq);
+        t.v[u] = *reinterpret_cast<const i32x4*>(vbase + token_offset(b, slot, h, tv) * ES + vbyte);
       }
     } else {
       // the item's base is the same in every lane (scalar registers); a lane adds a 32-bit offset (the host checks
       // that a slot's history spans less than 2 GiB and that the strides are whole scale rows)
       const int64_t item_base = slot * a.c0 + (int64_t)h * a.c2;
-      const uint8_t* kitem = kbase + item_base;
-      const uint8_t* vitem = vbase + item_base;
-      const uint32_t koff = (uint32_t)tk * (uint32_t)a.c1;
+      const uint8_t* kitem = kbase + item_base * ES;
+      const uint8_t* vitem = vbase + item_base * ES;
+      const uint32_t row_bytes = (uint32_t)a.c1 * ES;
+      const uint32_t koff = (uint32_t)tk * row_bytes + krow_byte;
 #pragma unroll
       for (int c = 0; c < 4; ++c) t.k[c] = *reinterpret_cast<const i32x4*>(kitem + koff + 16 * c);
-      const float* ks_item = a.ks + item_base / D;
-      const float* vs_item = a.vs + item_base / D;
-      const uint32_t soff = (uint32_t)tk * (uint32_t)(a.c1 / D);
-      t.sk = ks_item[soff];
-      t.sv = vs_item[soff];
+      if constexpr (FP8) {
+        const float* ks_item = a.ks + item_base / D;
+        const float* vs_item = a.vs + item_base / D;
+        const uint32_t soff = (uint32_t)tk * (uint32_t)(a.c1 / D);
+        t.sk = ks_item[soff];
+        t.sv = vs_item[soff];
+      }
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        int tv = T + 16 * u + 4 * g16 + g;
+        int tv = T + vstep * u + vtok;
         tv = tv < wend ? tv : wend - 1;
-        t.v[u] = *reinterpret_cast<const i32x4*>(vitem + (uint32_t)tv * (uint32_t)a.c1 + 16 * vq);
+        t.v[u] = *reinterpret_cast<const i32x4*>(vitem + (uint32_t)tv * row_bytes + vbyte);
       }
     }
+    if constexpr (!FP8) { t.sk = 1.f; t.sv = 1.f; }
     // this lane's share of the item's queries: head g (clamped into the tensor), dims 4 (lane / 4) .. + 3
     int row = h * a.G + g;
     row = row < a.QH ? row : a.QH - 1;
@@ -409,8 +423,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
   // receives byte s % 8 of the eight 8-byte pieces that lanes 2j + s / 8 (j = 0..7) point at.  With lane p pointing
   // at row p / 2, bytes 8 (p % 2) .. + 7 of a 16-dim column block, lane s gets 8 tokens of dim s: lane L of the
   // wave owns dim L for the whole tile and the item.
+  // The 16-bit form, ds_read_b64_tr_b16, gives lane s element s % 4 of the four 8-byte pieces that lanes
+  // 4j + s / 4 (j = 0..3) point at: with lane p pointing at row p / 4, bytes 8 (p % 4) .. + 7 of a 16-dim column
+  // block, lane s gets 4 tokens of dim s.
   const int s16 = lane & 15;
-  const uint8_t* v_piece = &lds_v[wave][s16 >> 1][16 * g16 + 8 * (s16 & 1)];
+  const uint8_t* v_piece = FP8 ? &lds_v[wave][s16 >> 1][16 * g16 + 8 * (s16 & 1)]
+                               : &lds_v[wave][s16 >> 2][32 * g16 + 8 * (s16 & 3)];
 
   // ---- prologue: the first item, the second item's record, the first tile
   int idx = first, idx_next = first + nwaves;
@@ -442,7 +460,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
     }
     // ---- the next tile of the stream: this item's, or the first of the next item (its record was asked for one
     // item ago); without a next item, the current tile again (a cache hit)
-    const bool last = T + 64 >= wend;
+    const bool last = T + TT >= wend;
     int nb = b, nlen = len, nh = h, nwbeg = wbeg, nwend = wend;
     int64_t nslot = slot;
     const bool have_next = last && idx_next < items;
@@ -452,15 +470,30 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
       nwend = nwbeg + kMfmaChunk;
       nwend = nwend < nlen ? nwend : nlen;
     }
-    const int fT = last ? (have_next ? nwbeg : T) : T + 64;
+    const int fT = last ? (have_next ? nwbeg : T) : T + TT;
     fetch(nb, nslot, nh, fT, nwend, nxt);
 
-    const bool valid = T + lane < wend;
+    const bool valid = T + tl < wend;
     const float sk = cur.sk, sv = cur.sv;
     // ---- S[0..3][token lane].  A operand: Q[head g][dims 4s..4s+3] for s = 0..15, read from LDS for every tile
     // rather than held in 32 registers (rows beyond the group hold a neighbouring head's queries: their results are
     // computed and never stored).
     f32x4 s = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (!FP8) {
+      // 16-bit history: a lane's K registers hold dims 32 (lane / 32) + 8c .. + 7; the two halves of the wave each
+      // sum over their 32 dims and exchange the sums
+      const __bf16* qrow = &lds_q[wave][g][32 * (lane >> 5)];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const i32x4 q8 = *reinterpret_cast<const i32x4*>(qrow + 8 * c);
+        const i32x2 qa = {q8[0], q8[1]}, qb = {q8[2], q8[3]};
+        const i32x2 ka = {cur.k[c][0], cur.k[c][1]}, kb = {cur.k[c][2], cur.k[c][3]};
+        s = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, qa), __builtin_bit_cast(s16x4, ka), s, 0, 0, 0);
+        s = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, qb), __builtin_bit_cast(s16x4, kb), s, 0, 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) s[i] = add_lane_xor32(s[i]);
+    } else {
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       const i32x4 q4 = *reinterpret_cast<const i32x4*>(&lds_q[wave][g][16 * c]);       // dims 16c .. 16c+7
@@ -471,10 +504,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
       s = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, qc), e4m3x4_to_bf16x4(cur.k[c][2]), s, 0, 0, 0);
       s = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, qd), e4m3x4_to_bf16x4(cur.k[c][3]), s, 0, 0, 0);
     }
+    }
     // the tile's V rows to LDS, as they arrived (row = token, 16 bytes per lane)
 #pragma unroll
-    for (int u = 0; u < 4; ++u) *reinterpret_cast<i32x4*>(&lds_v[wave][16 * u + 4 * g16 + g][16 * vq]) = cur.v[u];
-    const float kscale = a.scale_log2e * sk;
+    for (int u = 0; u < 4; ++u) *reinterpret_cast<i32x4*>(&lds_v[wave][vstep * u + vtok][vbyte]) = cur.v[u];
+    const float kscale = FP8 ? a.scale_log2e * sk : a.scale_log2e;
     bool raise = false;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -494,10 +528,24 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const float p = valid ? __builtin_amdgcn_exp2f(s[i] - m[i]) : 0.f;
-      l[i] += p;
-      lds_p[wave][i][lane] = (__bf16)(p * sv);
+      if constexpr (FP8) {
+        l[i] += p;
+        lds_p[wave][i][lane] = (__bf16)(p * sv);
+      } else {   // both halves of the wave hold the tile's 32 probabilities: count them once
+        l[i] += lane < 32 ? p : 0.f;
+        lds_p[wave][i][tl] = (__bf16)p;
+      }
     }
-    // ---- O[0..3][dim lane] += P . V, eight tokens per transposing read
+    // ---- O[0..3][dim lane] += P . V, eight (e4m3) or four (16-bit) tokens per transposing read
+    if constexpr (!FP8) {
+#pragma unroll
+      for (int tb = 0; tb < 8; ++tb) {
+        const s16x4 vt = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) s16x4*)(v_piece + tb * 4 * D * ES));
+        const i32x2 praw = *reinterpret_cast<const i32x2*>(&lds_p[wave][g][4 * tb]);
+        acc = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, praw), vt, acc, 0, 0, 0);
+      }
+    } else {
 #pragma unroll
     for (int tb = 0; tb < 8; ++tb) {
       const i32x2 vt = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
@@ -508,7 +556,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
         acc = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, praw), e4m3x4_to_bf16x4(vt[half]), acc, 0, 0, 0);
       }
     }
-    T += 64;
+    }
+    T += TT;
     if (!last) return true;
 
     // ---- item end.  Wave totals of l; lane L holds O[head 0..3][dim L], so a head's row leaves as 256 contiguous bytes
@@ -677,13 +726,14 @@ __global__ void __launch_bounds__(64) decode_combine_kernel(DecodeArgs a) {
   }
 }
 
-// The same merge for a whole row (all query heads) followed by the row's e4m3 quantisation, for callers whose next
-// step is an FP8 projection: values are rounded to the model dtype first, exactly as the two separate launches do.
+// The same merge for a whole row (all query heads), for rows of at most 4096 values; with QUANT followed by the row's
+// e4m3 quantisation, for callers whose next step is an FP8 projection: values are rounded to the model dtype first,
+// exactly as the two separate launches do.
 // Sixteen waves per row, wave w owning query heads w, w+16, ...; the chunk loops run in blocks of NC predicated
 // iterations so that a block's partial loads are in flight together (the partials were written by other XCDs and
 // come from beyond the local L2, so each dependent round costs a full memory latency).
-template <typename T, int NC>
-__global__ void __launch_bounds__(1024) decode_combine_fp8_kernel(DecodeArgs a, uint8_t* q_out, float* q_scales) {
+template <typename T, int NC, bool QUANT>
+__global__ void __launch_bounds__(1024) decode_combine_row_kernel(DecodeArgs a, uint8_t* q_out, float* q_scales) {
   constexpr int kMaxPerLane = 4, kWavesPerRow = 16;
   __shared__ float red[kWavesPerRow];
   const int b = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -738,6 +788,15 @@ __global__ void __launch_bounds__(1024) decode_combine_fp8_kernel(DecodeArgs a, 
       amax = fmaxf(amax, fabsf(y[i]));
     }
   }
+  if constexpr (!QUANT) {
+    T* out = (T*)a.out + (int64_t)b * a.QH * a.D;
+#pragma unroll
+    for (int i = 0; i < kMaxPerLane; ++i) {
+      const int qh = wave + kWavesPerRow * (i / per_head), d = lane + 64 * (i % per_head);
+      if (qh < a.QH && d < a.D) out[qh * a.D + d] = Elem<T>::store(y[i]);
+    }
+    return;
+  }
   amax = block_max<kWavesPerRow>(amax, red);
   const float scale = fmaxf(amax / LFM2_E4M3_MAX, 1.0e-12f);
   if (threadIdx.x == 0) q_scales[b] = scale;
@@ -751,7 +810,15 @@ __global__ void __launch_bounds__(1024) decode_combine_fp8_kernel(DecodeArgs a, 
 
 template <typename T>
 void launch_combine_fp8(const DecodeArgs& a, int64_t B, uint8_t* out_q, float* out_scales, hipStream_t s) {
-  hipLaunchKernelGGL((decode_combine_fp8_kernel<T, 12>), dim3(B), dim3(1024), 0, s, a, out_q, out_scales);
+  hipLaunchKernelGGL((decode_combine_row_kernel<T, 12, true>), dim3(B), dim3(1024), 0, s, a, out_q, out_scales);
+}
+// The merge alone: a row per workgroup when the row fits the row kernel's registers, a (row, head) per wave otherwise.
+template <typename T>
+void launch_combine(const DecodeArgs& a, int64_t B, hipStream_t s) {
+  if ((int64_t)((a.QH + 15) / 16) * ((a.D + 63) / 64) <= 4)
+    hipLaunchKernelGGL((decode_combine_row_kernel<T, 12, false>), dim3(B), dim3(1024), 0, s, a, nullptr, nullptr);
+  else
+    hipLaunchKernelGGL(decode_combine_kernel<T>, dim3(B, a.QH), dim3(64), 0, s, a);
 }
 
 // ===================================================================================== prefill attention
@@ -993,8 +1060,11 @@ extern "C" int lfm2_decode_attention(void* out, const void* q, const void* k_cac
   const int align = kv_fp8 ? 16 : 8;
   LFM2_REQUIRE(c0 % align == 0 && c1 % align == 0 && c2 % align == 0, "decode_attention: cache strides must be multiples of %d elements", align);
   const int G = QH / KH;
-  const bool mfma = kv_fp8 && D == 64 && G <= 4 && dtype == LFM2_DTYPE_BF16 &&
-                    (block_table || (c0 % 64 == 0 && c1 % 64 == 0 && c2 % 64 == 0 && capacity * c1 < (1ll << 31)));
+  // The scheduled kernel: head_dim 64, a GQA group of at most 4, bf16 queries, and an e4m3 or bf16 history whose
+  // rows it can address with 32-bit byte offsets within a slot (paged histories are addressed per token).
+  const bool mfma = D == 64 && G <= 4 && dtype == LFM2_DTYPE_BF16 &&
+                    (block_table || (kv_fp8 ? c0 % 64 == 0 && c1 % 64 == 0 && c2 % 64 == 0 && capacity * c1 < (1ll << 31)
+                                            : capacity * c1 * 2 < (1ll << 31)));
   const int chunk = mfma ? kMfmaChunk : kChunk;
   const int nch = (int)((capacity + chunk - 1) / chunk);
   DecodeArgs a;
@@ -1020,10 +1090,15 @@ extern "C" int lfm2_decode_attention(void* out, const void* q, const void* k_cac
     int64_t blocks = ((int64_t)B * nch * KH + 3) / 4;
     blocks = blocks < 768 ? blocks : 768;
     const dim3 mgrid((unsigned)blocks);
-    if (block_table) hipLaunchKernelGGL(decode_attn_mfma_kernel<true>, mgrid, dim3(256), 0, s, a);
-    else hipLaunchKernelGGL(decode_attn_mfma_kernel<false>, mgrid, dim3(256), 0, s, a);
+    if (kv_fp8) {
+      if (block_table) hipLaunchKernelGGL((decode_attn_mfma_kernel<true, true>), mgrid, dim3(256), 0, s, a);
+      else hipLaunchKernelGGL((decode_attn_mfma_kernel<false, true>), mgrid, dim3(256), 0, s, a);
+    } else {
+      if (block_table) hipLaunchKernelGGL((decode_attn_mfma_kernel<true, false>), mgrid, dim3(256), 0, s, a);
+      else hipLaunchKernelGGL((decode_attn_mfma_kernel<false, false>), mgrid, dim3(256), 0, s, a);
+    }
     if (out_q) launch_combine_fp8<__bf16>(a, B, out_q, out_scales, s);
-    else hipLaunchKernelGGL(decode_combine_kernel<__bf16>, dim3(B, QH), dim3(64), 0, s, a);
+    else launch_combine<__bf16>(a, B, s);
     LFM2_LAUNCH_CHECK();
   }
   const dim3 grid(nch, KH * ((G + kGB - 1) / kGB), B);
@@ -1036,7 +1111,7 @@ extern "C" int lfm2_decode_attention(void* out, const void* q, const void* k_cac
     case 128: DEC_(128); break;
     default: DEC_(256); break;
   } if (out_q) launch_combine_fp8<T>(a, B, out_q, out_scales, s);
-    else hipLaunchKernelGGL(decode_combine_kernel<T>, dim3(B, QH), dim3(64), 0, s, a));
+    else launch_combine<T>(a, B, s));
 #undef DEC_
   LFM2_LAUNCH_CHECK();
 }

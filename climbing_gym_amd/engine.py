@@ -295,7 +295,7 @@ class LFM25Engine:
         positions = cache.seq_lens if positions is None else positions
         rows = tokens.numel()
         # the attention layers of one step see the same lengths: build the work list of the attention kernel once
-        schedule = ops.decode_schedule(positions, active, slot_ids, capacity=cache.max_seq_len) if cache.fp8 else None
+        schedule = ops.decode_schedule(positions, active, slot_ids, capacity=cache.max_seq_len)
 
         def attention_op(op, qkv):
             # QK norm + RoPE with the new token's keys and values written straight into the cache, then attention over

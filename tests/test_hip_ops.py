@@ -372,22 +372,31 @@ def test_work_list_lists_every_chunk_once_longest_first(ops):
 
 
 @pytest.mark.parametrize("quantized", [False, True])
+@pytest.mark.parametrize("fp8", [True, False])
 @torch.inference_mode()
-def test_decode_over_more_rows_than_one_scan_block(ops, quantized):
+def test_decode_over_more_rows_than_one_scan_block(ops, quantized, fp8):
     """1100 rows (the device scan of the work list handles 1024 per block) with lengths across the chunk and tile
-    boundaries, inactive rows and slot indirection, against the oracle on sampled rows."""
+    boundaries, inactive rows and slot indirection, against the oracle on sampled rows; e4m3 history (64-token
+    tiles) and bf16 history stored head-major (32-token tiles)."""
     torch.manual_seed(17)
     rows, capacity, heads, groups, dim = 1100, 600, 8, 4, 64
     k = torch.randn(rows, capacity, heads, dim).bfloat16()
     v = torch.randn_like(k)
     q = torch.randn(rows, 1, heads * groups, dim).bfloat16()
     lengths = torch.randint(1, capacity + 1, (rows,))
-    lengths[:6] = torch.tensor([1, 64, 256, 257, 512, 600])
+    lengths[:10] = torch.tensor([1, 64, 256, 257, 512, 600, 31, 32, 33, 289])
     active = torch.rand(rows) > 0.1
     slots = torch.randperm(rows).to(torch.int32)
-    kc, vc, ks, vs = _cache_tensors(rows, capacity, heads, dim, "HND")
-    ops.store_kv(k.to(DEV), v.to(DEV), kc, vc, ks, vs)
-    hist = (kc.cpu(), vc.cpu(), ks.cpu(), vs.cpu())
+    picked = [int(torch.nonzero(slots == i)[0]) for i in range(10)]     # the rows that read the hand-picked lengths
+    active[picked] = True
+    if fp8:
+        kc, vc, ks, vs = _cache_tensors(rows, capacity, heads, dim, "HND")
+        ops.store_kv(k.to(DEV), v.to(DEV), kc, vc, ks, vs)
+        hist = (kc.cpu(), vc.cpu(), ks.cpu(), vs.cpu())
+    else:
+        head_major = lambda t: t.to(DEV).permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+        kc, vc, ks, vs = head_major(k), head_major(v), None, None
+        hist = (k, v, [None] * rows, [None] * rows)
     positions = (lengths[slots.long()] - 1).to(torch.int32)     # row i reads slot slots[i]
     out = ops.attend(q.to(DEV), kc, vc, ks, vs, positions.to(DEV), active=active.to(DEV), slot_ids=slots.to(DEV),
                      quantized=quantized)
@@ -396,7 +405,7 @@ def test_decode_over_more_rows_than_one_scan_block(ops, quantized):
         result = (codes.float() * scales[:, None]).view(rows, heads * groups, dim).cpu()
     else:
         result = out[:, 0].float().cpu()
-    for row in [0, 1, 2, 3, 4, 5, 511, 1023, 1024, 1025, 1099]:
+    for row in picked + [0, 1, 2, 3, 4, 5, 511, 1023, 1024, 1025, 1099]:
         if not active[row]:
             assert torch.count_nonzero(result[row]) == 0
             continue
