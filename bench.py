@@ -41,7 +41,97 @@ def parse_args():
     p.add_argument("--cpu-seqs", type=int, default=4, help="sequences of the workload the CPU baseline runs (0 = skip)")
     p.add_argument("--cpu-steps", type=int, default=8)
     p.add_argument("--attn-samples", type=int, default=20, help="timed launches of the decode-attention kernel per layer")
+    p.add_argument("--workload", choices=("decode", "attention"), default="decode",
+                   help="decode: the model's decode step (the headline metric); attention: the decode-attention call alone "
+                        "on 256 sequences of U[128, 8192] history tokens, dense and paged (block 16), e4m3 and bf16")
     return p.parse_args()
+
+
+def attention_workload(args):
+    """One ragged GQA decode-attention call (split kernel + combine) on 256 sequences with U[128, 8192] history tokens,
+    32 query heads over 8 KV heads of 64 dims: history stored dense (each head's tokens contiguous) and in 16-token
+    pages reached through a shuffled block table (pages token-major and head-major), e4m3 with scales and bf16.
+    Paged results must equal the dense ones bit for bit."""
+    from climbing_gym_amd import ops
+    rows, kv_heads, heads, dim, capacity, page = 256, 8, 32, 64, 8192, 16
+    lengths = torch.randint(128, capacity + 1, (rows,), generator=torch.Generator().manual_seed(0))
+    positions = (lengths - 1).to(torch.int32).cuda()
+    torch.manual_seed(0)
+    q = torch.randn(rows, 1, heads, dim, device="cuda", dtype=torch.bfloat16)
+    schedule = ops.decode_schedule(positions, None, None, capacity=capacity)
+    tokens = int(lengths.sum())
+    results = {}
+
+    def timed(name, bytes_per_token, call):
+        for _ in range(max(1, args.warmup // 4)):
+            call()
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        begin.record()
+        for _ in range(args.steps):
+            call()
+        end.record()
+        end.synchronize()
+        us = begin.elapsed_time(end) * 1000 / args.steps
+        alg = tokens * bytes_per_token + 2 * rows * heads * dim * 2
+        results[name] = {"us_per_call": round(us, 2), "GB/s": round(alg / us / 1e3, 1), "algorithmic_bytes": alg}
+
+    blocks = capacity // page
+    order = torch.randperm(rows * blocks, device="cuda")
+    table = order.view(rows, blocks).to(torch.int32)
+
+    def to_pages(t):   # [rows, capacity, ...] -> pool [pages, page, ...] under the block table
+        src = t.contiguous().reshape(rows * blocks, page, *t.shape[2:])
+        pool = torch.empty_like(src)
+        if t.dtype == torch.float8_e4m3fn:
+            pool.view(torch.uint8)[order] = src.view(torch.uint8)
+        else:
+            pool[order] = src
+        return pool
+
+    def head_major(t):   # the same pages with each head's tokens contiguous inside a page
+        rest = range(3, t.ndim)
+        return t.permute(0, 2, 1, *rest).contiguous().permute(0, 2, 1, *rest)
+
+    for fp8 in (True, False):
+        name = "e4m3" if fp8 else "bf16"
+        shape = (rows, kv_heads, capacity, dim)
+        if fp8:
+            make = lambda: torch.randint(0, 120, shape, device="cuda", dtype=torch.uint8).view(torch.float8_e4m3fn).permute(0, 2, 1, 3)
+            k, v = make(), make()
+            ks, vs = ((torch.rand(shape[:3], device="cuda") * 0.01).permute(0, 2, 1) for _ in range(2))
+        else:
+            k, v = (torch.randn(shape, device="cuda", dtype=torch.bfloat16).permute(0, 2, 1, 3) for _ in range(2))
+            ks = vs = None
+        per_token = 2 * kv_heads * dim * (1 if fp8 else 2) + (2 * kv_heads * 4 if fp8 else 0)
+        timed(f"{name} dense", per_token, lambda: ops.attend(q, k, v, ks, vs, positions, schedule=schedule))
+        dense = ops.attend(q, k, v, ks, vs, positions, schedule=schedule)
+        pk, pv = to_pages(k), to_pages(v)
+        pks, pvs = (None, None) if ks is None else (to_pages(ks), to_pages(vs))
+        del k, v
+        paged = lambda: ops.attend(q, pk, pv, pks, pvs, positions, block_table=table, page=page, schedule=schedule)
+        timed(f"{name} paged, token-major pages", per_token, paged)
+        same = torch.equal(paged(), dense)
+        pk, pv = head_major(pk), head_major(pv)
+        if pks is not None:
+            pks, pvs = head_major(pks), head_major(pvs)
+        timed(f"{name} paged, head-major pages", per_token, paged)
+        same = same and torch.equal(paged(), dense)
+        if not same:
+            raise SystemExit(f"paged {name} attention differs from dense")
+        del pk, pv, pks, pvs
+        torch.cuda.empty_cache()
+    head = results["e4m3 dense"]
+    print(json.dumps({
+        "metric": "decode attention algorithmic GB/s @256 ragged seqs, history U[128,8192], e4m3 KV", "value": head["GB/s"],
+        "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": max(1, args.warmup // 4),
+        "ms_per_step": round(head["us_per_call"] / 1000, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp8_e4m3 history, bf16 queries, fp32 accumulate", "data": "synthetic",
+        "config": {"workload": "one decode-attention call: 256 sequences, history U[128,8192] tokens, 32 query / 8 KV heads x 64, "
+                               "dense and 16-token pages, e4m3 + scales and bf16", "context_tokens": tokens, "variants": results},
+        "roofline": {"kernel": "decode_attn_mfma_kernel + decode_combine_row_kernel", "bound": "hbm", "achieved": head["GB/s"],
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(head["GB/s"] / HBM_PEAK_GBS, 4), "traffic": None},
+        "cpu_baseline": None}))
 
 
 def build_engine(args, state):
@@ -203,6 +293,10 @@ def main():
         print(f"bench.py measures one MI355X; --gpus {args.gpus} is not supported in this build "
               "(the path shards by slots across independent engines with no collective in the step).", file=sys.stderr)
         sys.exit(2)
+    if args.workload == "attention":
+        with torch.inference_mode():
+            attention_workload(args)
+        return
     from climbing_gym_amd.config import LFM25SamplingConfig
     from climbing_gym_amd.synthetic import LFM2_1P2B, random_prompts, random_state_dict
 

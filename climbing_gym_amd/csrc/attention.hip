@@ -728,10 +728,12 @@ __global__ void __launch_bounds__(64) decode_combine_kernel(DecodeArgs a) {
 
 // The same merge for a whole row (all query heads), for rows of at most 4096 values; with QUANT followed by the row's
 // e4m3 quantisation, for callers whose next step is an FP8 projection: values are rounded to the model dtype first,
-// exactly as the two separate launches do.
-// Sixteen waves per row, wave w owning query heads w, w+16, ...; the chunk loops run in blocks of NC predicated
-// iterations so that a block's partial loads are in flight together (the partials were written by other XCDs and
-// come from beyond the local L2, so each dependent round costs a full memory latency).
+// exactly as a separate quantisation of the stored row would.
+// Sixteen waves per row, wave w owning query heads w, w+16, ...; a lane owns one dim of a head.  The partials were
+// written by other XCDs and come from beyond the local L2, so every dependent round of loads costs a full memory
+// latency: a chunk's maximum and sum are loaded by the lane of the chunk's index (the chunks' weights
+// exp2(m_c - max) are then one exp2 per lane, read back lane by lane as scalars), and the accumulator loads do not
+// depend on them, so a row of up to NC chunks has every load of its merge in flight at once.
 template <typename T, int NC, bool QUANT>
 __global__ void __launch_bounds__(1024) decode_combine_row_kernel(DecodeArgs a, uint8_t* q_out, float* q_scales) {
   constexpr int kMaxPerLane = 4, kWavesPerRow = 16;
@@ -741,82 +743,95 @@ __global__ void __launch_bounds__(1024) decode_combine_row_kernel(DecodeArgs a, 
   const int len = rp.len;
   const int n = len > 0 ? (len + a.chunk - 1) / a.chunk : 0;
   const int per_head = (a.D + 63) / 64;
-  float y[kMaxPerLane];
-  float amax = 0.f;
+  auto head_of = [&](int i) { return wave + kWavesPerRow * (i / per_head); };
+  auto dim_of = [&](int i) { return lane + 64 * (i % per_head); };
+  auto owned = [&](int i) { return head_of(i) < a.QH && dim_of(i) < a.D; };   // dim_of < D can differ per lane only when D % 64 != 0
+  auto weight_of = [&](float f, int c) {   // lane c's value, the same for every lane
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, f), c));
+  };
+  float y[kMaxPerLane] = {0.f, 0.f, 0.f, 0.f};
+  if (n > 0 && n <= NC) {
+    float mv[kMaxPerLane], lv[kMaxPerLane], accv[kMaxPerLane][NC];
 #pragma unroll
-  for (int i = 0; i < kMaxPerLane; ++i) {
-    const int qh = wave + kWavesPerRow * (i / per_head), d = lane + 64 * (i % per_head);
-    y[i] = 0.f;
-    if (qh < a.QH && d < a.D && n > 0) {
-      auto prow = [&](int c) { return partial_row(a, rp, b, qh, c); };
-      float mm = -1.0e30f, lt = 0.f, o = 0.f;
-      // chunks in blocks of NC whose loads are all in flight together; the sums run in chunk order, exactly as
-      // the plain combine's loops do
-      float m[NC], l[NC], acc[NC];
-      auto load_block = [&](int c0, bool all) {
+    for (int i = 0; i < kMaxPerLane; ++i) {
+      const int qh = head_of(i) < a.QH ? head_of(i) : a.QH - 1, d = dim_of(i) < a.D ? dim_of(i) : a.D - 1;
+      if (head_of(i) < a.QH) {   // the same for the whole wave
+        const int64_t mine = partial_row(a, rp, b, qh, lane < n ? lane : 0);
+        mv[i] = a.ws_m[mine];
+        lv[i] = a.ws_l[mine];
 #pragma unroll
-        for (int c = 0; c < NC; ++c) {
-          const int cc = c0 + c < n ? c0 + c : 0;
-          const int64_t row = prow(cc);
-          m[c] = a.ws_m[row];
-          if (all) { l[c] = a.ws_l[row]; acc[c] = a.ws_acc[row * a.D + d]; }
-        }
-      };
-      auto add_block = [&](int c0) {
+        for (int c = 0; c < NC; ++c) accv[i][c] = a.ws_acc[partial_row(a, rp, b, qh, c < n ? c : 0) * a.D + d];
+      }
+    }
 #pragma unroll
-        for (int c = 0; c < NC; ++c)
-          if (c0 + c < n) {
-            const float f = exp2f(m[c] - mm);
-            lt = fmaf(l[c], f, lt);
-            o = fmaf(acc[c], f, o);
-          }
-      };
-      load_block(0, true);
+    for (int i = 0; i < kMaxPerLane; ++i) {
+      if (head_of(i) < a.QH) {
+        const float mm = wave_max(lane < n ? mv[i] : -1.0e30f);
+        const float f = lane < n ? exp2f(mv[i] - mm) : 0.f;
+        const float lt = wave_sum(lv[i] * f);
+        float o = 0.f;
 #pragma unroll
-      for (int c = 0; c < NC; ++c) if (c < n) mm = fmaxf(mm, m[c]);
-      if (n <= NC) {
-        add_block(0);
-      } else {
-        for (int c = NC; c < n; ++c) mm = fmaxf(mm, a.ws_m[prow(c)]);
-        add_block(0);
-        for (int c0 = NC; c0 < n; c0 += NC) {
-          load_block(c0, true);
-          add_block(c0);
+        for (int c = 0; c < NC; ++c) o = fmaf(accv[i][c], weight_of(f, c), o);   // chunks past the row's: weight 0
+        y[i] = round_to<T>(o * (1.0f / fmaxf(lt, 1.0e-20f)));
+      }
+    }
+  } else if (n > 0) {
+    // longer rows: the chunks' maxima and sums in groups of 64 (one per lane), the accumulators in blocks of NC
+    for (int i = 0; i < kMaxPerLane; ++i) {
+      if (head_of(i) >= a.QH) break;
+      const int qh = head_of(i), d = dim_of(i) < a.D ? dim_of(i) : a.D - 1;
+      float mm = -1.0e30f;
+      for (int c0 = 0; c0 < n; c0 += 64)
+        if (c0 + lane < n) mm = fmaxf(mm, a.ws_m[partial_row(a, rp, b, qh, c0 + lane)]);
+      mm = wave_max(mm);
+      float lt = 0.f, o = 0.f;
+      for (int c0 = 0; c0 < n; c0 += 64) {
+        const bool mine = c0 + lane < n;
+        const int64_t row = partial_row(a, rp, b, qh, mine ? c0 + lane : 0);
+        const float f = mine ? exp2f(a.ws_m[row] - mm) : 0.f;
+        lt = fmaf(a.ws_l[row], f, lt);
+        const int group = n - c0 < 64 ? n - c0 : 64;
+        for (int cb = 0; cb < group; cb += NC) {
+          float accv[NC];
+#pragma unroll
+          for (int c = 0; c < NC; ++c) accv[c] = a.ws_acc[partial_row(a, rp, b, qh, c0 + cb + c < n ? c0 + cb + c : 0) * a.D + d];
+#pragma unroll
+          for (int c = 0; c < NC; ++c) o = fmaf(accv[c], cb + c < 64 ? weight_of(f, cb + c) : 0.f, o);
         }
       }
+      lt = wave_sum(lt);
       y[i] = round_to<T>(o * (1.0f / fmaxf(lt, 1.0e-20f)));
-      amax = fmaxf(amax, fabsf(y[i]));
     }
   }
   if constexpr (!QUANT) {
     T* out = (T*)a.out + (int64_t)b * a.QH * a.D;
 #pragma unroll
-    for (int i = 0; i < kMaxPerLane; ++i) {
-      const int qh = wave + kWavesPerRow * (i / per_head), d = lane + 64 * (i % per_head);
-      if (qh < a.QH && d < a.D) out[qh * a.D + d] = Elem<T>::store(y[i]);
-    }
+    for (int i = 0; i < kMaxPerLane; ++i)
+      if (owned(i)) out[head_of(i) * a.D + dim_of(i)] = Elem<T>::store(y[i]);
     return;
   }
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < kMaxPerLane; ++i)
+    if (owned(i)) amax = fmaxf(amax, fabsf(y[i]));
   amax = block_max<kWavesPerRow>(amax, red);
   const float scale = fmaxf(amax / LFM2_E4M3_MAX, 1.0e-12f);
   if (threadIdx.x == 0) q_scales[b] = scale;
   uint8_t* dst = q_out + (int64_t)b * a.QH * a.D;
 #pragma unroll
-  for (int i = 0; i < kMaxPerLane; ++i) {
-    const int qh = wave + kWavesPerRow * (i / per_head), d = lane + 64 * (i % per_head);
-    if (qh < a.QH && d < a.D) dst[qh * a.D + d] = to_e4m3(y[i] / scale);
-  }
+  for (int i = 0; i < kMaxPerLane; ++i)
+    if (owned(i)) dst[head_of(i) * a.D + dim_of(i)] = to_e4m3(y[i] / scale);
 }
 
 template <typename T>
 void launch_combine_fp8(const DecodeArgs& a, int64_t B, uint8_t* out_q, float* out_scales, hipStream_t s) {
-  hipLaunchKernelGGL((decode_combine_row_kernel<T, 12, true>), dim3(B), dim3(1024), 0, s, a, out_q, out_scales);
+  hipLaunchKernelGGL((decode_combine_row_kernel<T, 16, true>), dim3(B), dim3(1024), 0, s, a, out_q, out_scales);
 }
 // The merge alone: a row per workgroup when the row fits the row kernel's registers, a (row, head) per wave otherwise.
 template <typename T>
 void launch_combine(const DecodeArgs& a, int64_t B, hipStream_t s) {
   if ((int64_t)((a.QH + 15) / 16) * ((a.D + 63) / 64) <= 4)
-    hipLaunchKernelGGL((decode_combine_row_kernel<T, 12, false>), dim3(B), dim3(1024), 0, s, a, nullptr, nullptr);
+    hipLaunchKernelGGL((decode_combine_row_kernel<T, 16, false>), dim3(B), dim3(1024), 0, s, a, nullptr, nullptr);
   else
     hipLaunchKernelGGL(decode_combine_kernel<T>, dim3(B, a.QH), dim3(64), 0, s, a);
 }
