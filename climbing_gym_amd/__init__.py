@@ -7,6 +7,7 @@ Reference module -> module of this package:
   inference/lfm25_session.py       -> session.py
   inference/text_stops.py          -> text_stops.py
   inference/lfm25_async_engine.py  -> async_engine.py;  inference/config.py, types.py -> inference_config.py, types.py
+  inference/benchmark.py           -> benchmark.py;     rollout/{runner,config,contracts,coordinator}.py -> rollout.py
 """
 from .config import LFM2Config, LFM25SamplingConfig
 
@@ -14,7 +15,8 @@ __all__ = ["LFM2Config", "LFM25SamplingConfig", "LFM25Engine", "LFM25PackedWeigh
            "LFM25PrefixBatch", "LFM25DecodeBatch", "LFM25StepOutput", "LFM25GenerationOutput", "LFM25HIPDecoder",
            "LFM25CUDADecoder", "LFM25GenerationSession", "LFM25ContinuationHandle", "LFM25SessionResult",
            "flatten_token_batches", "LFM25AsyncInferenceEngine", "SamplingConfig", "InferenceEngineConfig",
-           "GenerationOutput", "GenerationResult"]
+           "GenerationOutput", "GenerationResult", "RolloutRunner", "RolloutRunnerConfig", "RolloutConfig",
+           "RolloutCoordinator", "RolloutCoordinatorConfig", "DirectHarness"]
 
 _LAZY = {
     "LFM25Engine": "engine", "LFM25PrefixBatch": "engine", "LFM25DecodeBatch": "engine", "LFM25StepOutput": "engine",
@@ -23,6 +25,8 @@ _LAZY = {
     "LFM25GenerationSession": "session", "LFM25ContinuationHandle": "session", "LFM25SessionResult": "session",
     "LFM25AsyncInferenceEngine": "async_engine", "SamplingConfig": "inference_config",
     "InferenceEngineConfig": "inference_config", "GenerationOutput": "types", "GenerationResult": "types",
+    "RolloutRunner": "rollout", "RolloutRunnerConfig": "rollout", "RolloutConfig": "rollout",
+    "RolloutCoordinator": "rollout", "RolloutCoordinatorConfig": "rollout", "DirectHarness": "rollout",
 }
 
 

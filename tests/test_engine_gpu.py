@@ -577,3 +577,51 @@ def test_async_adapter_runs_batches_and_chains_on_the_hip_engine():
     assert adapter.last_session_stats["admitted_requests"] == 3
     adapter.close()
     engine.disable_cuda_graphs()
+
+
+@torch.inference_mode()
+def test_rollout_runner_collects_groups_through_the_adapter_on_the_hip_engine():
+    """The runner's requests (rollout/runner.py:272-305) go through the adapter's queue into batched generate calls of
+    the HIP engine: every trajectory carries the engine's ids and logprobs for its prompt, greedy rollouts of one
+    prompt are identical (so with dynamic sampling off the flat groups are kept), and the coordinator parks nothing
+    it should not and pushes weights through the adapter."""
+    import asyncio
+    from types import SimpleNamespace
+    from climbing_gym_amd.async_engine import LFM25AsyncInferenceEngine
+    from climbing_gym_amd.inference_config import InferenceEngineConfig, SamplingConfig
+    from climbing_gym_amd.rollout import DirectHarness, RolloutConfig, RolloutRunner, RolloutRunnerConfig
+    engine, _, _ = _engine()
+    engine.enable_cuda_graphs(max_graphs=2)
+    adapter = LFM25AsyncInferenceEngine.from_components(engine=engine, tokenizer=_ByteTokenizer(),
+                                                        config=InferenceEngineConfig(model_path="", seed=3), max_batch_size=8)
+    prompts = ["hello world", "abc", "the quick brown fox"]
+
+    class Env:
+        def __init__(self):
+            self.queue = [SimpleNamespace(prompt=p, target=None, dataset_index=i) for i, p in enumerate(prompts)]
+        pending_example_count = property(lambda self: len(self.queue))
+        def next_example(self):
+            return self.queue.pop(0) if self.queue else None
+        def next_batch(self, count):
+            raise RuntimeError("no dataset behind the queue")
+        def enqueue_examples(self, examples):
+            self.queue.extend(examples)
+        def evaluate_response(self, example, response, *, turn_count, turn_metadata):
+            return SimpleNamespace(reward=SimpleNamespace(reward=float(len(response))))
+
+    greedy = SamplingConfig(temperature=0.0, max_tokens=10, logprobs=1, extra_params={"ignore_eos": True})
+    runner = RolloutRunner(RolloutRunnerConfig(effective_batch_size=3, use_dynamic_sampling=False, stall_timeout_seconds=60.0))
+    found = asyncio.run(runner.collect(env=Env(), engine=adapter, harness=DirectHarness(),
+                                       rollout_config=RolloutConfig(num_rollouts=2, sampling=greedy)))
+    direct = engine.generate(*_flat([list(p.encode("latin-1")) for p in prompts]), repeats=1,
+                             sampling=LFM25SamplingConfig(temperature=0.0, max_new_tokens=10, ignore_eos=True))
+    assert len(found) == 6 and runner.last_stats["requests_completed"] == 6.0 and runner.last_stats["aborted_request_count"] == 0.0
+    for item in found:
+        row = item.example.dataset_index
+        (turn,) = item.turns
+        assert turn.prompt_token_ids == tuple(prompts[row].encode("latin-1"))
+        assert turn.completion_token_ids == tuple(direct.token_ids[row, 0].cpu().tolist())
+        assert len(turn.completion_logprobs) == 10 and turn.finish_reason == "length"
+        assert item.final_response == _ByteTokenizer().decode(turn.completion_token_ids)
+    adapter.close()
+    engine.disable_cuda_graphs()
