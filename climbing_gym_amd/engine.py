@@ -326,8 +326,11 @@ class LFM25Engine:
         return logits
 
     # ------------------------------------------------------------------ prefill
-    def _prefill_packed(self, cache: LFM25HybridCache, tokens, lengths: Sequence[int], fp8):
-        """Forward a packed batch of whole prompts into cache rows 0..n-1; returns next-token logits [n, V]."""
+    def _prefill_packed(self, cache: LFM25HybridCache, tokens, lengths: Sequence[int], fp8, lengths_device=None):
+        """Forward a packed batch of whole prompts into cache rows 0..n-1; returns next-token logits [n, V].
+        `lengths_device` (int32 on the device, the same numbers as `lengths`) lets a caller with many chunks copy all
+        lengths to the device once: a host-to-device copy per chunk waits for the stream and stops the host from
+        running ahead of the GPU."""
         cfg = self.config
         count, total, longest = len(lengths), int(sum(lengths)), int(max(lengths))
         if count > cache.max_slots:
@@ -336,9 +339,13 @@ class LFM25Engine:
             raise RuntimeError("cache capacity exceeded")
         if longest > self.max_model_len:
             raise RuntimeError("position exceeds engine max_model_len")
-        cu_host = torch.zeros(count + 1, dtype=torch.int32)
-        cu_host[1:] = torch.tensor(lengths, dtype=torch.int32).cumsum(0)
-        cu = cu_host.to(self.device)
+        if lengths_device is None:
+            cu_host = torch.zeros(count + 1, dtype=torch.int32)
+            cu_host[1:] = torch.tensor(lengths, dtype=torch.int32).cumsum(0)
+            cu = cu_host.to(self.device)
+        else:
+            cu = torch.zeros(count + 1, device=self.device, dtype=torch.int32)
+            cu[1:] = lengths_device.cumsum(0)
         seq_of_token, positions = ops.build_token_map(cu, total)
         slots = torch.arange(count, device=self.device, dtype=torch.int32)
 
@@ -396,10 +403,12 @@ class LFM25Engine:
         budget = MAX_PACKED_TOKENS if max_prefill_tokens is None else min(int(max_prefill_tokens), MAX_PACKED_TOKENS)
         fp8 = self._fp8()
         offsets = cu_host.tolist()
+        lengths_device = torch.tensor(lengths, dtype=torch.int32).to(self.device)
         for start, end, _ in plan_prefill_chunks(lengths, budget):
-            logits = self._prefill_packed(cache.rows(start, end), input_ids[offsets[start]:offsets[end]], lengths[start:end], fp8)
+            logits = self._prefill_packed(cache.rows(start, end), input_ids[offsets[start]:offsets[end]], lengths[start:end], fp8,
+                                          lengths_device[start:end])
             logits_out[start:end].copy_(logits)
-        return LFM25PrefixBatch(cache, logits_out, torch.tensor(lengths, device=self.device, dtype=torch.int32), input_ids)
+        return LFM25PrefixBatch(cache, logits_out, lengths_device, input_ids)
 
     # ------------------------------------------------------------------ fork / decode_step
     @torch.inference_mode()

@@ -198,16 +198,32 @@ class LFM25GenerationSession:
         return self._stop_tables[key][0]
 
     def _configure(self, slot, prompt, sampling, *, rng_position=0, stop_state=0):
-        self.versions[slot] += 1
-        self.requests[slot] = _Request(tuple(prompt), sampling, self.versions[slot])
-        if sampling.filtered:
-            self._filter = (sampling.top_k, sampling.top_p)
-        values = ((self.lengths, 0), (self.reasons, 0), (self.stop_states, stop_state), (self.rng_positions, rng_position),
-                  (self.limits, sampling.max_new_tokens), (self.seeds, sampling.seed & 0x7FFFFFFFFFFFFFFF),
-                  (self.temperatures, sampling.temperature), (self.ignore_eos, sampling.ignore_eos),
-                  (self.stop_offsets, self._stop_offset(sampling)), (self.alive, True), (self.pending, False))
-        for tensor, value in values:
-            tensor[slot] = value
+        self._configure_many([(slot, prompt, sampling)], rng_position=rng_position, stop_state=stop_state)
+
+    def _configure_many(self, work, *, rng_position=0, stop_state=0):
+        """Per-row state of newly admitted (slot, prompt, sampling) requests: one indexed write per state tensor for
+        the whole group (a write per row and tensor is eleven tiny launches per request)."""
+        for slot, prompt, sampling in work:
+            self.versions[slot] += 1
+            self.requests[slot] = _Request(tuple(prompt), sampling, self.versions[slot])
+            if sampling.filtered:
+                self._filter = (sampling.top_k, sampling.top_p)
+        samplings = [sampling for _, _, sampling in work]
+        columns = ((self.lengths, [0] * len(work)), (self.reasons, [0] * len(work)),
+                   (self.stop_states, [stop_state] * len(work)), (self.rng_positions, [rng_position] * len(work)),
+                   (self.limits, [s.max_new_tokens for s in samplings]),
+                   (self.seeds, [s.seed & 0x7FFFFFFFFFFFFFFF for s in samplings]),
+                   (self.temperatures, [s.temperature for s in samplings]), (self.ignore_eos, [s.ignore_eos for s in samplings]),
+                   (self.stop_offsets, [self._stop_offset(s) for s in samplings]), (self.alive, [True] * len(work)),
+                   (self.pending, [False] * len(work)))
+        if len(work) == 1:
+            slot = work[0][0]
+            for tensor, values in columns:
+                tensor[slot] = values[0]
+            return
+        index = torch.tensor([slot for slot, _, _ in work], dtype=torch.long).to(self.lengths.device)
+        for tensor, values in columns:
+            tensor[index] = torch.tensor(values, dtype=tensor.dtype).to(tensor.device)
 
     def _free_slots(self):
         return [i for i, r in enumerate(self.requests) if r is None]
@@ -248,9 +264,9 @@ class LFM25GenerationSession:
             begin = end
         for slot, prompt, sampling in work:
             self.stats['slot_refills'] += int(self.versions[slot] > 0)
-            self._configure(slot, prompt, sampling)
             self.stats['prefilled_tokens'] += len(prompt)
             self.stats['admitted_requests'] += 1
+        self._configure_many(work)
         self.stats['peak_live_slots'] = max(self.stats['peak_live_slots'], self._live_count())
         return slots
 
