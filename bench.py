@@ -41,6 +41,8 @@ def parse_args():
     p.add_argument("--cpu-seqs", type=int, default=4, help="sequences of the workload the CPU baseline runs (0 = skip)")
     p.add_argument("--cpu-steps", type=int, default=8)
     p.add_argument("--attn-samples", type=int, default=20, help="timed launches of the decode-attention kernel per layer")
+    p.add_argument("--top-k", type=int, default=0, help="top-k filter of the sampler (0: full support)")
+    p.add_argument("--top-p", type=float, default=1.0, help="top-p filter of the sampler (1: off)")
     p.add_argument("--workload", choices=("decode", "attention"), default="decode",
                    help="decode: the model's decode step (the headline metric); attention: the decode-attention call alone "
                         "on 256 sequences of U[128, 8192] history tokens, dense and paged (block 16), e4m3 and bf16")
@@ -304,8 +306,8 @@ def main():
     prompts = random_prompts(args.batch, args.prompt_low, args.prompt_high, LFM2_1P2B["vocab"], seed=0)
     engine, cfg = build_engine(args, state)
     new_tokens = min(4096, args.max_model_len - max(map(len, prompts)))
-    sampling = [LFM25SamplingConfig(temperature=1.0, seed=1000 + i, max_new_tokens=new_tokens, ignore_eos=True)
-                for i in range(args.batch)]
+    sampling = [LFM25SamplingConfig(temperature=1.0, seed=1000 + i, max_new_tokens=new_tokens, ignore_eos=True,
+                                    top_k=args.top_k, top_p=args.top_p) for i in range(args.batch)]
     with torch.inference_mode(), engine.generation_session(max_batch_size=args.batch, max_new_tokens=new_tokens,
                                                             cache_len=args.max_model_len) as session:
         torch.cuda.synchronize()
@@ -336,7 +338,8 @@ def main():
         "vs_baseline": None, "dtype": "fp8_e4m3 (W8A8, fp32 accumulate; bf16 activations)" if fp8 else "bf16",
         "data": "synthetic",
         "config": {"workload": f"LFM2.5-1.2B-shaped random-init model, {args.precision} linears and KV cache, {args.batch} "
-                               f"concurrent sequences, prompts U[{args.prompt_low},{args.prompt_high}] tokens, temperature 1, "
+                               f"concurrent sequences, prompts U[{args.prompt_low},{args.prompt_high}] tokens, temperature 1"
+                               f"{'' if args.top_k == 0 and args.top_p == 1.0 else f', top-k {args.top_k}, top-p {args.top_p}'}, "
                                f"max_model_len {args.max_model_len}, HIP-graph decode step",
                    "context_tokens": ctx_tokens, "prefill_tok_per_s": round(sum(map(len, prompts)) / prefill_s, 1),
                    "gemm": gemms, "step_algorithmic_bytes": step_bytes,

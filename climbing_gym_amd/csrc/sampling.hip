@@ -264,9 +264,11 @@ constexpr int kFT = 1024;  // threads of the filtered sampler
 
 // One workgroup per row.  All decisions use integer histograms (counts, and 2^40 fixed-point
 // softmax mass), so results do not depend on the order in which lanes reach the atomics.
+// This form re-reads the row from memory in every pass and serves vocabularies beyond what a workgroup can hold in
+// registers; the register form below makes the same decisions.
 template <typename T>
 __global__ void __launch_bounds__(kFT)
-sample_filtered_kernel(const T* logits, int64_t* tokens, float* logprobs, int32_t* kept_count, const int64_t* seeds,
+sample_filtered_stream_kernel(const T* logits, int64_t* tokens, float* logprobs, int32_t* kept_count, const int64_t* seeds,
                        const int64_t* steps, int64_t seed, int64_t step, float temperature, int top_k, float top_p, int64_t V) {
   __shared__ uint32_t h_cnt[256];
   __shared__ unsigned long long h_mass[256];
@@ -460,6 +462,341 @@ sample_filtered_kernel(const T* logits, int64_t* tokens, float* logprobs, int32_
   }
 }
 
+// The same sampler for rows of at most kFT * kFV logits (65536): the row is read from memory ONCE, 16 bytes per load,
+// and stays in registers (64 tempered logits per thread) for every later pass.  The selections are radix selections
+// on the order keys with 12-bit digits: one pass is 4096-bin histograms of counts (and of 2^40 fixed-point masses for
+// the nucleus) filled with LDS atomics, then every thread looks at its four bins with the totals of the bins above
+// them (a wave scan and sixteen wave totals) and the highest bin that crosses the limit wins.  Three passes fix a
+// 32-bit key; after the first one only the elements of one bin take part.  Same integer decisions as the streaming
+// form, so results do not depend on the order of the atomics.
+// What such a kernel costs is its instruction count: every pass over 64 registers per thread is a few hundred
+// instructions whether or not an element takes part.  So the elements that can still matter are copied to a list
+// in LDS as soon as they are few (at most kCand), and every later step walks the list.  With top_k <= 1024 that is
+// right at the start: the k-th largest of the threads' own maxima is a lower bound of the k-th largest logit (k
+// threads hold a value that large) and only a handful of logits lie above it; otherwise after the top-k selection.
+// A nucleus without top-k keeps working on the registers.
+constexpr int kFV = 64, kBins = 4096, kCand = 2048;
+
+struct Crossed { int bin; uint32_t count_above, count_at; unsigned long long mass_above; };
+
+template <typename T>
+__global__ void __launch_bounds__(kFT)
+sample_filtered_kernel(const T* logits, int64_t* tokens, float* logprobs, int32_t* kept_count, const int64_t* seeds,
+                       const int64_t* steps, int64_t seed, int64_t step, float temperature, int top_k, float top_p, int64_t V) {
+  constexpr int EPV = 16 / sizeof(T), CHUNKS = kFV / EPV, WAVES = kFT / 64;
+  __shared__ uint32_t h_cnt[kBins];
+  __shared__ unsigned long long h_mass[kBins];
+  __shared__ uint32_t w_cnt[WAVES];
+  __shared__ unsigned long long w_mass[WAVES];
+  __shared__ float s_f[WAVES];
+  __shared__ int s_i[WAVES];
+  __shared__ int s_best;
+  __shared__ Crossed s_crossed;
+  __shared__ unsigned long long s_total;
+  __shared__ uint32_t c_key[kCand];
+  __shared__ int c_col[kCand];
+  __shared__ int s_candidates;
+  const int64_t row = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const T* src = logits + row * V;
+  const uint64_t key64 = seeds ? row_key(seeds[row], steps[row]) : row_key(seed, step);
+  const bool vector_ok = V % EPV == 0;
+  // element j of a thread is column tid * EPV + (j / EPV) * kFT * EPV + j % EPV; columns beyond V hold -inf, the
+  // smallest key with no mass, so only the steps that count or pick elements need to look at the column
+  const int V32 = (int)V, col0 = tid * EPV;
+  auto column = [&](int j) { return col0 + (j / EPV) * (kFT * EPV) + j % EPV; };
+
+  // ---- the row, once: raw maximum and normaliser (for the returned log-probability), then the tempered logits
+  float xs[kFV];
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) load_columns(src, (int64_t)(c * kFT + tid) * EPV, V, vector_ok, xs + c * EPV);
+  float mx = xs[0];
+#pragma unroll
+  for (int j = 1; j < kFV; ++j) mx = fmaxf(mx, xs[j]);
+  mx = wave_max(mx);
+  if (lane == 0) s_f[wave] = mx;
+  __syncthreads();
+  mx = s_f[0];
+  for (int w = 1; w < WAVES; ++w) mx = fmaxf(mx, s_f[w]);
+  __syncthreads();
+  float raw_sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < kFV; ++j) {
+    raw_sum += __expf(xs[j] - mx);
+    __builtin_amdgcn_sched_barrier(0);   // one element at a time: interleaved, the unrolled bodies need more registers than there are
+  }
+  raw_sum = wave_sum(raw_sum);
+  if (lane == 0) s_f[wave] = raw_sum;
+  __syncthreads();
+  raw_sum = 0.f;
+  for (int w = 0; w < WAVES; ++w) raw_sum += s_f[w];
+  __syncthreads();
+  const float xmax = mx / temperature;
+  // from here on the row lives in registers as the order keys of the tempered logits: every selection compares keys,
+  // and the few places that need a value turn the key back into it
+  uint32_t ks[kFV];
+#pragma unroll
+  for (int j = 0; j < kFV; ++j) ks[j] = order_key(xs[j] / temperature);
+  auto value_of = [](uint32_t k) { return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k); };
+  auto mass_of = [&](float x) -> unsigned long long { return (unsigned long long)(exp2f((x - xmax) * LFM2_LOG2E) * 1099511627776.0f); };
+  // A mass is recomputed wherever it is used: kept from one pass to the next, sixty-four 64-bit masses per thread
+  // would not fit in registers.  The empty statement hides the value's origin from common-subexpression elimination.
+  auto fresh = [](uint32_t k) { asm volatile("" : "+v"(k)); return k; };
+
+  // One selection pass over the histograms just filled: thread t owns bins 4t .. 4t+3.  Walking from the highest
+  // bin down with the running totals (count, mass) of everything above, the first bin where the limit is crossed
+  // (by_mass: above + mass > mass_limit; else: above + count >= count_limit) is reported in s_crossed; bin -1: none.
+  auto select = [&](bool by_mass, uint32_t count_limit, unsigned long long mass_limit, uint32_t count_base,
+                    unsigned long long mass_base) {
+    uint32_t cnt[4], mine_c = 0;
+    unsigned long long mass[4], mine_m = 0;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      cnt[b] = h_cnt[4 * tid + b]; mass[b] = by_mass ? h_mass[4 * tid + b] : 0ull;
+      mine_c += cnt[b]; mine_m += mass[b];
+    }
+    uint32_t c = mine_c;
+    unsigned long long m = mine_m;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {   // totals of this lane and the lanes above it in the wave
+      const uint32_t oc = __shfl_down(c, o, 64);
+      const unsigned long long om = __shfl_down(m, o, 64);
+      if (lane + o < 64) { c += oc; m += om; }
+    }
+    if (lane == 0) { w_cnt[wave] = c; w_mass[wave] = m; }
+    if (tid == 0) s_best = -1;
+    __syncthreads();
+    uint32_t above_c = count_base + c - mine_c;
+    unsigned long long above_m = mass_base + m - mine_m;
+    for (int w = wave + 1; w < WAVES; ++w) { above_c += w_cnt[w]; above_m += w_mass[w]; }
+    Crossed found{-1, 0, 0, 0};
+#pragma unroll
+    for (int b = 3; b >= 0; --b) {
+      if (cnt[b] == 0) continue;
+      const bool crosses = by_mass ? above_m + mass[b] > mass_limit : above_c + cnt[b] >= count_limit;
+      if (crosses && found.bin < 0) found = Crossed{4 * tid + b, above_c, cnt[b], above_m};
+      above_c += cnt[b]; above_m += mass[b];
+    }
+    if (found.bin >= 0) atomicMax(&s_best, found.bin);
+    __syncthreads();
+    if (found.bin >= 0 && found.bin == s_best) s_crossed = found;
+    if (tid == 0 && s_best < 0) s_crossed = Crossed{-1, above_c, 0, above_m};   // thread 0 ends with the totals of all bins
+    __syncthreads();
+  };
+  auto clear_bins = [&](bool with_mass) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) { h_cnt[4 * tid + b] = 0; if (with_mass) h_mass[4 * tid + b] = 0; }
+    __syncthreads();
+  };
+  constexpr int kShift[3] = {20, 8, 0};
+  constexpr uint32_t kDigit[3] = {0xFFFu, 0xFFFu, 0xFFu}, kDone[3] = {0xFFF00000u, 0xFFFFFF00u, 0xFFFFFFFFu};
+
+  // ---- the elements that can still matter, as a list in LDS once they are few: (key, column) of every logit whose
+  // key is at least `floor`.  All later steps then walk the list (a few entries per thread at most) instead of the
+  // 64 registers of every thread.
+  bool listed = false;
+  int list_size = 0;
+  auto try_list = [&](uint32_t floor) {
+    if (tid == 0) s_candidates = 0;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kFV; ++j) {
+      if (ks[j] >= floor && column(j) < V32) {
+        const int at = atomicAdd(&s_candidates, 1);
+        if (at < kCand) { c_key[at] = ks[j]; c_col[at] = column(j); }
+      }
+    }
+    __syncthreads();
+    list_size = s_candidates;
+    listed = list_size <= kCand;
+    __syncthreads();
+  };
+  // visit(key, column) for the elements with key >= at_least that this thread is responsible for; without a list
+  // that includes the -inf padding beyond the row's end when at_least is below every real key
+  auto for_each = [&](uint32_t at_least, auto&& visit) {
+    if (listed) {
+      for (int e = tid; e < list_size; e += kFT) {
+        const uint32_t k = c_key[e];
+        if (k >= at_least) visit(k, c_col[e]);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < kFV; ++j) {
+        if (ks[j] >= at_least) visit(fresh(ks[j]), column(j));
+        __builtin_amdgcn_sched_barrier(0);   // one element at a time: interleaved, the unrolled bodies need more registers than there are
+      }
+    }
+  };
+
+  // ---- top-k: key of the k-th largest tempered logit
+  uint32_t key_k = 0;
+  if (top_k > 0 && top_k < V) {
+    // the k-th largest of the keys that `keys` visits
+    auto kth_largest = [&](auto&& keys) -> uint32_t {
+      uint32_t prefix = 0, mask = 0, remaining = (uint32_t)top_k;
+      for (int pass = 0; pass < 3; ++pass) {
+        clear_bins(false);
+        keys([&](uint32_t k, int) {
+          if ((k & mask) == prefix) atomicAdd(&h_cnt[(k >> kShift[pass]) & kDigit[pass]], 1u);
+        });
+        __syncthreads();
+        select(false, remaining, 0ull, 0u, 0ull);
+        prefix |= (uint32_t)s_crossed.bin << kShift[pass];
+        mask = kDone[pass];
+        remaining -= s_crossed.count_above;
+        __syncthreads();
+      }
+      return prefix;
+    };
+    uint32_t floor_key = 0;
+    if (top_k <= kFT) {
+      // k threads hold a logit at least as large as the k-th largest of the threads' maxima: a lower bound of the
+      // k-th largest logit, above which only a handful of logits lie
+      uint32_t top = ks[0];
+#pragma unroll
+      for (int j = 1; j < kFV; ++j) top = top > ks[j] ? top : ks[j];
+      floor_key = kth_largest([&](auto&& visit) { visit(top, 0); });
+      try_list(floor_key);
+    }
+    key_k = kth_largest([&](auto&& visit) { for_each(floor_key, visit); });
+    if (!listed) try_list(key_k);
+  }
+
+  // ---- nucleus: walk keys downward until the inclusive cumulative mass exceeds top_p * Z
+  uint32_t kp = key_k;
+  int ties_kept = kNoIndex, ties_total = 0;
+  uint32_t cnt_above = 0;
+  bool crossed = false;
+  if (top_p < 1.0f) {
+    unsigned long long z = 0;
+    for_each(key_k, [&](uint32_t k, int) { z += mass_of(value_of(k)); });
+    if (tid == 0) s_total = 0;
+    __syncthreads();
+    if (z) atomicAdd(&s_total, z);
+    __syncthreads();
+    const unsigned long long limit = (unsigned long long)((double)top_p * (double)s_total);
+    uint32_t prefix = 0, mask = 0;
+    unsigned long long mass_above = 0;
+    crossed = true;
+    for (int pass = 0; pass < 3 && crossed; ++pass) {
+      clear_bins(true);
+      for_each(key_k, [&](uint32_t k, int) {
+        if ((k & mask) == prefix) {
+          const uint32_t bin = (k >> kShift[pass]) & kDigit[pass];
+          atomicAdd(&h_cnt[bin], 1u);
+          atomicAdd(&h_mass[bin], mass_of(value_of(k)));
+        }
+      });
+      __syncthreads();
+      select(true, 0u, limit, cnt_above, mass_above);
+      crossed = s_crossed.bin >= 0;
+      cnt_above = s_crossed.count_above;
+      mass_above = s_crossed.mass_above;
+      if (crossed) {
+        prefix |= (uint32_t)s_crossed.bin << kShift[pass];
+        mask = kDone[pass];
+        ties_total = (int)s_crossed.count_at;
+      }
+      __syncthreads();
+    }
+    if (crossed) {
+      kp = prefix;
+      const unsigned long long w = mass_of(value_of(kp));
+      unsigned long long fit = w ? (limit - mass_above) / w : 0;
+      if (fit >= (unsigned long long)ties_total) fit = ties_total;
+      ties_kept = (int)fit;
+      if (cnt_above == 0 && ties_kept == 0) ties_kept = 1;  // rank 0 always survives
+    }
+  }
+
+  // Number of elements of the row (padding excluded) with key >= at_least that a predicate holds for.
+  auto block_count = [&](uint32_t at_least, auto&& holds) -> int {
+    int c = 0;
+    for_each(at_least, [&](uint32_t k, int col) { c += (col < V32 && holds(k, col)) ? 1 : 0; });
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o, 64);
+    __syncthreads();
+    if (lane == 0) s_i[wave] = c;
+    __syncthreads();
+    int total = 0;
+    for (int w = 0; w < WAVES; ++w) total += s_i[w];
+    return total;
+  };
+
+  // ---- when only some of the ties at kp survive, keep the lowest-index ones: find the cut column (rare: two
+  // equal logits exactly on the nucleus boundary), by bisection on the column
+  int cut = kNoIndex;
+  if (crossed) {
+    if (ties_kept == 0) {
+      cut = -1;
+    } else if (ties_kept < ties_total) {
+      int lo = 0, hi = V32 - 1;
+      while (lo < hi) {
+        const int mid = lo + (hi - lo) / 2;
+        if (block_count(kp, [&](uint32_t k, int col) { return k == kp && col <= mid; }) >= ties_kept) hi = mid;
+        else lo = mid + 1;
+      }
+      cut = lo;
+    }
+    if (kept_count && tid == 0) kept_count[row] = (int)cnt_above + ties_kept;
+  } else if (kept_count) {
+    const int kept = block_count(kp, [&](uint32_t, int) { return true; });
+    if (tid == 0) kept_count[row] = kept;
+  }
+
+  // ---- Gumbel-max over the survivors
+  float best = -INFINITY;
+  int best_i = kNoIndex;
+  auto consider = [&](float x, int i) {
+    uint32_t rnd[4];
+    // per-row streams depend on the row's own (seed, step) only; a shared seed also counts the row
+    philox((uint32_t)(i >> 2), seeds ? 0u : (uint32_t)row, 0x5eed5eedu, seeds ? 0u : (uint32_t)((uint64_t)row >> 32),
+           (uint32_t)key64, (uint32_t)(key64 >> 32), rnd);
+    const float score = x + gumbel(rnd[i & 3]);
+    if (best_i == kNoIndex || score > best || (score == best && i < best_i)) { best = score; best_i = i; }
+  };
+  if (listed) {
+    for (int e = tid; e < list_size; e += kFT) {
+      const uint32_t k = c_key[e];
+      const int i = c_col[e];
+      if (k > kp || (k == kp && i <= cut)) consider(value_of(k), i);
+    }
+  } else {
+    // a thread's survivors as a bit mask first, then a loop over the set bits that reads the survivor's logit again:
+    // registers cannot be indexed by a loop variable, and sixty-four unrolled Philox blocks would not fit in them
+    uint64_t survivors = 0;
+#pragma unroll
+    for (int j = 0; j < kFV; ++j) {
+      const uint32_t k = ks[j];
+      if (column(j) < V32 && (k > kp || (k == kp && column(j) <= cut))) survivors |= 1ull << j;
+    }
+    while (survivors) {
+      const int j = __builtin_ctzll(survivors);
+      survivors &= survivors - 1;
+      const int i = col0 + (j / EPV) * (kFT * EPV) + j % EPV;
+      consider(Elem<T>::load(src[i]) / temperature, i);
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ob = __shfl_xor(best, o, 64);
+    const int oi = __shfl_xor(best_i, o, 64);
+    if (oi != kNoIndex && (best_i == kNoIndex || ob > best || (ob == best && oi < best_i))) { best = ob; best_i = oi; }
+  }
+  __syncthreads();
+  if (lane == 0) { s_f[wave] = best; s_i[wave] = best_i; }
+  __syncthreads();
+  if (tid == 0) {
+    float b = s_f[0];
+    int bi = s_i[0];
+    for (int w = 1; w < WAVES; ++w)
+      if (s_i[w] != kNoIndex && (bi == kNoIndex || s_f[w] > b || (s_f[w] == b && s_i[w] < bi))) { b = s_f[w]; bi = s_i[w]; }
+    if (bi == kNoIndex) bi = 0;
+    tokens[row] = bi;
+    if (logprobs) logprobs[row] = Elem<T>::load(src[bi]) - (mx + logf(raw_sum));
+  }
+}
+
 // ------------------------------------------------------------------------------------ small row kernels
 template <typename T>
 __global__ void head_logprobs_kernel(float* out, const T* logits, const int64_t* selected, const float* logprobs,
@@ -573,8 +910,13 @@ extern "C" int lfm2_sample_filtered(int64_t* tokens, float* logprobs, int32_t* k
   LFM2_REQUIRE(V < (1ll << 31), "sample_filtered: vocabulary too large");
   LFM2_REQUIRE((seeds == nullptr) == (steps == nullptr), "sample_filtered: seeds and steps go together");
   DISPATCH_DTYPE(dtype, "sample_filtered",
-                 hipLaunchKernelGGL(sample_filtered_kernel<T>, dim3(B), dim3(kFT), 0, (hipStream_t)stream, (const T*)logits,
-                                    tokens, logprobs, kept_count, seeds, steps, seed, step, temperature, top_k, top_p, V));
+                 if (V <= (int64_t)kFT * kFV)
+                   hipLaunchKernelGGL(sample_filtered_kernel<T>, dim3(B), dim3(kFT), 0, (hipStream_t)stream, (const T*)logits,
+                                      tokens, logprobs, kept_count, seeds, steps, seed, step, temperature, top_k, top_p, V);
+                 else
+                   hipLaunchKernelGGL(sample_filtered_stream_kernel<T>, dim3(B), dim3(kFT), 0, (hipStream_t)stream,
+                                      (const T*)logits, tokens, logprobs, kept_count, seeds, steps, seed, step, temperature,
+                                      top_k, top_p, V));
   LFM2_LAUNCH_CHECK();
 }
 

@@ -580,6 +580,27 @@ def test_filtered_sampling_keeps_exactly_the_oracle_support(ops, top_k, top_p, d
         assert torch.equal(draws[0], logits.float().argmax(-1))
 
 
+@pytest.mark.parametrize("top_k,top_p", [(50, 0.95), (0, 0.9), (7, 1.0), (0, 0.3)])
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float32))
+@torch.inference_mode()
+def test_filtered_sampling_in_registers_and_streamed_make_the_same_draws(ops, top_k, top_p, dtype):
+    """Rows of up to 65536 logits are sampled from registers, longer ones by re-reading the row in every pass.  A row
+    padded with -inf columns beyond 65536 has the same survivors and the same per-column random numbers as the
+    unpadded row, so both forms must return the same tokens, survivor counts and log-probabilities; bf16 rows with
+    many equal values put ties on the top-k and nucleus boundaries."""
+    torch.manual_seed(21)
+    rows, vocab, wide = 24, 6000, 70000
+    logits = (torch.randn(rows, vocab) * 2.0).to(dtype)
+    logits[:8] = (torch.randn(8, vocab) * 0.5).to(torch.bfloat16).to(dtype)       # coarse values: many ties
+    padded = torch.full((rows, wide), -math.inf, dtype=dtype)
+    padded[:, :vocab] = logits
+    for step in range(6):
+        a = ops.sample_filtered(logits.to(DEV), temperature=0.7, top_k=top_k, top_p=top_p, seed=11, step=step, return_kept=True)
+        b = ops.sample_filtered(padded.to(DEV), temperature=0.7, top_k=top_k, top_p=top_p, seed=11, step=step, return_kept=True)
+        assert torch.equal(a[0], b[0]) and torch.equal(a[2], b[2])
+        torch.testing.assert_close(a[1], b[1], atol=2e-6, rtol=1e-6)
+
+
 @torch.inference_mode()
 def test_filtered_sampling_distribution_follows_renormalised_survivors(ops):
     probs = torch.tensor([0.4, 0.3, 0.15, 0.1, 0.05])
