@@ -5,6 +5,7 @@
 // lives at slot*c0 + pos*c1 + head*c2 + d, and the e4m3 scale of (slot, pos, head) at that offset
 // divided by D.  With a block table, c0 is the page stride and pos is the in-page index.
 #include "lfm2_common.h"
+#include <type_traits>
 
 namespace {
 
@@ -750,31 +751,43 @@ __global__ void __launch_bounds__(1024) decode_combine_row_kernel(DecodeArgs a, 
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, f), c));
   };
   float y[kMaxPerLane] = {0.f, 0.f, 0.f, 0.f};
-  if (n > 0 && n <= NC) {
-    float mv[kMaxPerLane], lv[kMaxPerLane], accv[kMaxPerLane][NC];
+  // outputs first .. first + COUNT - 1 of a row of at most CHUNKS chunks, with every load issued before the first use
+  auto merge_at_once = [&](auto count, auto chunks, int first) {
+    constexpr int COUNT = decltype(count)::value, CHUNKS = decltype(chunks)::value;
+    float mv[COUNT], lv[COUNT], accv[COUNT][CHUNKS];
 #pragma unroll
-    for (int i = 0; i < kMaxPerLane; ++i) {
+    for (int u = 0; u < COUNT; ++u) {
+      const int i = first + u;
       const int qh = head_of(i) < a.QH ? head_of(i) : a.QH - 1, d = dim_of(i) < a.D ? dim_of(i) : a.D - 1;
       if (head_of(i) < a.QH) {   // the same for the whole wave
         const int64_t mine = partial_row(a, rp, b, qh, lane < n ? lane : 0);
-        mv[i] = a.ws_m[mine];
-        lv[i] = a.ws_l[mine];
+        mv[u] = a.ws_m[mine];
+        lv[u] = a.ws_l[mine];
 #pragma unroll
-        for (int c = 0; c < NC; ++c) accv[i][c] = a.ws_acc[partial_row(a, rp, b, qh, c < n ? c : 0) * a.D + d];
+        for (int c = 0; c < CHUNKS; ++c) accv[u][c] = a.ws_acc[partial_row(a, rp, b, qh, c < n ? c : 0) * a.D + d];
       }
     }
 #pragma unroll
-    for (int i = 0; i < kMaxPerLane; ++i) {
+    for (int u = 0; u < COUNT; ++u) {
+      const int i = first + u;
       if (head_of(i) < a.QH) {
-        const float mm = wave_max(lane < n ? mv[i] : -1.0e30f);
-        const float f = lane < n ? exp2f(mv[i] - mm) : 0.f;
-        const float lt = wave_sum(lv[i] * f);
+        const float mm = wave_max(lane < n ? mv[u] : -1.0e30f);
+        const float f = lane < n ? exp2f(mv[u] - mm) : 0.f;
+        const float lt = wave_sum(lv[u] * f);
         float o = 0.f;
 #pragma unroll
-        for (int c = 0; c < NC; ++c) o = fmaf(accv[i][c], weight_of(f, c), o);   // chunks past the row's: weight 0
+        for (int c = 0; c < CHUNKS; ++c) o = fmaf(accv[u][c], weight_of(f, c), o);   // chunks past the row's: weight 0
         y[i] = round_to<T>(o * (1.0f / fmaxf(lt, 1.0e-20f)));
       }
     }
+  };
+  typedef std::integral_constant<int, kMaxPerLane> AllOutputs;
+  typedef std::integral_constant<int, kMaxPerLane / 2> HalfOutputs;
+  if (n > 0 && n <= NC) {
+    merge_at_once(AllOutputs{}, std::integral_constant<int, NC>{}, 0);
+  } else if (n > 0 && n <= 2 * NC) {   // twice the chunks, half the outputs at a time: the same registers
+    merge_at_once(HalfOutputs{}, std::integral_constant<int, 2 * NC>{}, 0);
+    merge_at_once(HalfOutputs{}, std::integral_constant<int, 2 * NC>{}, kMaxPerLane / 2);
   } else if (n > 0) {
     // longer rows: the chunks' maxima and sums in groups of 64 (one per lane), the accumulators in blocks of NC
     for (int i = 0; i < kMaxPerLane; ++i) {
