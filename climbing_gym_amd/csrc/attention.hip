@@ -734,10 +734,11 @@ __global__ void __launch_bounds__(64) decode_combine_kernel(DecodeArgs a) {
 // written by other XCDs and come from beyond the local L2, so every dependent round of loads costs a full memory
 // latency: a chunk's maximum and sum are loaded by the lane of the chunk's index (the chunks' weights
 // exp2(m_c - max) are then one exp2 per lane, read back lane by lane as scalars), and the accumulator loads do not
-// depend on them, so a row of up to NC chunks has every load of its merge in flight at once.
+// depend on them, so a row of up to NC chunks (all outputs of a lane together) or 32 chunks (half of them at a time) has every
+// load of its merge in flight at once.
 template <typename T, int NC, bool QUANT>
 __global__ void __launch_bounds__(1024) decode_combine_row_kernel(DecodeArgs a, uint8_t* q_out, float* q_scales) {
-  constexpr int kMaxPerLane = 4, kWavesPerRow = 16;
+  constexpr int kMaxPerLane = 4, kWavesPerRow = 16, kMidChunks = 32;
   __shared__ float red[kWavesPerRow];
   const int b = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const RowPairs rp = row_pairs(a, b);
@@ -785,9 +786,9 @@ __global__ void __launch_bounds__(1024) decode_combine_row_kernel(DecodeArgs a, 
   typedef std::integral_constant<int, kMaxPerLane / 2> HalfOutputs;
   if (n > 0 && n <= NC) {
     merge_at_once(AllOutputs{}, std::integral_constant<int, NC>{}, 0);
-  } else if (n > 0 && n <= 2 * NC) {   // twice the chunks, half the outputs at a time: the same registers
-    merge_at_once(HalfOutputs{}, std::integral_constant<int, 2 * NC>{}, 0);
-    merge_at_once(HalfOutputs{}, std::integral_constant<int, 2 * NC>{}, kMaxPerLane / 2);
+  } else if (n > 0 && n <= kMidChunks) {   // more chunks, half the outputs at a time: about the same registers
+    merge_at_once(HalfOutputs{}, std::integral_constant<int, kMidChunks>{}, 0);
+    merge_at_once(HalfOutputs{}, std::integral_constant<int, kMidChunks>{}, kMaxPerLane / 2);
   } else if (n > 0) {
     // longer rows: the chunks' maxima and sums in groups of 64 (one per lane), the accumulators in blocks of NC
     for (int i = 0; i < kMaxPerLane; ++i) {
@@ -838,13 +839,13 @@ __global__ void __launch_bounds__(1024) decode_combine_row_kernel(DecodeArgs a, 
 
 template <typename T>
 void launch_combine_fp8(const DecodeArgs& a, int64_t B, uint8_t* out_q, float* out_scales, hipStream_t s) {
-  hipLaunchKernelGGL((decode_combine_row_kernel<T, 16, true>), dim3(B), dim3(1024), 0, s, a, out_q, out_scales);
+  hipLaunchKernelGGL((decode_combine_row_kernel<T, 12, true>), dim3(B), dim3(1024), 0, s, a, out_q, out_scales);
 }
 // The merge alone: a row per workgroup when the row fits the row kernel's registers, a (row, head) per wave otherwise.
 template <typename T>
 void launch_combine(const DecodeArgs& a, int64_t B, hipStream_t s) {
   if ((int64_t)((a.QH + 15) / 16) * ((a.D + 63) / 64) <= 4)
-    hipLaunchKernelGGL((decode_combine_row_kernel<T, 16, false>), dim3(B), dim3(1024), 0, s, a, nullptr, nullptr);
+    hipLaunchKernelGGL((decode_combine_row_kernel<T, 12, false>), dim3(B), dim3(1024), 0, s, a, nullptr, nullptr);
   else
     hipLaunchKernelGGL(decode_combine_kernel<T>, dim3(B, a.QH), dim3(64), 0, s, a);
 }

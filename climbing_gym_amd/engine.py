@@ -404,10 +404,16 @@ class LFM25Engine:
         fp8 = self._fp8()
         offsets = cu_host.tolist()
         lengths_device = torch.tensor(lengths, dtype=torch.int32).to(self.device)
+        in_flight = []   # the host stays at most two chunks (a few hundred launches) ahead of the GPU
         for start, end, _ in plan_prefill_chunks(lengths, budget):
             logits = self._prefill_packed(cache.rows(start, end), input_ids[offsets[start]:offsets[end]], lengths[start:end], fp8,
                                           lengths_device[start:end])
             logits_out[start:end].copy_(logits)
+            marker = torch.cuda.Event()
+            marker.record()
+            in_flight.append(marker)
+            if len(in_flight) > 2:
+                in_flight.pop(0).synchronize()
         return LFM25PrefixBatch(cache, logits_out, lengths_device, input_ids)
 
     # ------------------------------------------------------------------ fork / decode_step
