@@ -308,6 +308,11 @@ def main():
     new_tokens = min(4096, args.max_model_len - max(map(len, prompts)))
     sampling = [LFM25SamplingConfig(temperature=1.0, seed=1000 + i, max_new_tokens=new_tokens, ignore_eos=True,
                                     top_k=args.top_k, top_p=args.top_p) for i in range(args.batch)]
+    # a first admission of a few prompts into a throw-away session: kernel code objects and the allocator's blocks are
+    # loaded once per process, and the prefill rate reported is that of an engine that has served before
+    with torch.inference_mode(), engine.generation_session(max_batch_size=8, max_new_tokens=new_tokens,
+                                                            cache_len=args.max_model_len) as session:
+        session.admit(prompts[:8], sampling[:8])
     with torch.inference_mode(), engine.generation_session(max_batch_size=args.batch, max_new_tokens=new_tokens,
                                                             cache_len=args.max_model_len) as session:
         torch.cuda.synchronize()

@@ -163,7 +163,7 @@ class LFM25GenerationSession:
             raise ValueError('Request behavior head exceeds the session reservation')
         if not prompt:
             raise ValueError("Empty prompts are not supported")
-        if any(type(t) is not int or not 0 <= t < vocab for t in prompt):
+        if set(map(type, prompt)) != {int} or min(prompt) < 0 or max(prompt) >= vocab:   # C-level passes over the ids
             raise ValueError("Prompt token outside the model vocabulary")
         if len(prompt) + sampling.max_new_tokens > self.entry.cache.max_seq_len:
             raise ValueError("Request exceeds reserved session context capacity")
