@@ -873,10 +873,13 @@ prefill_attn_kernel(T* __restrict__ out, const T* __restrict__ q, const T* __res
                     const int32_t* __restrict__ cu, int QH, int KH, float scale_log2e) {
   typedef typename HalfMfma<T>::vec8 vec8;
   typedef T vec4 __attribute__((ext_vector_type(4)));
-  constexpr int KC = D / 8;          // 16-byte chunks per K row
-  constexpr int VP = 64 + 8;         // padded token stride of the transposed V tile
+  constexpr int KC = D / 8;          // 16-byte chunks per K or V row
+  constexpr int NCH = 64 * KC / 256; // chunks of a 64-token tile per thread, for K and for V
+  // K and V tiles sit in LDS as they are in memory (row = token), 16-byte chunks XOR-swizzled by the token.  The
+  // V^T operand comes out of the row-major tile through ds_read_b64_tr_b16: lane p of 16 points at token p / 4,
+  // bytes 8 (p % 4) .. of a 16-dim block, and lane s receives 4 consecutive tokens of dim s.
   __shared__ vec8 ldsK[64 * KC];
-  __shared__ T ldsVt[D * VP];
+  __shared__ vec8 ldsV[64 * KC];
 
   const int seq = blockIdx.z, qh = blockIdx.y, kh = qh / (QH / KH);
   const int begin = cu[seq], len = cu[seq + 1] - begin;
@@ -899,19 +902,30 @@ prefill_attn_kernel(T* __restrict__ out, const T* __restrict__ q, const T* __res
 
   int kv_end = q0 + 64;
   kv_end = kv_end < len ? kv_end : len;
-  for (int t0 = 0; t0 < kv_end; t0 += 64) {
-    __syncthreads();
-    for (int idx = tid; idx < 64 * KC; idx += 256) {
-      const int tok = idx / KC, c = idx % KC;
+  // the next tile's rows travel to registers while the current tile is multiplied (tokens clamped into the sequence)
+  vec8 kreg[NCH], vreg[NCH];
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int idx = tid + 256 * i, tok = idx / KC, c = idx % KC;
       int gt = t0 + tok;
       gt = gt < len ? gt : len - 1;
       const int64_t src = ((int64_t)(begin + gt) * KH + kh) * D + c * 8;
-      ldsK[tok * KC + (c ^ (tok & (KC - 1)))] = *reinterpret_cast<const vec8*>(k + src);
-      const vec8 vv = *reinterpret_cast<const vec8*>(v + src);
+      kreg[i] = *reinterpret_cast<const vec8*>(k + src);
+      vreg[i] = *reinterpret_cast<const vec8*>(v + src);
+    }
+  };
+  fetch(0);
+  for (int t0 = 0; t0 < kv_end; t0 += 64) {
+    __syncthreads();
 #pragma unroll
-      for (int e = 0; e < 8; ++e) ldsVt[(c * 8 + e) * VP + tok] = vv[e];
+    for (int i = 0; i < NCH; ++i) {
+      const int idx = tid + 256 * i, tok = idx / KC, c = idx % KC;
+      ldsK[tok * KC + (c ^ (tok & (KC - 1)))] = kreg[i];
+      ldsV[tok * KC + (c ^ (tok & (KC - 1)))] = vreg[i];
     }
     __syncthreads();
+    fetch(t0 + 64 < kv_end ? t0 + 64 : t0);
 
     f32x4 st[4];
 #pragma unroll
@@ -924,42 +938,62 @@ prefill_attn_kernel(T* __restrict__ out, const T* __restrict__ q, const T* __res
         st[j] = HalfMfma<T>::run(ldsK[tok * KC + (c ^ (tok & (KC - 1)))], qf[kk], st[j]);
       }
     }
-    float mx = -1.0e30f;
+    // Only a tile that reaches this wave's diagonal or the end of the sequence needs the causal mask (the test is
+    // the same for the whole wave).  The softmax is the wave's arithmetic cost, several times the MFMAs': scores stay
+    // unscaled and the scale goes into the one multiply-add in front of the hardware exp2.
+    const bool edge = t0 + 63 > q0 + 16 * wave || t0 + 63 >= len;
+    float mx = -3.0e38f;
+    if (edge) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int tk = t0 + 16 * j + 4 * grp + i;
-        const bool ok = tk <= qpos && tk < len;
-        st[j][i] = ok ? st[j][i] * scale_log2e : -1.0e30f;
-        mx = fmaxf(mx, st[j][i]);
-      }
+        for (int i = 0; i < 4; ++i) {
+          const int tk = t0 + 16 * j + 4 * grp + i;
+          st[j][i] = (tk <= qpos && tk < len) ? st[j][i] : -3.0e38f;
+          mx = fmaxf(mx, st[j][i]);
+        }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mx = fmaxf(mx, st[j][i]);
+    }
     mx = max_lane_xor32(max_lane_xor16(mx));
-    const float mnew = fmaxf(m, mx);
-    const float alpha = exp2f(m - mnew);
+    const float mnew = fmaxf(m, fmaxf(mx * scale_log2e, -1.0e30f));   // a fully masked row keeps its old maximum
+    const float alpha = __builtin_amdgcn_exp2f(m - mnew);
     float rs = 0.f;
     vec8 pf[2];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float p = st[j][i] > -0.9e30f ? exp2f(st[j][i] - mnew) : 0.f;
+        const float p = __builtin_amdgcn_exp2f(fmaf(st[j][i], scale_log2e, -mnew));   // masked: exp2(-inf) = 0
         rs += p;
         pf[j >> 1][(j & 1) * 4 + i] = (T)p;
       }
     rs = add_lane_xor32(add_lane_xor16(rs));
     l = fmaf(l, alpha, rs);
     m = mnew;
+    const bool rescale = __any(alpha != 1.0f);   // the running maximum rarely moves after the first tiles
 #pragma unroll
     for (int dd = 0; dd < D / 16; ++dd) {
+      if (rescale) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) o[dd][i] *= alpha;
-      const T* vrow = ldsVt + (16 * dd + r) * VP + 4 * grp;
+        for (int i = 0; i < 4; ++i) o[dd][i] *= alpha;
+      }
 #pragma unroll
       for (int kk2 = 0; kk2 < 2; ++kk2) {
-        const vec4 lo = *reinterpret_cast<const vec4*>(vrow + 16 * (2 * kk2));
-        const vec4 hi = *reinterpret_cast<const vec4*>(vrow + 16 * (2 * kk2 + 1));
-        const vec8 vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        // tokens 32 kk2 + 4 grp + 0..3 and the same + 16 of dim 16 dd + r: the order P holds them in
+        vec4 half[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int tok = 32 * kk2 + 16 * h + 4 * grp + (r >> 2), c = 2 * dd + ((r & 3) >> 1);
+          const char* piece = reinterpret_cast<const char*>(&ldsV[tok * KC + (c ^ (tok & (KC - 1)))]) + 8 * (r & 1);
+          typedef short s16x4_t __attribute__((ext_vector_type(4)));
+          const s16x4_t raw = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)piece);
+          half[h] = __builtin_bit_cast(vec4, raw);
+        }
+        const vec8 vf = {half[0][0], half[0][1], half[0][2], half[0][3], half[1][0], half[1][1], half[1][2], half[1][3]};
         o[dd] = HalfMfma<T>::run(vf, pf[kk2], o[dd]);
       }
     }
