@@ -468,10 +468,11 @@ def test_varlen_prefill_attention_matches_causal_sdpa(ops, dim, qh, kh):
         torch.testing.assert_close(got[a:b], want, atol=0.02, rtol=0.02)
 
 
+@pytest.mark.parametrize("H", [128, 100])     # 16-byte accesses, 8 channels x 4 tokens per thread; scalar form
 @torch.inference_mode()
-def test_packed_prefill_conv_and_kv_store_match_per_sequence_oracle(ops):
+def test_packed_prefill_conv_and_kv_store_match_per_sequence_oracle(ops, H):
     torch.manual_seed(12)
-    H, lengths, slots = 128, [1, 2, 5, 3, 40], [4, 0, 2, 5, 1]
+    lengths, slots = [1, 2, 5, 3, 40], [4, 0, 2, 5, 1]
     total = sum(lengths)
     cu = torch.tensor([0, *torch.tensor(lengths).cumsum(0).tolist()], dtype=torch.int32)
     bcx = torch.randn(total, 3 * H).bfloat16()
