@@ -774,6 +774,56 @@ __global__ void __launch_bounds__(kThreads) prepare_qkv_wave_kernel(PrepArgs a) 
   }
 }
 
+// head_dim 64 into q, k, v tensors (prefill: thousands of rows), 16 bytes per access: eight lanes share a head
+// unit, lane s of the eight owns elements 8s .. 8s+7, its rotate-half partner is the lane four away.  Same rounding
+// points as the wave-per-unit form.
+template <typename T>
+__global__ void __launch_bounds__(kThreads) prepare_qkv_vec64_kernel(PrepArgs a) {
+  typedef T vec8 __attribute__((ext_vector_type(8)));
+  constexpr int D = 64, half = 32;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, sub = lane & 7;
+  const int U = a.QH + 2 * a.KH;
+  const int64_t units = a.M * U;
+  int64_t unit = ((int64_t)blockIdx.x * kWaves + wave) * 8 + (lane >> 3);
+  const bool live = unit < units;
+  unit = live ? unit : units - 1;
+  const int64_t row = unit / U;
+  const int u = (int)(unit % U);
+  const vec8 raw = *reinterpret_cast<const vec8*>((const T*)a.x + row * U * D + (int64_t)u * D + 8 * sub);
+  float val[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) val[e] = Elem<T>::load(raw[e]);
+  if (u < a.QH + a.KH) {
+    const vec8 gw = *reinterpret_cast<const vec8*>((u < a.QH ? (const T*)a.qw : (const T*)a.kw) + 8 * sub);
+    int64_t pos = a.positions[row];
+    pos = pos < 0 ? 0 : (pos >= a.max_positions ? a.max_positions - 1 : pos);
+    const f32x4* cs = reinterpret_cast<const f32x4*>(a.cosT + pos * half + 8 * (sub & 3));
+    const f32x4* sn = reinterpret_cast<const f32x4*>(a.sinT + pos * half + 8 * (sub & 3));
+    const f32x4 c0 = cs[0], c1 = cs[1], s0 = sn[0], s1 = sn[1];
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += val[e] * val[e];
+    ss += __shfl_xor(ss, 1, 64); ss += __shfl_xor(ss, 2, 64); ss += __shfl_xor(ss, 4, 64);
+    const float rstd = 1.0f / sqrtf(ss / (float)D + a.eps);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float n = round_to<T>(val[e] * rstd);
+      const float w = round_to<T>(n * Elem<T>::load(gw[e]));
+      const float partner = __shfl_xor(w, 4, 64);
+      const float c = round_to<T>(e < 4 ? c0[e & 3] : c1[e & 3]), s = round_to<T>(e < 4 ? s0[e & 3] : s1[e & 3]);
+      const float left = round_to<T>(w * c), right = round_to<T>(partner * s);
+      val[e] = round_to<T>(sub < 4 ? left - right : left + right);
+    }
+  }
+  if (!live) return;
+  vec8 outv;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) outv[e] = Elem<T>::store(val[e]);
+  T* dst = u < a.QH ? (T*)a.q + (row * a.QH + u) * D
+                    : (u < a.QH + a.KH ? (T*)a.k + (row * a.KH + (u - a.QH)) * D : (T*)a.v + (row * a.KH + (u - a.QH - a.KH)) * D);
+  *reinterpret_cast<vec8*>(dst + 8 * sub) = outv;
+}
+
 template <typename T, int STORE>
 int launch_prepare(const PrepArgs& a, int D, hipStream_t s) {
   const int64_t units = a.M * (a.QH + 2 * a.KH);
@@ -797,6 +847,14 @@ extern "C" int lfm2_prepare_qkv(void* q, void* k, void* v, const void* x, const 
   if (D == 32 || D == 64 || D == 128 || D == 256) {
     const PrepArgs a{q, k, v, x, q_weight, k_weight, cos, sin, positions, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
                      M, max_positions, 0, 0, 0, QH, KH, eps};
+    const uintptr_t pointers = (uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)x | (uintptr_t)q_weight |
+                               (uintptr_t)k_weight | (uintptr_t)cos | (uintptr_t)sin;
+    if (D == 64 && dtype != LFM2_DTYPE_F32 && M >= 512 && (pointers & 15) == 0) {
+      const dim3 grid(ceil_div(M * (QH + 2 * KH), kWaves * 8));
+      if (dtype == LFM2_DTYPE_BF16) hipLaunchKernelGGL(prepare_qkv_vec64_kernel<__bf16>, grid, dim3(kThreads), 0, (hipStream_t)stream, a);
+      else hipLaunchKernelGGL(prepare_qkv_vec64_kernel<_Float16>, grid, dim3(kThreads), 0, (hipStream_t)stream, a);
+      LFM2_LAUNCH_CHECK();
+    }
     DISPATCH_DTYPE(dtype, (launch_prepare<T, 0>(a, D, (hipStream_t)stream)));
     LFM2_LAUNCH_CHECK();
   }

@@ -77,6 +77,26 @@ def test_fused_decode_kernels_match_oracle(ops, dtype):
     _close_mostly_exact(k, ek, dtype, 5e-3)
 
 
+@pytest.mark.parametrize("dtype", (torch.bfloat16, torch.float16))
+@torch.inference_mode()
+def test_prepare_qkv_on_a_prefill_sized_batch_matches_oracle(ops, dtype):
+    """From 512 rows on, head_dim 64 runs the 16-bytes-per-lane form (eight lanes per head); the rows' count is not a
+    multiple of what a workgroup takes, positions are spread over the rotary table."""
+    torch.manual_seed(19)
+    rows, QH, KH, D = 777, 32, 8, 64
+    qkv = torch.randn(rows, (QH + 2 * KH) * D, dtype=dtype)
+    qw, kw = torch.randn(D, dtype=dtype), torch.randn(D, dtype=dtype)
+    pos = torch.randint(0, 4096, (rows,), dtype=torch.int32)
+    cos, sin = O.rope_tables(D, 1e6, 4096)
+    q, k, v = ops.prepare_qkv(qkv.to(DEV), qw.to(DEV), kw.to(DEV), cos.to(DEV), sin.to(DEV), pos.to(DEV), QH, KH, D, 1e-5)
+    eq, ek, ev = O.k_prepare_qkv(qkv, qw, kw, cos, sin, pos, QH, KH, D, 1e-5)
+    assert torch.equal(v.cpu(), ev)
+    _close_mostly_exact(q, eq, dtype, 5e-3)
+    _close_mostly_exact(k, ek, dtype, 5e-3)
+    few = ops.prepare_qkv(qkv[:40].to(DEV), qw.to(DEV), kw.to(DEV), cos.to(DEV), sin.to(DEV), pos[:40].to(DEV), QH, KH, D, 1e-5)
+    _close_mostly_exact(q[:40], few[0].cpu(), dtype, 5e-3)      # the wave-per-head form on the same rows
+
+
 @torch.inference_mode()
 def test_conv_update_masks_rows_and_follows_slot_ids(ops):
     torch.manual_seed(3)
