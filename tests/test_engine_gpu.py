@@ -56,7 +56,7 @@ def _flat(prompts):
 
 # ------------------------------------------------------------------------------------------------ config 1
 def _config1():
-    """BASELINE config 1: hidden 256, [conv, attn, conv, attn], 4 q / 2 kv heads, head_dim 64, SwiGLU 768, vocab 4096,
+    """The small CPU-runnable benchmark configuration: hidden 256, [conv, attn, conv, attn], 4 q / 2 kv heads, head_dim 64, SwiGLU 768, vocab 4096,
     N(0, 0.02) weights from seed 0; prompts of 7, 33, 64 and 120 uniform token ids."""
     engine, ocfg, state = _engine(TINY, seed=0, max_model_len=256)
     g = torch.Generator().manual_seed(0)
