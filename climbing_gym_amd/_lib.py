@@ -29,6 +29,8 @@ _SIGNATURES = {
     "lfm2_prepare_qkv_store": "ppppppppppppp" "liiilflllii" "p",
     "lfm2_rms_norm_fp8_split": "pppp" "i" "pppp" "llfip",
     "lfm2_fp8_gemm_partials": "ppp" "llliip",
+    "lfm2_bf16_gemm_partials": "ppp" "llliip",
+    "lfm2_rms_norm_split": "ppp" "i" "pppp" "llfip",
     "lfm2_prepare_qkv": "ppppppppp" "liiilfip",
     "lfm2_conv_prefill": "ppppppp" "llllip",
     "lfm2_fp8_gemm": "pppppp" "llliiip",
@@ -54,6 +56,7 @@ _SIGNATURES = {
 _INT64_RESULT = {
     "lfm2_fp8_gemm_workspace": "lll",
     "lfm2_fp8_gemm_default_splits": "lll",
+    "lfm2_bf16_gemm_default_splits": "lll",
     "lfm2_bf16_gemm_workspace": "lll",
     "lfm2_decode_attention_workspace": "liil",
     "lfm2_decode_schedule_size": "ll",

@@ -125,7 +125,7 @@ rms_norm_kernel(T* out, uint8_t* q, float* scales, T* summed, const T* x, const 
       const int64_t i = (int64_t)(j * kRowThreads + threadIdx.x) * N;
       if (i < H) {
         if (split.partial) {
-          const float sa = split.a_scales[row];
+          const float sa = split.a_scales ? split.a_scales[row] : 1.0f;   // a bf16 product has no scales
 #pragma unroll
           for (int e = 0; e < N; ++e) v[j][e] = 0.f;
           for (int sp = 0; sp < split.splits; ++sp) {
@@ -134,7 +134,7 @@ rms_norm_kernel(T* out, uint8_t* q, float* scales, T* summed, const T* x, const 
             for (int e = 0; e < N; ++e) v[j][e] += p[e];
           }
 #pragma unroll
-          for (int e = 0; e < N; ++e) v[j][e] = round_to<T>((v[j][e] * sa) * split.w_scales[i + e]);
+          for (int e = 0; e < N; ++e) v[j][e] = round_to<T>(split.w_scales ? (v[j][e] * sa) * split.w_scales[i + e] : v[j][e]);
         } else {
           load_vec<T>(x + i, v[j]);
         }
@@ -267,7 +267,8 @@ extern "C" int lfm2_rms_norm_fp8_split(uint8_t* q, float* scales, void* summed, 
                                        const float* a_scales, const float* w_scales, const void* weight,
                                        const void* residual, int64_t M, int64_t H, float eps, int dtype, void* stream) {
   LFM2_REQUIRE(M > 0 && H > 0, "rms_norm_fp8_split: empty shape");
-  LFM2_REQUIRE(partial && a_scales && w_scales && splits >= 1, "rms_norm_fp8_split: partial products and both scale vectors are required");
+  LFM2_REQUIRE(partial && splits >= 1, "rms_norm_fp8_split: partial products are required");
+  LFM2_REQUIRE((a_scales == nullptr) == (w_scales == nullptr), "rms_norm_fp8_split: both scale vectors or neither");
   LFM2_REQUIRE(residual == nullptr || summed != nullptr, "rms_norm_fp8_split: residual given without a summed output");
   const int vec = dtype == LFM2_DTYPE_F32 ? 4 : 8;
   LFM2_REQUIRE(H % vec == 0 && H <= (int64_t)16 * kRowThreads * vec, "rms_norm_fp8_split: width %ld is not a multiple of %d or too wide", (long)H, vec);
@@ -275,6 +276,22 @@ extern "C" int lfm2_rms_norm_fp8_split(uint8_t* q, float* scales, void* summed, 
   hipStream_t s = (hipStream_t)stream;
   DISPATCH_DTYPE(dtype, if (residual) launch_rms<T, true, true>(nullptr, q, scales, summed, nullptr, weight, residual, M, H, eps, s, split);
                  else launch_rms<T, false, true>(nullptr, q, scales, nullptr, nullptr, weight, nullptr, M, H, eps, s, split));
+  LFM2_LAUNCH_CHECK();
+}
+
+extern "C" int lfm2_rms_norm_split(void* out, void* summed, const float* partial, int splits, const float* a_scales,
+                                   const float* w_scales, const void* weight, const void* residual, int64_t M, int64_t H,
+                                   float eps, int dtype, void* stream) {
+  LFM2_REQUIRE(M > 0 && H > 0, "rms_norm_split: empty shape");
+  LFM2_REQUIRE(partial && splits >= 1, "rms_norm_split: partial products are required");
+  LFM2_REQUIRE((a_scales == nullptr) == (w_scales == nullptr), "rms_norm_split: both scale vectors or neither");
+  LFM2_REQUIRE(residual == nullptr || summed != nullptr, "rms_norm_split: residual given without a summed output");
+  const int vec = dtype == LFM2_DTYPE_F32 ? 4 : 8;
+  LFM2_REQUIRE(H % vec == 0 && H <= (int64_t)16 * kRowThreads * vec, "rms_norm_split: width %ld is not a multiple of %d or too wide", (long)H, vec);
+  const SplitInput split{partial, a_scales, w_scales, M * H, splits};
+  hipStream_t s = (hipStream_t)stream;
+  DISPATCH_DTYPE(dtype, if (residual) launch_rms<T, true, false>(out, nullptr, nullptr, summed, nullptr, weight, residual, M, H, eps, s, split);
+                 else launch_rms<T, false, false>(out, nullptr, nullptr, nullptr, nullptr, weight, nullptr, M, H, eps, s, split));
   LFM2_LAUNCH_CHECK();
 }
 

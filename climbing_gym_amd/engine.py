@@ -240,7 +240,7 @@ class LFM25Engine:
         if packed is not None:
             q, scales, residual = ops.rms_norm_fp8(x, norm_weight, self.config.norm_eps, residual)
             return packed.linear_quantized(q, scales, dtype=self.dtype, place=place), residual
-        if isinstance(x, ops.SplitProduct):
+        if isinstance(x, ops.SplitProduct) and residual is None:
             x = x.materialize()
         normed, residual = ops.rms_norm(x, norm_weight, self.config.norm_eps, residual)
         return ops.linear(normed, weight, place=place), residual
@@ -273,7 +273,7 @@ class LFM25Engine:
                 q, scales = ops.swiglu_fp8(gate_up)
                 hidden = down.linear_quantized(q, scales, dtype=self.dtype, defer_reduce=defer_reduce)
             else:
-                hidden = ops.linear(ops.swiglu(gate_up), layer.w2_weight)
+                hidden = ops.linear(ops.swiglu(gate_up), layer.w2_weight, defer_reduce=defer_reduce)
         return hidden, residual
 
     def _head(self, hidden, residual, fp8, place=None):

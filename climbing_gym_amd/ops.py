@@ -50,8 +50,19 @@ def embedding(tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
     return out.view(*tokens.shape, table.size(1))
 
 
-def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: torch.Tensor | None = None):
-    """lfm25_cuda_kernels.py:47-55: returns (norm(x+residual)*w, x+residual); `summed is x` without residual."""
+def rms_norm(x, weight: torch.Tensor, eps: float, residual: torch.Tensor | None = None):
+    """lfm25_cuda_kernels.py:47-55: returns (norm(x+residual)*w, x+residual); `summed is x` without residual.
+    `x` may be a `SplitProduct` (then a residual is required and the projection's reduce pass runs inside the norm)."""
+    if isinstance(x, SplitProduct):
+        _check(weight, residual)
+        if residual is None:
+            raise ValueError("a deferred projection can only feed a norm that adds a residual")
+        rows, width = x.shape
+        out = torch.empty((rows, width), device=weight.device, dtype=x.dtype)
+        summed = torch.empty_like(out)
+        call("lfm2_rms_norm_split", out, summed, x.partials, x.partials.size(0), x.a_scales, x.w_scales, weight, residual,
+             rows, width, float(eps), _code(x.dtype))
+        return out, summed
     _check(x, weight, residual)
     out = torch.empty_like(x)
     summed = torch.empty_like(x) if residual is not None else x
@@ -62,12 +73,13 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: torch.
 
 @dataclass
 class SplitProduct:
-    """An FP8 projection left as split-K partial sums (`PackedFP8Weight.linear_quantized(..., defer_reduce=True)`):
-    the value is round((sum of partials) * a_scales[m] * w_scales[n]) in `dtype`.  `rms_norm_fp8` folds that reduction
-    into its own pass; `materialize()` gives the ordinary tensor."""
+    """A projection left as split-K partial sums (`PackedFP8Weight.linear_quantized(..., defer_reduce=True)`,
+    `linear(..., defer_reduce=True)`): the value is round((sum of partials) * a_scales[m] * w_scales[n]) in `dtype`,
+    without the scales for a bf16 product.  `rms_norm_fp8` and `rms_norm` fold that reduction into their own pass;
+    `materialize()` gives the ordinary tensor."""
     partials: torch.Tensor   # [splits, M, N] fp32
-    a_scales: torch.Tensor
-    w_scales: torch.Tensor
+    a_scales: Optional[torch.Tensor]
+    w_scales: Optional[torch.Tensor]
     dtype: torch.dtype
 
     @property
@@ -78,6 +90,8 @@ class SplitProduct:
         total = self.partials[0].clone()
         for part in self.partials[1:]:
             total += part
+        if self.a_scales is None:
+            return total.to(self.dtype)
         return ((total * self.a_scales[:, None]) * self.w_scales[None, :]).to(self.dtype)
 
 
@@ -222,9 +236,10 @@ class RowPlacement:
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, *, tile: int = -1, split_k: int = 0,
-           place: Optional[RowPlacement] = None) -> torch.Tensor:
+           place: Optional[RowPlacement] = None, defer_reduce: bool = False):
     """lfm25_cuda_kernels.py:19-29: y = x W^T.  bf16 runs the MFMA kernel of this package; other dtypes
-    (only used by tests of the fp32 plumbing) go to the vendor GEMM.  With `place`, rows land in `place.out`."""
+    (only used by tests of the fp32 plumbing) go to the vendor GEMM.  With `place`, rows land in `place.out`.  With
+    `defer_reduce`, a product the plan splits along K comes back as a `SplitProduct` for `rms_norm` to reduce."""
     if x.dtype != torch.bfloat16:
         if place is not None:
             raise ValueError("placed rows need a bf16 product")
@@ -238,6 +253,12 @@ def linear(x: torch.Tensor, weight: torch.Tensor, *, tile: int = -1, split_k: in
         place.check(m, n, x.dtype)
         call("lfm2_bf16_gemm_rows", place.out, x, weight, place.slots, place.active, place.out.size(0), m, n, k, tile)
         return place.out
+    if defer_reduce and x.ndim == 2:
+        splits = query("lfm2_bf16_gemm_default_splits", m, n, k) if split_k == 0 else split_k
+        if splits > 1:
+            partials = torch.empty((splits, m, n), device=x.device, dtype=torch.float32)
+            call("lfm2_bf16_gemm_partials", partials, x, weight, m, n, k, tile, splits)
+            return SplitProduct(partials, None, None, x.dtype)
     out = torch.empty((*x.shape[:-1], n), device=x.device, dtype=x.dtype)
     need = query("lfm2_bf16_gemm_workspace", m, n, k) if split_k == 0 else max(split_k, 1) * m * n
     ws = torch.empty(need, device=x.device, dtype=torch.float32) if need and split_k != 1 else None

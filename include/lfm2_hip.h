@@ -46,10 +46,17 @@ int lfm2_rms_norm_fp8(uint8_t* q, float* scales, void* summed, const void* x, co
 /* rms_norm_fp8 whose input x[M,H] is given as split-K partial products of an FP8 projection:
  * x = round((sum_s partial[s]) * a_scales[m] * w_scales[h]) in the model dtype, i.e. what lfm2_fp8_gemm would have
  * stored; then exactly lfm2_rms_norm_fp8.  Fuses the projection's reduce pass into the norm that follows it in
- * lfm25_cuda.py:166-184. */
+ * lfm25_cuda.py:166-184.  (a_scales and w_scales both NULL: partial products of a bf16 projection, no scaling.) */
 int lfm2_rms_norm_fp8_split(uint8_t* q, float* scales, void* summed, const float* partial, int splits,
                             const float* a_scales, const float* w_scales, const void* weight, const void* residual,
                             int64_t M, int64_t H, float eps, int dtype, void* stream);
+
+/* rms_norm (model-dtype output) over the same kind of input; a_scales and w_scales both NULL for the partial
+ * products of a bf16 projection (lfm2_bf16_gemm_partials), whose value is round(sum_s partial[s]).  The fused
+ * add + norm of lfm25_cuda_kernels.py:32-55 with the projection's reduce pass folded in. */
+int lfm2_rms_norm_split(void* out, void* summed, const float* partial, int splits, const float* a_scales,
+                        const float* w_scales, const void* weight, const void* residual, int64_t M, int64_t H, float eps,
+                        int dtype, void* stream);
 
 /* swiglu of lfm25_cuda_kernels.py:58-72.  x [M,2I] (gate first) -> out [M,I]. */
 int lfm2_swiglu(void* out, const void* x, int64_t M, int64_t I, int dtype, void* stream);
@@ -122,6 +129,11 @@ int64_t lfm2_fp8_gemm_workspace(int64_t M, int64_t N, int64_t K);
 int lfm2_bf16_gemm(void* out, const void* x, const void* w, float* workspace, int64_t M, int64_t N, int64_t K,
                    int tile, int split_k, void* stream);
 int64_t lfm2_bf16_gemm_workspace(int64_t M, int64_t N, int64_t K);
+/* The bf16 product left as split-K partial sums, float[split_k, M, N] (see lfm2_fp8_gemm_partials), and the split
+ * count lfm2_bf16_gemm would choose for a shape.  No counterpart in the reference. */
+int lfm2_bf16_gemm_partials(float* partials, const void* x, const void* w, int64_t M, int64_t N, int64_t K, int tile,
+                            int split_k, void* stream);
+int64_t lfm2_bf16_gemm_default_splits(int64_t M, int64_t N, int64_t K);
 
 /* The two products with placed output rows: row m of the product is written to out row out_rows[m] (m itself when
  * out_rows is NULL) unless that index is negative or >= out_capacity, or row_active[m] is 0 (row_active may be

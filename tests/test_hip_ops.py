@@ -797,3 +797,26 @@ def test_split_k_partials_reduce_inside_the_following_norm(ops):
     assert torch.equal(got[2].view(torch.int16), expected[2].view(torch.int16))
     unsplit = weight.linear_quantized(xq, xs, defer_reduce=True)
     assert isinstance(unsplit, torch.Tensor)  # nothing to defer when the plan does not split
+
+
+@torch.inference_mode()
+def test_bf16_split_k_partials_reduce_inside_the_following_norm(ops):
+    """The bf16 down projection at decode size is split along K by default; left as partial sums and reduced by the
+    norm that follows, it gives the bytes of the materialised projection followed by rms_norm (and by rms_norm_fp8)."""
+    torch.manual_seed(31)
+    rows, width, outputs = 256, 5632, 2048
+    act = torch.randn(rows, width, dtype=torch.bfloat16, device=DEV)
+    weight = torch.randn(outputs, width, dtype=torch.bfloat16, device=DEV) * 0.02
+    norm_w = torch.randn(outputs, dtype=torch.bfloat16, device=DEV)
+    residual = torch.randn(rows, outputs, dtype=torch.bfloat16, device=DEV)
+    deferred = ops.linear(act, weight, defer_reduce=True)
+    assert isinstance(deferred, ops.SplitProduct) and deferred.partials.size(0) == 4 and deferred.a_scales is None
+    whole = ops.linear(act, weight)
+    assert torch.equal(deferred.materialize().view(torch.int16), whole.view(torch.int16))
+    torch.testing.assert_close(whole.float(), act.float() @ weight.float().T, atol=0.06, rtol=0.02)
+    expected, got = ops.rms_norm(whole, norm_w, 1e-5, residual), ops.rms_norm(deferred, norm_w, 1e-5, residual)
+    assert torch.equal(got[0].view(torch.int16), expected[0].view(torch.int16))
+    assert torch.equal(got[1].view(torch.int16), expected[1].view(torch.int16))
+    expected, got = ops.rms_norm_fp8(whole, norm_w, 1e-5, residual), ops.rms_norm_fp8(deferred, norm_w, 1e-5, residual)
+    assert torch.equal(got[0].view(torch.uint8), expected[0].view(torch.uint8)) and torch.equal(got[1], expected[1])
+    assert isinstance(ops.linear(act[:, :2048].contiguous(), weight[:, :2048].contiguous(), defer_reduce=True), torch.Tensor)
