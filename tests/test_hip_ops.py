@@ -466,8 +466,17 @@ def test_paged_slot_mapped_history_equals_dense_history(ops, fp8):
         else:
             pool[table.view(-1).long().to(DEV)] = src
         return pool
-    paged = ops.attend(q, to_pages(kc), to_pages(vc), None if ks is None else to_pages(ks), None if vs is None else to_pages(vs),
-                       positions, block_table=table.to(DEV), page=page)
+    pools = [to_pages(kc), to_pages(vc), None if ks is None else to_pages(ks), None if vs is None else to_pages(vs)]
+    paged = ops.attend(q, *pools, positions, block_table=table.to(DEV), page=page)
+    assert torch.equal(paged, dense)
+    # the same pages stored head-major ([pages, heads, page, ...] behind the [pages, page, heads, ...] view): the
+    # strides of a page are arguments, and a head's tokens are then contiguous inside a page
+    def head_major(t):
+        if t is None:
+            return None
+        rest = range(3, t.ndim)
+        return t.permute(0, 2, 1, *rest).contiguous().permute(0, 2, 1, *rest)
+    paged = ops.attend(q, *[head_major(t) for t in pools], positions, block_table=table.to(DEV), page=page)
     assert torch.equal(paged, dense)
 
 
