@@ -39,7 +39,7 @@ def parse_args():
     p.add_argument("--max-model-len", type=int, default=8192)
     p.add_argument("--precision", choices=("fp8", "bf16"), default="fp8")
     p.add_argument("--cpu-seqs", type=int, default=4, help="sequences of the workload the CPU baseline runs (0 = skip)")
-    p.add_argument("--cpu-steps", type=int, default=8)
+    p.add_argument("--cpu-steps", type=int, default=96)
     p.add_argument("--attn-samples", type=int, default=20, help="timed launches of the decode-attention kernel per layer")
     p.add_argument("--top-k", type=int, default=0, help="top-k filter of the sampler (0: full support)")
     p.add_argument("--top-p", type=float, default=1.0, help="top-p filter of the sampler (1: off)")
