@@ -29,6 +29,7 @@ _SIGNATURES = {
     "lfm2_prepare_qkv_store": "ppppppppppppp" "liiilflllii" "p",
     "lfm2_rms_norm_fp8_split": "pppp" "i" "pppp" "llfip",
     "lfm2_fp8_gemm_partials": "ppp" "llliip",
+    "lfm2_fp8_gemm_qkv_store": "pppppppppppppppp" "liiillflllii" "p",
     "lfm2_bf16_gemm_partials": "ppp" "llliip",
     "lfm2_rms_norm_split": "ppp" "i" "pppp" "llfip",
     "lfm2_prepare_qkv": "ppppppppp" "liiilfip",

@@ -77,11 +77,28 @@ __device__ __forceinline__ void store_out(void* out, int out_dtype, int64_t idx,
   else ((float*)out)[idx] = v;
 }
 
-template <int EB, int BM, int BN, int WM, int WN, int SW, int KS, bool KTAIL, int ST = 0>
+// Epilogue of the fused QKV projection (EPI = 1; 64 x 64 tiles, head_dim 64, so a column tile is one head of 64 rows):
+// what prepare_qkv with cache append does to the projection's bf16 output (lfm25_cuda_kernels.py:113-151 then the
+// append of lfm25_fp8_kv.py:58-69 or lfm25_batching.py:49-69), with the same rounding points and the same
+// summation tree for the head's mean square, so the results are bit for bit those of the two launches.
+struct QkvEpilogue {
+  void* q;                 // [M, QH, 64] model dtype
+  const void *qw, *kw;     // q/k norm weights [64]
+  const float *cosT, *sinT;
+  const int32_t *positions, *slot_ids;
+  const uint8_t* active;
+  void *kc, *vc;           // caches addressed slot*c0 + pos*c1 + head*c2 + d
+  float *ks, *vs;          // e4m3 cache scales (same offsets / 64) or NULL for a model-dtype cache
+  int64_t max_positions, c0, c1, c2;
+  int QH, KH;
+  float eps;
+};
+
+template <int EB, int BM, int BN, int WM, int WN, int SW, int KS, bool KTAIL, int ST = 0, int EPI = 0>
 __global__ void __launch_bounds__(WM * WN * 64)
 gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_t* __restrict__ A,
                const uint8_t* __restrict__ W, const float* __restrict__ a_scales, const float* __restrict__ w_scales,
-               int M, int N, int64_t Kb, int steps_per_split, int out_dtype, RowMap rows) {
+               int M, int N, int64_t Kb, int steps_per_split, int out_dtype, RowMap rows, QkvEpilogue epi) {
   constexpr int NT = WM * WN * 64;
   constexpr int TM = BM / WM, TN = BN / WN, MI = TM / 16, NI = TN / 16;
   constexpr int kChunksPerRow = KS / 16;  // KS = K bytes staged per step and row: 128, or 256 (two MFMA sub-steps per barrier)
@@ -268,6 +285,117 @@ gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_
   }
   }
 
+  if constexpr (EPI == 1) {
+    static_assert(BM == 64 && BN == 64 && NT == 256 && EB == 1, "the QKV epilogue works on 64 x 64 tiles of 256 threads");
+    typedef __bf16 T;
+    constexpr int LD = 68;   // padded row of the fp32 tile
+    // every load into LDS has landed and every wave is done with the staged operands: the ring becomes the tile
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    float* tile = reinterpret_cast<float*>(&lds[0][0]);
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+      const int ml = wm * TM + i * 16 + lrow;
+      const int mg = m_base + ml < M ? m_base + ml : M - 1;
+      const float sa = a_scales[mg];
+#pragma unroll
+      for (int j = 0; j < NI; ++j) {
+        const int nl = wn * TN + j * 16 + 4 * lgrp;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) tile[ml * LD + nl + r] = round_to<T>((acc[i][j][r] * sa) * w_scales[n_base + nl + r]);
+      }
+    }
+    __syncthreads();
+    // four adjacent lanes own a row of the head: 16 consecutive dims each
+    const int row = tid >> 2, part = tid & 3;
+    const bool live = m_base + row < M;
+    const int64_t m = live ? m_base + row : M - 1;
+    const int u = n_base / 64;   // head unit: query heads, then key heads, then value heads
+    float val[16];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) val[e] = tile[row * LD + 16 * part + e];
+    if (u < epi.QH + epi.KH) {
+      typedef T vec8 __attribute__((ext_vector_type(8)));
+      const T* wgt = (u < epi.QH ? (const T*)epi.qw : (const T*)epi.kw) + 16 * part;
+      const vec8 g0 = *reinterpret_cast<const vec8*>(wgt), g1 = *reinterpret_cast<const vec8*>(wgt + 8);
+      int64_t pos = epi.positions[m];
+      pos = pos < 0 ? 0 : (pos >= epi.max_positions ? epi.max_positions - 1 : pos);
+      const f32x4* cs = reinterpret_cast<const f32x4*>(epi.cosT + pos * 32 + 16 * (part & 1));
+      const f32x4* sn = reinterpret_cast<const f32x4*>(epi.sinT + pos * 32 + 16 * (part & 1));
+      float c[16], sv[16];
+#pragma unroll
+      for (int v4 = 0; v4 < 4; ++v4) {
+        const f32x4 cv = cs[v4], xv = sn[v4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { c[4 * v4 + e] = round_to<T>(cv[e]); sv[4 * v4 + e] = round_to<T>(xv[e]); }
+      }
+      // mean square by the pairwise tree of a wave's butterfly reduction over one dim per lane
+      float sq[16];
+#pragma unroll
+      for (int e = 0; e < 16; ++e) sq[e] = val[e] * val[e];
+#pragma unroll
+      for (int width = 1; width < 16; width *= 2)
+#pragma unroll
+        for (int e = 0; e < 16; e += 2 * width) sq[e] = sq[e] + sq[e + width];
+      float ss = sq[0];
+      ss = ss + __shfl_xor(ss, 1, 64);
+      ss = ss + __shfl_xor(ss, 2, 64);
+      const float rstd = 1.0f / sqrtf(ss / 64.0f + epi.eps);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const float nrm = round_to<T>(val[e] * rstd);
+        val[e] = round_to<T>(nrm * Elem<T>::load(e < 8 ? g0[e & 7] : g1[e & 7]));
+      }
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const float partner = __shfl_xor(val[e], 2, 64);   // the dim 32 away
+        const float left = round_to<T>(val[e] * c[e]), right = round_to<T>(partner * sv[e]);
+        sq[e] = round_to<T>(part < 2 ? left - right : left + right);
+      }
+#pragma unroll
+      for (int e = 0; e < 16; ++e) val[e] = sq[e];
+    }
+    typedef T vec8 __attribute__((ext_vector_type(8)));
+    auto store_model = [&](T* dst) {
+      vec8 lo, hi;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { lo[e] = Elem<T>::store(val[e]); hi[e] = Elem<T>::store(val[8 + e]); }
+      *reinterpret_cast<vec8*>(dst) = lo;
+      *reinterpret_cast<vec8*>(dst + 8) = hi;
+    };
+    if (u < epi.QH) {
+      if (live) store_model((T*)epi.q + (m * epi.QH + u) * 64 + 16 * part);
+      return;
+    }
+    const bool is_v = u >= epi.QH + epi.KH;
+    const int h = is_v ? u - epi.QH - epi.KH : u - epi.QH;
+    float amax = 0.f;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(val[e]));
+    amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+    const int64_t slot = epi.slot_ids ? epi.slot_ids[m] : m;
+    const int64_t at = epi.positions[m];
+    if (!live || (epi.active && !epi.active[m]) || slot < 0 || at < 0) return;
+    const int64_t dst = slot * epi.c0 + at * epi.c1 + (int64_t)h * epi.c2;
+    if (epi.ks == nullptr) {
+      store_model((T*)(is_v ? epi.vc : epi.kc) + dst + 16 * part);
+    } else {
+      const float sc = fmaxf(amax / LFM2_E4M3_MAX, 1.0e-12f);
+      i32x4 packed;
+#pragma unroll
+      for (int wd = 0; wd < 4; ++wd) {
+        uint32_t bits = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) bits |= (uint32_t)to_e4m3(val[4 * wd + e] / sc) << (8 * e);
+        packed[wd] = (int)bits;
+      }
+      *reinterpret_cast<i32x4*>((uint8_t*)(is_v ? epi.vc : epi.kc) + dst + 16 * part) = packed;
+      if (part == 0) (is_v ? epi.vs : epi.ks)[dst / 64] = sc;
+    }
+    return;
+  }
+
   // Epilogue: lane holds out[m = .. + lrow][n = .. + 4*lgrp + r], r = 0..3.
   const bool split = partial != nullptr;
   auto finish = [&](f32x4 v, int m_out, int n, float sa) {  // scale (row then column) and store up to 4 columns
@@ -391,10 +519,20 @@ void launch_tile(void* out, float* partial, const uint8_t* A, const uint8_t* W, 
   const dim3 grid((tiles + 7) / 8 * 8, splits), block(WM * WN * 64);
   if (Kb % KS == 0)
     hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN, SW, KS, false, ST>), grid, block, 0, s, out, (splits > 1 || keep_partials) ? partial : nullptr, A, W,
-                       as, ws, M, N, Kb, per, out_dtype, rows);
+                       as, ws, M, N, Kb, per, out_dtype, rows, QkvEpilogue{});
   else
     hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN, SW, KS, true>), grid, block, 0, s, out, (splits > 1 || keep_partials) ? partial : nullptr, A, W,
-                       as, ws, M, N, Kb, per, out_dtype, rows);
+                       as, ws, M, N, Kb, per, out_dtype, rows, QkvEpilogue{});
+}
+
+// The fused QKV projection on one of the 64 x 64 tiles (ring of ST buffers, or register staged with ST = 0).
+template <int ST>
+void launch_qkv(const uint8_t* A, const uint8_t* W, const float* as, const float* ws, int M, int N, int64_t Kb,
+                const QkvEpilogue& epi, hipStream_t s) {
+  const int tiles = ((M + 63) / 64) * (N / 64);
+  const dim3 grid((tiles + 7) / 8 * 8, 1), block(256);
+  hipLaunchKernelGGL((gemm_nt_kernel<1, 64, 64, 2, 2, 1, 128, false, ST, 1>), grid, block, 0, s, nullptr, nullptr, A, W, as, ws, M,
+                     N, Kb, (int)(Kb / 128), LFM2_DTYPE_BF16, RowMap{nullptr, nullptr, 0x7fffffff}, epi);
 }
 
 template <int EB>
@@ -468,6 +606,35 @@ extern "C" int lfm2_fp8_gemm(void* out, const uint8_t* a_q, const float* a_scale
   LFM2_REQUIRE(a_scales && w_scales, "fp8_gemm: scales are required");
   LFM2_REQUIRE(split_k <= 16, "fp8_gemm: split_k above 16");
   return gemm_entry<1>("fp8_gemm", out, a_q, a_scales, w_q, w_scales, workspace, M, N, K, out_dtype, tile, split_k, stream);
+}
+
+extern "C" int lfm2_fp8_gemm_qkv_store(void* q, const uint8_t* a_q, const float* a_scales, const uint8_t* w_q,
+                                        const float* w_scales, const void* q_weight, const void* k_weight, const float* cos,
+                                        const float* sin, const int32_t* positions, void* k_cache, void* v_cache,
+                                        float* k_scales, float* v_scales, const uint8_t* active, const int32_t* slot_ids,
+                                        int64_t M, int QH, int KH, int D, int64_t K, int64_t max_positions, float eps,
+                                        int64_t c0, int64_t c1, int64_t c2, int kv_fp8, int dtype, void* stream) {
+  LFM2_REQUIRE(M > 0 && QH > 0 && KH > 0 && K > 0, "fp8_gemm_qkv_store: empty shape");
+  LFM2_REQUIRE(M < (1 << 30), "fp8_gemm_qkv_store: too many rows");
+  LFM2_REQUIRE(D == 64 && dtype == LFM2_DTYPE_BF16 && K % 128 == 0,
+               "fp8_gemm_qkv_store: needs head_dim 64, bf16 and K a multiple of 128 (got %d, dtype %d, %ld)", D, dtype, (long)K);
+  LFM2_REQUIRE(q && a_q && a_scales && w_q && w_scales && q_weight && k_weight && cos && sin && positions && k_cache && v_cache,
+               "fp8_gemm_qkv_store: a required pointer is null");
+  LFM2_REQUIRE(!kv_fp8 || (k_scales && v_scales), "fp8_gemm_qkv_store: e4m3 cache without scale tensors");
+  LFM2_REQUIRE(max_positions > 0, "fp8_gemm_qkv_store: empty rotary table");
+  LFM2_REQUIRE(c0 % 16 == 0 && c1 % 16 == 0 && c2 % 16 == 0, "fp8_gemm_qkv_store: cache strides must be multiples of 16 elements");
+  LFM2_REQUIRE((((uintptr_t)q | (uintptr_t)a_q | (uintptr_t)w_q | (uintptr_t)q_weight | (uintptr_t)k_weight | (uintptr_t)cos |
+                 (uintptr_t)sin | (uintptr_t)k_cache | (uintptr_t)v_cache) & 15) == 0, "fp8_gemm_qkv_store: pointers must be 16-byte aligned");
+  const QkvEpilogue epi{q, q_weight, k_weight, cos, sin, positions, slot_ids, active, k_cache, v_cache,
+                        kv_fp8 ? k_scales : nullptr, kv_fp8 ? v_scales : nullptr, max_positions, c0, c1, c2, QH, KH, eps};
+  const int N = (QH + 2 * KH) * 64;
+  hipStream_t s = (hipStream_t)stream;
+  // the 64 x 64 tile the plain product would take for the shape, else the ring of four
+  const int tile = default_plan(M, N, K).tile;
+  if (M <= 64) launch_qkv<0>(a_q, w_q, a_scales, w_scales, (int)M, N, K, epi, s);
+  else if (tile == 13) launch_qkv<3>(a_q, w_q, a_scales, w_scales, (int)M, N, K, epi, s);
+  else launch_qkv<4>(a_q, w_q, a_scales, w_scales, (int)M, N, K, epi, s);
+  LFM2_LAUNCH_CHECK();
 }
 
 extern "C" int lfm2_fp8_gemm_partials(float* partials, const uint8_t* a_q, const uint8_t* w_q, int64_t M, int64_t N,

@@ -252,17 +252,30 @@ class LFM25Engine:
             return packed.linear_quantized(x[0], x[1], dtype=self.dtype)
         return packed.linear(x) if packed is not None else ops.linear(x, weight)
 
-    def _backbone(self, tokens, attention_op, conv_op, fp8, *, defer_reduce=False):
+    def _backbone(self, tokens, attention_op, conv_op, fp8, *, defer_reduce=False, projecting_attention_op=None):
         """Embedding and all layers with the fused residual chain of lfm25_cuda.py:134-184: every RMSNorm also adds
         the previous block's output into the running residual.  Returns (last MLP output, residual).  With
-        `defer_reduce` (decode) a split-K down projection hands its partial sums to the next norm."""
+        `defer_reduce` (decode) a split-K down projection hands its partial sums to the next norm.
+        `projecting_attention_op(op, packed, rows_q, row_scales)` (decode), when it takes the layer (returns something),
+        runs the W8A8 QKV projection itself, with the head preparation and the KV append as the product's epilogue."""
         hidden = ops.embedding(tokens, self.weights.embed_tokens)
         residual = None
         for layer in self.weights.layers:
             if layer.attention is not None:
                 op = layer.attention
-                qkv, residual = self._norm_linear(hidden, layer.operator_norm_weight, residual, op.qkv_weight, fp8)
-                mixed = self._linear(attention_op(op, qkv), op.out_weight, fp8)
+                packed = fp8.get(id(op.qkv_weight))
+                attended = None
+                if projecting_attention_op is not None and packed is not None:
+                    rows_q, row_scales, summed = ops.rms_norm_fp8(hidden, layer.operator_norm_weight, self.config.norm_eps, residual)
+                    attended = projecting_attention_op(op, packed, rows_q, row_scales)
+                    if attended is None:   # shape not covered: the plain projection of the rows just quantised
+                        qkv = packed.linear_quantized(rows_q, row_scales, dtype=self.dtype)
+                        attended = attention_op(op, qkv)
+                    residual = summed
+                else:
+                    qkv, residual = self._norm_linear(hidden, layer.operator_norm_weight, residual, op.qkv_weight, fp8)
+                    attended = attention_op(op, qkv)
+                mixed = self._linear(attended, op.out_weight, fp8)
             else:
                 op = layer.conv
                 bcx, residual = self._norm_linear(hidden, layer.operator_norm_weight, residual, op.in_weight, fp8)
@@ -324,7 +337,24 @@ class LFM25Engine:
                 return ops.conv_update_fp8(bcx, op.conv_weight, state, active, slot_ids)
             return ops.conv_update(bcx, op.conv_weight, state, active, slot_ids)
 
-        hidden, residual = self._backbone(tokens, attention_op, conv_op, fp8, defer_reduce=True)
+        def projecting_attention_op(op, packed, rows_q, row_scales):
+            i = op.cache_index
+            if not ops.qkv_project_store_supported(packed, cfg.head_dim, self.dtype, cache.k_cache[i]):
+                return None
+            k_scales = cache.k_scales[i] if cache.fp8 else None
+            v_scales = cache.v_scales[i] if cache.fp8 else None
+            q = ops.qkv_project_store(rows_q, row_scales, packed, op.q_norm_weight, op.k_norm_weight, self._rope_cos,
+                                      self._rope_sin, positions, cfg.num_attention_heads, cfg.num_key_value_heads,
+                                      cfg.head_dim, cfg.norm_eps, cache.k_cache[i], cache.v_cache[i], k_scales, v_scales,
+                                      active=active, slot_ids=slot_ids)
+            quantized = (id(op.out_weight) in fp8
+                         and -(-cfg.num_attention_heads // 16) * -(-cfg.head_dim // 64) <= 4)
+            out = ops.attend(q, cache.k_cache[i], cache.v_cache[i], k_scales, v_scales, positions, active=active,
+                             scale=self._scaling, slot_ids=slot_ids, schedule=schedule, quantized=quantized)
+            return out if quantized else out.view(rows, -1)
+
+        hidden, residual = self._backbone(tokens, attention_op, conv_op, fp8, defer_reduce=True,
+                                          projecting_attention_op=projecting_attention_op)
         place = None if logits_out is None else ops.RowPlacement(logits_out, slot_ids, active)
         logits = self._head(hidden, residual, fp8, place)
         ops.advance_positions(cache.seq_lens, positions, slot_ids, active)

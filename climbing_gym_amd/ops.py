@@ -188,6 +188,32 @@ def prepare_qkv_store(x, q_weight, k_weight, cos, sin, positions, q_heads: int, 
     return q
 
 
+def qkv_project_store_supported(packed, head_dim: int, dtype, k_cache) -> bool:
+    """Whether `qkv_project_store` covers the shape: an e4m3 weight, head_dim 64, bf16, K a multiple of 128 and cache
+    strides that keep a head's 16-byte pieces aligned."""
+    return (packed is not None and head_dim == 64 and dtype == torch.bfloat16 and packed.values.size(1) % 128 == 0
+            and all(stride % 16 == 0 for stride in _cache_strides(k_cache)))
+
+
+def qkv_project_store(xq, x_scales, packed, q_weight, k_weight, cos, sin, positions, q_heads: int, kv_heads: int,
+                      head_dim: int, eps: float, k_cache, v_cache, k_scales=None, v_scales=None, *, active=None, slot_ids=None):
+    """The W8A8 QKV projection (`PackedFP8Weight.linear_quantized`, lfm25_fp8.py:141-168) with `prepare_qkv_store` as
+    its epilogue: quantised rows in, q [M,1,QH,D] out, keys and values appended to the cache.  Same bytes as the two
+    calls."""
+    _check(xq, x_scales, q_weight, k_weight, cos, sin, positions, active, slot_ids)
+    if positions.dtype != torch.int32:
+        raise ValueError("positions must be int32")
+    m, width = xq.shape
+    if packed.values.shape != ((q_heads + 2 * kv_heads) * head_dim, width):
+        raise ValueError("QKV weight does not match the activation width and head counts")
+    q = torch.empty((m, 1, q_heads, head_dim), device=xq.device, dtype=q_weight.dtype)
+    c0, c1, c2 = _cache_strides(k_cache)
+    call("lfm2_fp8_gemm_qkv_store", q, xq, x_scales, packed.values, packed.scales, q_weight, k_weight, cos, sin, positions,
+         k_cache, v_cache, k_scales, v_scales, active, slot_ids, m, q_heads, kv_heads, head_dim, width, cos.size(0),
+         float(eps), c0, c1, c2, int(k_scales is not None), _code(q_weight.dtype))
+    return q
+
+
 def prepare_qkv(x, q_weight, k_weight, cos, sin, positions, q_heads: int, kv_heads: int, head_dim: int, eps: float):
     """lfm25_cuda_kernels.py:143-151: QK RMSNorm + rotate-half RoPE + split; q/k/v come back as [M,1,heads,D]."""
     _check(x, q_weight, k_weight, cos, sin, positions)

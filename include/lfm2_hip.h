@@ -114,6 +114,17 @@ int lfm2_conv_prefill(void* out, void* state, const void* bcx, const void* weigh
 int lfm2_fp8_gemm(void* out, const uint8_t* a_q, const float* a_scales, const uint8_t* w_q,
                   const float* w_scales, float* workspace, int64_t M, int64_t N, int64_t K, int out_dtype,
                   int tile, int split_k, void* stream);
+/* The QKV projection of an attention layer at decode with lfm2_prepare_qkv_store as its epilogue (head_dim 64, bf16,
+ * K a multiple of 128): x_q[M,K] . w_q[(QH+2KH)*64, K]^T scaled and rounded to bf16 as lfm2_fp8_gemm stores it, then
+ * per head QK-norm + RoPE, q [M,QH,64] written, keys and values appended to the cache at positions[m] (e4m3 with one
+ * scale per token and head when kv_fp8, else the model dtype).  Bit for bit the two launches it replaces
+ * (lfm25_fp8.py:141-168 then lfm25_cuda_kernels.py:113-151 and lfm25_fp8_kv.py:58-69 / lfm25_batching.py:49-69). */
+int lfm2_fp8_gemm_qkv_store(void* q, const uint8_t* a_q, const float* a_scales, const uint8_t* w_q, const float* w_scales,
+                            const void* q_weight, const void* k_weight, const float* cos, const float* sin,
+                            const int32_t* positions, void* k_cache, void* v_cache, float* k_scales, float* v_scales,
+                            const uint8_t* active, const int32_t* slot_ids, int64_t M, int QH, int KH, int D, int64_t K,
+                            int64_t max_positions, float eps, int64_t c0, int64_t c1, int64_t c2, int kv_fp8, int dtype,
+                            void* stream);
 /* The same product left as split-K partial sums: partials float[split_k, M, N], unscaled (no activation or weight
  * scale applied), split s covering its contiguous share of K.  For a consumer that folds the reduction into its own
  * pass (lfm2_rms_norm_fp8_split).  No counterpart in the reference, which always materialises the projection. */

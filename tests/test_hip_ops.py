@@ -740,6 +740,50 @@ def test_prepare_qkv_with_cache_append_equals_the_two_separate_launches(ops, dim
         assert torch.equal(ks0, ks1) and torch.equal(vs0, vs1)
 
 
+@pytest.mark.parametrize("rows", [5, 64, 256, 300])      # register-staged tile, one ring tile, the decode batch, a ragged last tile
+@pytest.mark.parametrize("fp8", [True, False])
+@torch.inference_mode()
+def test_qkv_projection_with_prepare_and_append_as_its_epilogue_equals_the_two_launches(ops, rows, fp8):
+    """The W8A8 QKV projection whose epilogue does QK norm + RoPE + KV append, against linear_quantized followed by
+    prepare_qkv_store (pinned above): q, cache bytes and scales identical, untouched cache rows untouched."""
+    torch.manual_seed(7)
+    qh, kh, dim, hidden, slots, cap = 32, 8, 64, 2048, 320, 24
+    act = torch.randn(rows, hidden, dtype=torch.bfloat16, device=DEV)
+    packed = ops.PackedFP8Weight.from_weight(torch.randn((qh + 2 * kh) * dim, hidden, dtype=torch.bfloat16, device=DEV) * 0.03)
+    xq, xs = ops.quantize_rows(act)
+    qw, kw = (torch.randn(dim, dtype=torch.bfloat16, device=DEV) for _ in range(2))
+    cos, sin = (t.to(DEV) for t in O.rope_tables(dim, 1e6, 64))
+    positions = torch.randint(0, cap, (rows,), dtype=torch.int32, device=DEV)
+    slot_ids = torch.randperm(slots, device=DEV)[:rows].to(torch.int32)
+    slot_ids[1] = -1
+    active = torch.rand(rows, device=DEV) > 0.2
+    assert ops.qkv_project_store_supported(packed, dim, torch.bfloat16, torch.empty(slots, cap, kh, dim, device=DEV))
+
+    def caches():
+        torch.manual_seed(8)
+        if fp8:
+            kc = torch.randint(0, 255, (slots, kh, cap, dim), dtype=torch.uint8, device=DEV).view(torch.float8_e4m3fn)
+            vc = torch.randint(0, 255, (slots, kh, cap, dim), dtype=torch.uint8, device=DEV).view(torch.float8_e4m3fn)
+            ks, vs = (torch.rand(slots, kh, cap, device=DEV) for _ in range(2))
+            return kc.transpose(1, 2), vc.transpose(1, 2), ks.transpose(1, 2), vs.transpose(1, 2)
+        kc, vc = (torch.randn(slots, kh, cap, dim, dtype=torch.bfloat16, device=DEV).transpose(1, 2) for _ in range(2))
+        return kc, vc, None, None
+
+    kc0, vc0, ks0, vs0 = caches()
+    qkv = packed.linear_quantized(xq, xs)
+    q0 = ops.prepare_qkv_store(qkv, qw, kw, cos, sin, positions, qh, kh, dim, 1e-5, kc0, vc0, ks0, vs0, active=active,
+                               slot_ids=slot_ids)
+    kc1, vc1, ks1, vs1 = caches()
+    q1 = ops.qkv_project_store(xq, xs, packed, qw, kw, cos, sin, positions, qh, kh, dim, 1e-5, kc1, vc1, ks1, vs1,
+                               active=active, slot_ids=slot_ids)
+    torch.cuda.synchronize()
+    assert torch.equal(q0, q1)
+    as_bytes = (lambda t: t.contiguous().view(torch.uint8)) if fp8 else (lambda t: t.contiguous().view(torch.int16))
+    assert torch.equal(as_bytes(kc0), as_bytes(kc1)) and torch.equal(as_bytes(vc0), as_bytes(vc1))
+    if fp8:
+        assert torch.equal(ks0, ks1) and torch.equal(vs0, vs1)
+
+
 @pytest.mark.parametrize("width", (256, 2048, 4096))
 @torch.inference_mode()
 def test_conv_update_with_quantised_output_equals_the_two_separate_launches(ops, width):
