@@ -94,11 +94,13 @@ struct QkvEpilogue {
   float eps;
 };
 
-template <int EB, int BM, int BN, int WM, int WN, int SW, int KS, bool KTAIL, int ST = 0, int EPI = 0>
-__global__ void __launch_bounds__(WM * WN * 64)
-gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_t* __restrict__ A,
-               const uint8_t* __restrict__ W, const float* __restrict__ a_scales, const float* __restrict__ w_scales,
-               int M, int N, int64_t Kb, int steps_per_split, int out_dtype, RowMap rows, QkvEpilogue epi) {
+// The kernel body; the two entry points below differ in their arguments only (the fused QKV projection carries its
+// epilogue's arguments, the plain products do not pay for them in every launch's argument block).
+template <int EB, int BM, int BN, int WM, int WN, int SW, int KS, bool KTAIL, int ST, int EPI>
+__device__ __forceinline__ void
+gemm_nt_body(void* __restrict__ out, float* __restrict__ partial, const uint8_t* __restrict__ A,
+             const uint8_t* __restrict__ W, const float* __restrict__ a_scales, const float* __restrict__ w_scales,
+             int M, int N, int64_t Kb, int steps_per_split, int out_dtype, const RowMap& rows, const QkvEpilogue& epi) {
   constexpr int NT = WM * WN * 64;
   constexpr int TM = BM / WM, TN = BN / WN, MI = TM / 16, NI = TN / 16;
   constexpr int kChunksPerRow = KS / 16;  // KS = K bytes staged per step and row: 128, or 256 (two MFMA sub-steps per barrier)
@@ -431,6 +433,23 @@ gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_
   }
 }
 
+template <int EB, int BM, int BN, int WM, int WN, int SW, int KS, bool KTAIL, int ST = 0>
+__global__ void __launch_bounds__(WM * WN * 64)
+gemm_nt_kernel(void* __restrict__ out, float* __restrict__ partial, const uint8_t* __restrict__ A,
+               const uint8_t* __restrict__ W, const float* __restrict__ a_scales, const float* __restrict__ w_scales,
+               int M, int N, int64_t Kb, int steps_per_split, int out_dtype, RowMap rows) {
+  gemm_nt_body<EB, BM, BN, WM, WN, SW, KS, KTAIL, ST, 0>(out, partial, A, W, a_scales, w_scales, M, N, Kb, steps_per_split,
+                                                         out_dtype, rows, QkvEpilogue{});
+}
+
+template <int ST>
+__global__ void __launch_bounds__(256)
+gemm_qkv_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ W, const float* __restrict__ a_scales,
+                const float* __restrict__ w_scales, int M, int N, int64_t Kb, QkvEpilogue epi) {
+  gemm_nt_body<1, 64, 64, 2, 2, 1, 128, false, ST, 1>(nullptr, nullptr, A, W, a_scales, w_scales, M, N, Kb, (int)(Kb / 128),
+                                                      LFM2_DTYPE_BF16, RowMap{nullptr, nullptr, 0x7fffffff}, epi);
+}
+
 // Sum split-K partials in split order, then scale (row scale, then column scale).  A separate launch on purpose:
 // the eight XCDs have private L2s, so partials written by workgroups on other XCDs are only visible to a reader
 // cheaply at a kernel boundary; an in-kernel "last workgroup reduces" scheme needs device-scope fences that write
@@ -519,10 +538,10 @@ void launch_tile(void* out, float* partial, const uint8_t* A, const uint8_t* W, 
   const dim3 grid((tiles + 7) / 8 * 8, splits), block(WM * WN * 64);
   if (Kb % KS == 0)
     hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN, SW, KS, false, ST>), grid, block, 0, s, out, (splits > 1 || keep_partials) ? partial : nullptr, A, W,
-                       as, ws, M, N, Kb, per, out_dtype, rows, QkvEpilogue{});
+                       as, ws, M, N, Kb, per, out_dtype, rows);
   else
     hipLaunchKernelGGL((gemm_nt_kernel<EB, BM, BN, WM, WN, SW, KS, true>), grid, block, 0, s, out, (splits > 1 || keep_partials) ? partial : nullptr, A, W,
-                       as, ws, M, N, Kb, per, out_dtype, rows, QkvEpilogue{});
+                       as, ws, M, N, Kb, per, out_dtype, rows);
 }
 
 // The fused QKV projection on one of the 64 x 64 tiles (ring of ST buffers, or register staged with ST = 0).
@@ -531,8 +550,7 @@ void launch_qkv(const uint8_t* A, const uint8_t* W, const float* as, const float
                 const QkvEpilogue& epi, hipStream_t s) {
   const int tiles = ((M + 63) / 64) * (N / 64);
   const dim3 grid((tiles + 7) / 8 * 8, 1), block(256);
-  hipLaunchKernelGGL((gemm_nt_kernel<1, 64, 64, 2, 2, 1, 128, false, ST, 1>), grid, block, 0, s, nullptr, nullptr, A, W, as, ws, M,
-                     N, Kb, (int)(Kb / 128), LFM2_DTYPE_BF16, RowMap{nullptr, nullptr, 0x7fffffff}, epi);
+  hipLaunchKernelGGL(gemm_qkv_kernel<ST>, grid, block, 0, s, A, W, as, ws, M, N, Kb, epi);
 }
 
 template <int EB>
