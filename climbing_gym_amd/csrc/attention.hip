@@ -89,7 +89,8 @@ constexpr int kChunk = 512;        // history tokens per workgroup
 constexpr int kWaveTok = kChunk / 4;
 constexpr int kGB = 4;             // query heads per workgroup (one GQA group, padded)
 
-// Schedule layout (int32): [0] number of (row, chunk) pairs; from kSchedRows on one 16-byte record per row (index of
+// Schedule layout (int32): [0] number of (row, chunk) pairs; [1] tokens per chunk (the kernel that builds the list
+// picks 256 or 512 from the rows' lengths); from kSchedRows on one 16-byte record per row (index of
 // the pair of its first full chunk, index of the pair of its partial chunk, its length or 0 when it sits out, 0);
 // then one 16-byte record per pair (row, chunk, length, slot).
 constexpr int kSchedRows = 4;
@@ -108,14 +109,15 @@ struct DecodeArgs {
 
 // Row of the partial-result arrays that holds chunk c of (row b, query head qh).  The generic kernel's rows are dense,
 // [b][qh][chunk]; the scheduled kernel's are [pair][qh], so that one item's heads are one contiguous block.
-struct RowPairs { int full_first, partial, nfull, len; };
+struct RowPairs { int full_first, partial, nfull, len, chunk; };
 // The row's length (0: inactive, padding or empty) and, for the scheduled kernel, where its partial results are:
 // one load of the row's record there, the rows' own arrays otherwise.
 __device__ __forceinline__ RowPairs row_pairs(const DecodeArgs& a, int b) {
-  RowPairs r{0, 0, 0, 0};
+  RowPairs r{0, 0, 0, 0, a.chunk};
   if (a.schedule) {
     const i32x4 rec = *reinterpret_cast<const i32x4*>(a.schedule + kSchedRows + 4 * b);
-    r.full_first = rec[0]; r.partial = rec[1]; r.len = rec[2]; r.nfull = rec[2] / a.chunk;
+    r.chunk = a.schedule[1];
+    r.full_first = rec[0]; r.partial = rec[1]; r.len = rec[2]; r.nfull = rec[2] / r.chunk;
     return r;
   }
   r.len = a.positions[b] + 1;
@@ -292,7 +294,9 @@ __global__ void __launch_bounds__(256) decode_attn_kernel(DecodeArgs a) {
 //               are added once per wave.
 //
 // e4m3 -> bf16 conversion is v_cvt_scalef32_pk_bf16_fp8 (two values per instruction, scale 1).
-constexpr int kMfmaChunk = 256;  // history tokens per item (one wave)
+constexpr int kMfmaChunk = 256;      // history tokens per item (one wave) ...
+constexpr int kMfmaLongChunk = 512;  // ... or this many, when the batch holds at least kLongPairs items of the short kind:
+constexpr int kLongPairs = 3072;     // with enough items for every wave, longer ones halve the partial results and their merge
 constexpr float kMaxSlack = 8.0f;  // log2 units
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -440,8 +444,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
     b = rec[0]; chunk = rec[1]; len = rec[2]; slot = rec[3]; h = idx % a.KH;
   }
   i32x4 rec_next = read_record(idx_next);
-  int wbeg = chunk * kMfmaChunk;
-  int wend = wbeg + kMfmaChunk;
+  const int chunk_tokens = a.schedule[1];
+  int wbeg = chunk * chunk_tokens;
+  int wend = wbeg + chunk_tokens;
   wend = wend < len ? wend : len;
   Tile tile, ahead;
   fetch(b, slot, h, wbeg, wend, tile);
@@ -467,8 +472,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
     const bool have_next = last && idx_next < items;
     if (have_next) {
       nb = rec_next[0]; nlen = rec_next[2]; nslot = rec_next[3]; nh = idx_next % a.KH;
-      nwbeg = rec_next[1] * kMfmaChunk;
-      nwend = nwbeg + kMfmaChunk;
+      nwbeg = rec_next[1] * chunk_tokens;
+      nwend = nwbeg + chunk_tokens;
       nwend = nwend < nlen ? nwend : nlen;
     }
     const int fT = last ? (have_next ? nwbeg : T) : T + TT;
@@ -599,20 +604,30 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
 // items round robin, so the r-th items of all waves are (nearly) equally long and every wave gets the same work.
 // One counting sweep over the rows gives the classes' sizes, a second one places the rows: in each, a thread's rank
 // within its class comes from a wave scan and the waves' totals.
-constexpr int kSchedClasses = 5;   // full chunks, then partial chunks of 4, 3, 2, 1 tiles (chunk = 256)
+constexpr int kSchedClasses = 9;   // full chunks, then partial chunks of 8 (512-token chunks only), 7, ... 1 tiles
 __global__ void __launch_bounds__(1024)
-decode_schedule_kernel(int32_t* schedule, const int32_t* positions, const uint8_t* active, const int32_t* slot_ids, int B,
-                       int chunk) {
+decode_schedule_kernel(int32_t* schedule, const int32_t* positions, const uint8_t* active, const int32_t* slot_ids, int B) {
   __shared__ int wave_total[kSchedClasses][16];
   __shared__ int class_base[kSchedClasses + 1];   // where each class starts; running, during the second sweep
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int pairs_at = kSchedRows + 4 * B;
-  const int tiles_per_chunk = chunk / 64;
   auto row_length = [&](int b) {
     int len = 0;
     if (b < B && (!active || active[b]) && (!slot_ids || slot_ids[b] >= 0)) len = positions[b] + 1;
     return len > 0 ? len : 0;
   };
+  // sweep 0: the chunk size, from the number of items the rows would make at the short one
+  int short_items = 0;
+  for (int base = 0; base < B; base += 1024) short_items += (row_length(base + threadIdx.x) + kMfmaChunk - 1) / kMfmaChunk;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) short_items += __shfl_xor(short_items, o, 64);
+  if (lane == 0) wave_total[0][wave] = short_items;
+  __syncthreads();
+  short_items = 0;
+  for (int w = 0; w < 16; ++w) short_items += wave_total[0][w];
+  __syncthreads();
+  const int chunk = short_items >= kLongPairs ? kMfmaLongChunk : kMfmaChunk;
+  const int tiles_per_chunk = chunk / 64;
   auto classify = [&](int len, int* n) {   // how many items of each class the row contributes
 #pragma unroll
     for (int k = 0; k < kSchedClasses; ++k) n[k] = 0;
@@ -625,7 +640,7 @@ decode_schedule_kernel(int32_t* schedule, const int32_t* positions, const uint8_
     }
   };
   // sweep 1: class sizes
-  int mine[kSchedClasses] = {0, 0, 0, 0, 0};
+  int mine[kSchedClasses] = {};
   for (int base = 0; base < B; base += 1024) {
     int n[kSchedClasses];
     classify(row_length(base + threadIdx.x), n);
@@ -648,6 +663,7 @@ decode_schedule_kernel(int32_t* schedule, const int32_t* positions, const uint8_
     }
     class_base[kSchedClasses] = at;
     schedule[0] = at;
+    schedule[1] = chunk;
   }
   __syncthreads();
   // sweep 2: places
@@ -713,7 +729,7 @@ __global__ void __launch_bounds__(64) decode_combine_kernel(DecodeArgs a) {
     for (int d = threadIdx.x; d < a.D; d += 64) out[d] = Elem<T>::store(0.f);
     return;
   }
-  const int n = (len + a.chunk - 1) / a.chunk;
+  const int n = (len + rp.chunk - 1) / rp.chunk;
   auto prow = [&](int c) { return partial_row(a, rp, b, qh, c); };
   float mm = -1.0e30f;
   for (int c = 0; c < n; ++c) mm = fmaxf(mm, a.ws_m[prow(c)]);
@@ -743,7 +759,7 @@ __global__ void __launch_bounds__(1024) decode_combine_row_kernel(DecodeArgs a, 
   const int b = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const RowPairs rp = row_pairs(a, b);
   const int len = rp.len;
-  const int n = len > 0 ? (len + a.chunk - 1) / a.chunk : 0;
+  const int n = len > 0 ? (len + rp.chunk - 1) / rp.chunk : 0;
   const int per_head = (a.D + 63) / 64;
   auto head_of = [&](int i) { return wave + kWavesPerRow * (i / per_head); };
   auto dim_of = [&](int i) { return lane + 64 * (i % per_head); };
@@ -1099,7 +1115,7 @@ extern "C" int lfm2_decode_schedule(int32_t* schedule, const int32_t* positions,
                                     const int32_t* slot_ids, int64_t B, void* stream) {
   LFM2_REQUIRE(B > 0 && schedule && positions, "decode_schedule: bad arguments");
   hipLaunchKernelGGL(decode_schedule_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, schedule, positions, active,
-                     slot_ids, (int)B, kMfmaChunk);
+                     slot_ids, (int)B);
   LFM2_LAUNCH_CHECK();
 }
 
@@ -1144,7 +1160,7 @@ extern "C" int lfm2_decode_attention(void* out, const void* q, const void* k_cac
   if (mfma) {
     if (schedule == nullptr) {  // no shared schedule from the caller: build one in the tail of the workspace
       int32_t* own = reinterpret_cast<int32_t*>(workspace + B * QH * ((capacity + kMinChunk - 1) / kMinChunk) * (D + 2));
-      hipLaunchKernelGGL(decode_schedule_kernel, dim3(1), dim3(1024), 0, s, own, positions, active, slot_ids, (int)B, kMfmaChunk);
+      hipLaunchKernelGGL(decode_schedule_kernel, dim3(1), dim3(1024), 0, s, own, positions, active, slot_ids, (int)B);
       schedule = own;
     }
     a.schedule = schedule;

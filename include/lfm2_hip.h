@@ -198,8 +198,8 @@ int lfm2_decode_attention(void* out, const void* q, const void* k_cache, const v
                           void* stream);
 int64_t lfm2_decode_attention_workspace(int64_t B, int QH, int D, int64_t capacity);
 
-/* Work list of the persistent decode-attention kernel: one (row, 256-token chunk) item per chunk of every active
- * row's history, longest first (used for e4m3 and bf16 histories of head_dim 64 with GQA groups of at most 4 and
+/* Work list of the persistent decode-attention kernel: one (row, chunk) item per chunk of every active row's history
+ * (chunks of 256 tokens, or of 512 when the batch would make at least 3072 chunks of 256), longest first (used for e4m3 and bf16 histories of head_dim 64 with GQA groups of at most 4 and
  * bf16 queries; other shapes ignore it).  It depends only on positions/active/slot_ids, so the attention layers of one
  * decode step can share it (pass it as `schedule`; NULL makes lfm2_decode_attention build its own in the workspace).
  * schedule: int32[lfm2_decode_schedule_size(B, capacity)].  No counterpart in the reference, whose Triton grid is

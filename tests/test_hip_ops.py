@@ -351,21 +351,25 @@ def test_decode_matches_independent_fp32_softmax_with_ragged_lengths_and_inactiv
     assert torch.count_nonzero(moved[3]) == 0
 
 
+@pytest.mark.parametrize("rows,longest", [(1500, 3000), (300, 1200)])
 @torch.inference_mode()
-def test_work_list_lists_every_chunk_once_longest_first(ops):
-    """Layout of the decode-attention work list: pair count; a record per row (first full pair, partial pair,
-    length or 0 for rows that sit out); a record per pair (row, chunk, length, slot), full 256-token chunks first,
-    then partial chunks of 4, 3, 2, 1 tiles.  1500 rows: more than one block of the device scan."""
+def test_work_list_lists_every_chunk_once_longest_first(ops, rows, longest):
+    """Layout of the decode-attention work list: pair count and chunk size (512 tokens when the rows would make at
+    least 3072 chunks of 256, else 256); a record per row (first full pair, partial pair, length or 0 for rows that
+    sit out); a record per pair (row, chunk, length, slot), full chunks first, then partial chunks by decreasing
+    number of 64-token tiles.  1500 rows: more than one block of the device scan."""
     torch.manual_seed(3)
-    rows, chunk = 1500, 256
-    lengths = torch.randint(1, 3000, (rows,))
-    lengths[:8] = torch.tensor([1, 64, 65, 256, 257, 512, 2999, 255])
+    lengths = torch.randint(1, longest, (rows,))
+    lengths[:8] = torch.tensor([1, 64, 65, 256, 257, 512, longest - 1, 255])
     active = torch.rand(rows) > 0.1
     slots = torch.randperm(rows).to(torch.int32)
     slots[torch.rand(rows) < 0.05] = -1
     schedule = ops.decode_schedule((lengths - 1).to(torch.int32).to(DEV), active.to(DEV), slots.to(DEV), capacity=3072).cpu()
     live = active & (slots >= 0)
     eff = torch.where(live, lengths, torch.zeros_like(lengths))
+    short_pairs = int((eff + 255).div(256, rounding_mode="floor").sum())
+    chunk = 512 if short_pairs >= 3072 else 256
+    assert int(schedule[1]) == chunk and chunk == (512 if rows == 1500 else 256)
     pairs = int((eff + chunk - 1).div(chunk, rounding_mode="floor").sum())
     assert int(schedule[0]) == pairs
     row_rec = schedule[4:4 + 4 * rows].view(rows, 4)
