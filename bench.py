@@ -11,6 +11,7 @@ baseline (the oracle's fp32 restatement of the reference CPU engine on a bounded
 from __future__ import annotations
 
 import argparse
+import itertools
 import json
 import os
 import sys
@@ -43,10 +44,128 @@ def parse_args():
     p.add_argument("--attn-samples", type=int, default=20, help="timed launches of the decode-attention kernel per layer")
     p.add_argument("--top-k", type=int, default=0, help="top-k filter of the sampler (0: full support)")
     p.add_argument("--top-p", type=float, default=1.0, help="top-p filter of the sampler (1: off)")
-    p.add_argument("--workload", choices=("decode", "attention"), default="decode",
+    p.add_argument("--workload", choices=("decode", "attention", "gemm", "prefill"), default="decode",
                    help="decode: the model's decode step (the headline metric); attention: the decode-attention call alone "
-                        "on 256 sequences of U[128, 8192] history tokens, dense and paged (block 16), e4m3 and bf16")
+                        "on 256 sequences of U[128, 8192] history tokens, dense and paged (block 16), e4m3 and bf16; "
+                        "gemm: the W8A8 projection shapes at 1..4096 rows; prefill: causal varlen attention over a packed "
+                        "4096-token chunk")
     return p.parse_args()
+
+
+def gemm_workload(args):
+    """The W8A8 product `y = (xq * xs) (Wq * ws)^T` on the model's five projection shapes at 1 to 4096 rows:
+    activations N(0,1) with 1 % of the entries scaled by 20 and quantised per token, weights N(0, 0.02) quantised per
+    output channel, bf16 out.  Each shape cycles through enough weight copies (>= 1 GiB) that they stream from HBM.
+    Every product is checked against the fp32 matmul of the dequantised operands (1e-2 relative, Frobenius)."""
+    from climbing_gym_amd import ops
+    shapes = {"w13": (11264, 2048), "conv_in": (6144, 2048), "qkv": (3072, 2048), "out": (2048, 2048), "w2": (2048, 5632)}
+    rows_list = (1, 8, 64, 256, 1024, 4096)
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    stream = torch.cuda.current_stream()
+    table, worst = {}, 0.0
+    for name, (n, k) in shapes.items():
+        copies = -(-(1 << 30) // (n * k))
+        packs = [ops.PackedFP8Weight.from_weight((torch.randn(n, k, device="cuda", generator=gen) * 0.02).bfloat16())
+                 for _ in range(copies)]
+        for m in rows_list:
+            x = torch.randn(m, k, device="cuda", generator=gen)
+            x = torch.where(torch.rand(m, k, device="cuda", generator=gen) < 0.01, x * 20, x).bfloat16()
+            xq, xs = ops.quantize_rows(x)
+            got = packs[0].linear_quantized(xq, xs).float()
+            want = (xq.float() * xs[:, None]) @ (packs[0].values.float() * packs[0].scales[:, None]).t()
+            err = float((got - want).norm() / want.norm())
+            worst = max(worst, err)
+            if not err < 1e-2:
+                raise SystemExit(f"W8A8 product differs from the dequantised matmul: {name} rows {m}: {err:.3e}")
+            repeats = max(1, 64 // copies)
+            def body():
+                for _ in range(repeats):
+                    for p in packs:
+                        p.linear_quantized(xq, xs)
+            body()
+            torch.cuda.synchronize()
+            side, graph = torch.cuda.Stream(), torch.cuda.CUDAGraph()
+            with torch.cuda.stream(side), torch.cuda.graph(graph, stream=side):
+                body()
+            torch.cuda.synchronize()
+            graph.replay()
+            begin.record(stream)
+            for _ in range(args.steps):
+                graph.replay()
+            end.record(stream)
+            end.synchronize()
+            sec = begin.elapsed_time(end) / 1000 / (args.steps * repeats * copies)
+            moved = n * k + 4 * n + m * k + 4 * m + 2 * m * n
+            table[f"{name} n{n} k{k} m{m}"] = {"us": round(sec * 1e6, 2), "GBps": round(moved / sec / 1e9, 1),
+                                               "TFLOPs": round(2 * m * n * k / sec / 1e12, 1)}
+            del graph
+        del packs
+        torch.cuda.empty_cache()
+    big, small = table["w13 n11264 k2048 m4096"], table["w13 n11264 k2048 m256"]
+    print(json.dumps({
+        "metric": "W8A8 FP8 GEMM, gate+up projection (N 11264, K 2048) at 4096 rows", "value": big["TFLOPs"],
+        "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": 1, "ms_per_step": round(big["us"] / 1000, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3 (fp32 accumulate, bf16 out)",
+        "data": "synthetic",
+        "config": {"workload": "W8A8 products of the LFM2.5-1.2B projection shapes at 1, 8, 64, 256, 1024 and 4096 rows, "
+                               "per-token and per-channel scales, weights streamed from HBM",
+                   "worst_relative_error": round(worst, 6), "shapes": table},
+        "roofline": {"kernel": "gemm_nt_kernel (128x128 ring tile) at 4096 rows", "bound": "mfma", "achieved": big["TFLOPs"],
+                     "peak": 5000.0, "unit": "TFLOP/s", "frac": round(big["TFLOPs"] / 5000.0, 4), "traffic": None,
+                     "decode_rows_256": {"bound": "hbm", "achieved": small["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                         "frac": round(small["GBps"] / HBM_PEAK_GBS, 4)}},
+        "cpu_baseline": None}))
+
+
+def prefill_workload(args):
+    """Causal GQA attention over one packed prefill chunk: sequences of U[64, 2048] tokens drawn until they fill 4096
+    tokens (the last one cut), 32 query heads over 8 KV heads of 64 dims, bf16.  Checked per sequence against fp32
+    softmax attention (2e-2 absolute on N(0,1) inputs)."""
+    from climbing_gym_amd import ops
+    heads, kv_heads, dim, budget = 32, 8, 64, 4096
+    gen = torch.Generator().manual_seed(0)
+    lengths = []
+    while sum(lengths) < budget:
+        lengths.append(min(int(torch.randint(64, 2049, (1,), generator=gen)), budget - sum(lengths)))
+    cu = torch.tensor([0] + list(itertools.accumulate(lengths)), dtype=torch.int32, device="cuda")
+    torch.manual_seed(0)
+    q = torch.randn(budget, heads, dim, device="cuda", dtype=torch.bfloat16)
+    k = torch.randn(budget, kv_heads, dim, device="cuda", dtype=torch.bfloat16)
+    v = torch.randn(budget, kv_heads, dim, device="cuda", dtype=torch.bfloat16)
+    call = lambda: ops.prefill_attention(q, k, v, cu, max(lengths))
+    out = call().float()
+    worst = 0.0
+    for first, n in zip(cu.tolist(), lengths):
+        qs = q[first:first + n].float().transpose(0, 1)
+        ks = k[first:first + n].float().transpose(0, 1).repeat_interleave(heads // kv_heads, 0)
+        vs = v[first:first + n].float().transpose(0, 1).repeat_interleave(heads // kv_heads, 0)
+        want = torch.nn.functional.scaled_dot_product_attention(qs, ks, vs, is_causal=True).transpose(0, 1)
+        worst = max(worst, float((out[first:first + n] - want).abs().max()))
+    if not worst < 2e-2:
+        raise SystemExit(f"varlen prefill attention differs from fp32 softmax attention: {worst:.3e}")
+    for _ in range(max(args.warmup, 1)):
+        call()
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    stream = torch.cuda.current_stream()
+    begin.record(stream)
+    for _ in range(args.steps):
+        call()
+    end.record(stream)
+    end.synchronize()
+    sec = begin.elapsed_time(end) / 1000 / args.steps
+    flops = sum(4 * heads * dim * n * (n + 1) // 2 for n in lengths)   # QK^T and PV over the causal triangle
+    moved = (2 * budget * heads * dim + 2 * budget * kv_heads * dim) * 2
+    print(json.dumps({
+        "metric": "causal varlen prefill attention, 4096 packed tokens", "value": round(budget / sec, 1), "unit": "tok/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec * 1000, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 (fp32 softmax and accumulate)",
+        "data": "synthetic",
+        "config": {"workload": f"one packed chunk of {len(lengths)} sequences, lengths {lengths}, 32 query / 8 KV heads x 64",
+                   "worst_abs_error": round(worst, 5), "algorithmic_bytes": moved},
+        "roofline": {"kernel": "prefill_attn_kernel", "bound": "mfma", "achieved": round(flops / sec / 1e12, 1), "peak": 2500.0,
+                     "unit": "TFLOP/s", "frac": round(flops / sec / 1e12 / 2500.0, 4), "traffic": None},
+        "cpu_baseline": None}))
 
 
 def attention_workload(args):
@@ -295,9 +414,9 @@ def main():
         print(f"bench.py measures one MI355X; --gpus {args.gpus} is not supported in this build "
               "(the path shards by slots across independent engines with no collective in the step).", file=sys.stderr)
         sys.exit(2)
-    if args.workload == "attention":
+    if args.workload != "decode":
         with torch.inference_mode():
-            attention_workload(args)
+            {"attention": attention_workload, "gemm": gemm_workload, "prefill": prefill_workload}[args.workload](args)
         return
     from climbing_gym_amd.config import LFM25SamplingConfig
     from climbing_gym_amd.synthetic import LFM2_1P2B, random_prompts, random_state_dict

@@ -510,23 +510,32 @@ struct Plan { int tile, splits; };
 Plan default_plan(int64_t M, int64_t N, int64_t Kb) {
   auto count = [&](int t) { return ((M + kTiles[t].bm - 1) / kTiles[t].bm) * ((N + kTiles[t].bn - 1) / kTiles[t].bn); };
   const int64_t steps = (Kb + kStepBytes - 1) / kStepBytes;
-  int tile;
-  if (M <= 16) tile = 0;
-  else if (M <= 32) tile = 1;
-  else if (M <= 64) tile = 2;
-  else if (steps >= 64 && count(13) <= 256) {
+  // Few output tiles on a K loop of 32 steps or more: split K (2 or 4 ways) while every part keeps 8 steps and the
+  // launch stays within about 256 workgroups.  Weights streamed from HBM, product + reduce launch, 16 rows: e4m3
+  // N 2048 K 5632 7.9 us against 19.6 unsplit; bf16 N 2048 K 2048 6.4 against 14.6, N 6144 8.8 against 9.4,
+  // K 5632 9.6 against 35.  K loops of 16 steps (e4m3, K 2048) gain nothing from a split.
+  auto splits_for = [&](int64_t tiles) {
+    if (steps < 32) return 1;
+    const int64_t most = std::min<int64_t>(std::min<int64_t>(4, steps / 8), 256 / std::max<int64_t>(tiles, 1));
+    return most >= 4 ? 4 : most >= 2 ? 2 : 1;
+  };
+  // up to 64 rows the direct-to-LDS rings win over register staging by 25-40 % once the weights come from HBM
+  // (e4m3 N 3072: 6.2 / 7.2 / 7.1 us at 16 / 32 / 64 rows against 9.2 / 10.9 / 12.9)
+  if (M <= 16) return {18, splits_for(count(18))};            // 16x64, 256-byte steps, ring of 3
+  if (M <= 32) return {17, splits_for(count(17))};            // 32x64, ring of 5
+  if (M <= 64 && count(1) <= 256) return {17, splits_for(count(17))};
+  if (steps >= 64 && count(13) <= 256) {
     // a long K loop on few output tiles (the bf16 down projection at decode: 88 steps on 128 tiles): split K so that
     // about 512 workgroups share it.  M 256, N 2048, 11264 K bytes: 16.5 us against 24.3 (bf16), 21.1 against 22.4
     // (e4m3); M 128: 13.0 against 24.5
     const int splits = (int)(512 / count(13));
     return {13, splits > 4 ? 4 : splits};
   }
-  else if (count(6) >= 256) tile = 14;               // 128x128, ring of 2
-  else if (count(2) >= 512) tile = 13;               // 64x64, ring of 3
-  else if (count(1) > 384) tile = 15;                // 32x64, 256-byte steps, ring of 2
-  else if (count(1) > 256) tile = 16;                // 64x64, ring of 4
-  else tile = steps >= 32 ? 17 : 12;                 // 32x64, ring of 5 (long K) or 4
-  return {tile, 1};
+  if (count(6) >= 256) return {14, 1};                // 128x128, ring of 2
+  if (count(2) >= 512) return {13, 1};                // 64x64, ring of 3
+  if (count(1) > 384) return {15, 1};                 // 32x64, 256-byte steps, ring of 2
+  if (count(1) > 256) return {16, 1};                 // 64x64, ring of 4
+  return {steps >= 32 ? 17 : 12, splits_for(count(1))};   // 32x64, ring of 5 (long K) or 4
 }
 
 template <int EB, int BM, int BN, int WM, int WN, int SW, int KS, int ST = 0>
@@ -544,7 +553,7 @@ void launch_tile(void* out, float* partial, const uint8_t* A, const uint8_t* W, 
                        as, ws, M, N, Kb, per, out_dtype, rows);
 }
 
-// The fused QKV projection on one of the 64 x 64 tiles (ring of ST buffers, or register staged with ST = 0).
+// The fused QKV projection on one of the 64 x 64 ring tiles (ST buffers).
 template <int ST>
 void launch_qkv(const uint8_t* A, const uint8_t* W, const float* as, const float* ws, int M, int N, int64_t Kb,
                 const QkvEpilogue& epi, hipStream_t s) {
@@ -649,8 +658,7 @@ extern "C" int lfm2_fp8_gemm_qkv_store(void* q, const uint8_t* a_q, const float*
   hipStream_t s = (hipStream_t)stream;
   // the 64 x 64 tile the plain product would take for the shape, else the ring of four
   const int tile = default_plan(M, N, K).tile;
-  if (M <= 64) launch_qkv<0>(a_q, w_q, a_scales, w_scales, (int)M, N, K, epi, s);
-  else if (tile == 13) launch_qkv<3>(a_q, w_q, a_scales, w_scales, (int)M, N, K, epi, s);
+  if (tile == 13) launch_qkv<3>(a_q, w_q, a_scales, w_scales, (int)M, N, K, epi, s);
   else launch_qkv<4>(a_q, w_q, a_scales, w_scales, (int)M, N, K, epi, s);
   LFM2_LAUNCH_CHECK();
 }

@@ -744,7 +744,7 @@ def test_prepare_qkv_with_cache_append_equals_the_two_separate_launches(ops, dim
         assert torch.equal(ks0, ks1) and torch.equal(vs0, vs1)
 
 
-@pytest.mark.parametrize("rows", [5, 64, 256, 300])      # register-staged tile, one ring tile, the decode batch, a ragged last tile
+@pytest.mark.parametrize("rows", [5, 64, 256, 300])      # a few rows of one ring tile, a full tile, the decode batch, a ragged last tile
 @pytest.mark.parametrize("fp8", [True, False])
 @torch.inference_mode()
 def test_qkv_projection_with_prepare_and_append_as_its_epilogue_equals_the_two_launches(ops, rows, fp8):
