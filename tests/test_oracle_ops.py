@@ -215,7 +215,7 @@ def test_w8a8_emulation_is_exact_on_grid_inputs_and_bounded_otherwise():
     """Inputs that already sit on the e4m3 grid of their row (maximum mapped to 448) survive quantisation unchanged,
     so the emulated projection equals the exact one; for arbitrary inputs the deviation obeys the half-ulp bound
     |dy| <= sum |x||w| * ((1 + 2^-4)^2 - 1) of two relative roundings of at most 2^-4 each."""
-    from climbing_gym_amd.synthetic import TINY, random_state_dict
+    from climbing_gym_amd.synthetic import random_state_dict
     codes = torch.tensor([v for v, _ in _all_e4m3_values() if abs(v) >= 2 ** -6 or v == 0])
     g = torch.Generator().manual_seed(9)
     pick = lambda r, c: codes[torch.randint(0, len(codes), (r, c), generator=g)]
