@@ -160,7 +160,7 @@ def test_quantize_rows_is_bit_exact_with_oracle_and_rejects_bad_input(ops):
 
 
 @pytest.mark.parametrize("batch,width,outputs", [(3, 129, 193), (128, 2048, 512), (32, 8192, 128), (1, 2048, 3072),
-                                                 (257, 5632, 2048), (64, 2048, 1040)])
+                                                 (257, 5632, 2048), (64, 2048, 1040), (16, 5632, 2048), (48, 5632, 2048)])
 @torch.inference_mode()
 def test_fp8_projection_matches_independently_dequantized_operands(ops, batch, width, outputs):
     torch.manual_seed(42)
