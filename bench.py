@@ -44,11 +44,14 @@ def parse_args():
     p.add_argument("--attn-samples", type=int, default=20, help="timed launches of the decode-attention kernel per layer")
     p.add_argument("--top-k", type=int, default=0, help="top-k filter of the sampler (0: full support)")
     p.add_argument("--top-p", type=float, default=1.0, help="top-p filter of the sampler (1: off)")
-    p.add_argument("--workload", choices=("decode", "attention", "gemm", "prefill"), default="decode",
+    p.add_argument("--workload", choices=("decode", "attention", "gemm", "prefill", "serve"), default="decode",
                    help="decode: the model's decode step (the headline metric); attention: the decode-attention call alone "
                         "on 256 sequences of U[128, 8192] history tokens, dense and paged (block 16), e4m3 and bf16; "
                         "gemm: the W8A8 projection shapes at 1..4096 rows; prefill: causal varlen attention over a packed "
-                        "4096-token chunk")
+                        "4096-token chunk; serve: --requests requests through one session with continuous admit/retire")
+    p.add_argument("--requests", type=int, default=1024, help="requests of the serve workload")
+    p.add_argument("--output-low", type=int, default=64, help="serve workload: shortest output, tokens")
+    p.add_argument("--output-high", type=int, default=256, help="serve workload: longest output, tokens")
     return p.parse_args()
 
 
@@ -255,6 +258,66 @@ def attention_workload(args):
         "cpu_baseline": None}))
 
 
+def serve_workload(args):
+    """Continuous admit/retire: `--requests` requests (prompts U[prompt-low, prompt-high], output lengths
+    U[output-low, output-high], seed 0) flow through one session of `--batch` slots; a finished request frees its slot, and waiting requests are
+    admitted (prefilled) as soon as 16 slots are free or nothing is running.  The figure is whole-job generated tokens
+    per second, prefill and host bookkeeping included."""
+    import collections
+    from climbing_gym_amd.config import LFM25SamplingConfig
+    from climbing_gym_amd.synthetic import LFM2_1P2B, random_prompts, random_state_dict
+    state = random_state_dict(**LFM2_1P2B, seed=0)
+    prompts = random_prompts(args.requests, args.prompt_low, args.prompt_high, LFM2_1P2B["vocab"], seed=0)
+    lengths = torch.randint(args.output_low, args.output_high + 1, (args.requests,), generator=torch.Generator().manual_seed(1)).tolist()
+    engine, _ = build_engine(args, state)
+    sampling = [LFM25SamplingConfig(temperature=1.0, seed=1000 + i, max_new_tokens=n, ignore_eos=True, top_k=args.top_k,
+                                    top_p=args.top_p) for i, n in enumerate(lengths)]
+    with engine.generation_session(max_batch_size=8, max_new_tokens=args.output_high, cache_len=args.max_model_len) as session:
+        session.admit(prompts[:8], sampling[:8])     # loads code objects and warms the allocator
+    waiting = collections.deque(range(args.requests))
+    running = generated = polls = admissions = 0
+    owner = {}
+    with engine.generation_session(max_batch_size=args.batch, max_new_tokens=args.output_high, cache_len=args.max_model_len) as session:
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        while waiting or running:
+            free = args.batch - running
+            if waiting and (free >= 16 or running == 0):
+                take = [waiting.popleft() for _ in range(min(free, len(waiting)))]
+                slots = session.admit([prompts[i] for i in take], [sampling[i] for i in take])
+                owner.update(zip(slots, take))
+                running += len(take)
+                admissions += 1
+            for result in session.poll():
+                if len(result.token_ids) != lengths[owner[result.handle.slot]]:
+                    raise SystemExit("a request finished at the wrong length")
+                generated += len(result.token_ids)
+                session.release(result.handle)
+                running -= 1
+            polls += 1
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        stats = dict(session.stats)
+    if generated != sum(lengths):
+        raise SystemExit(f"generated {generated} tokens, expected {sum(lengths)}")
+    steps = stats["decode_steps"]
+    print(json.dumps({
+        "metric": "whole-job output tok/s, continuous admit/retire", "value": round(generated / elapsed, 1), "unit": "tok/s",
+        "n_gpus": 1, "steps": steps, "warmup": 0, "ms_per_step": round(elapsed / steps * 1000, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp8_e4m3 (W8A8, fp32 accumulate; bf16 activations)" if fp8_requested(args) else "bf16", "data": "synthetic",
+        "config": {"workload": f"{args.requests} requests through {args.batch} slots, prompts U[{args.prompt_low},"
+                               f"{args.prompt_high}], output lengths U[{args.output_low},{args.output_high}], temperature 1"
+                               f"{'' if args.top_k == 0 and args.top_p == 1.0 else f', top-k {args.top_k}, top-p {args.top_p}'}, "
+                               f"LFM2.5-1.2B shape, {args.precision} linears and KV cache",
+                   "generated_tokens": generated, "prompt_tokens": sum(map(len, prompts)), "seconds": round(elapsed, 3),
+                   "admissions": admissions, "polls": polls, "decode_steps": steps,
+                   "prompt_plus_output_tok_per_s": round((generated + sum(map(len, prompts))) / elapsed, 1),
+                   "mean_compute_rows_per_step": round(stats["decode_row_steps"] / max(steps, 1), 1),
+                   "slot_refills": stats["slot_refills"]},
+        "roofline": None, "cpu_baseline": None}))
+
+
 def build_engine(args, state):
     from climbing_gym_amd.config import LFM2Config
     from climbing_gym_amd.engine import LFM25Engine
@@ -416,7 +479,8 @@ def main():
         sys.exit(2)
     if args.workload != "decode":
         with torch.inference_mode():
-            {"attention": attention_workload, "gemm": gemm_workload, "prefill": prefill_workload}[args.workload](args)
+            {"attention": attention_workload, "gemm": gemm_workload, "prefill": prefill_workload,
+             "serve": serve_workload}[args.workload](args)
         return
     from climbing_gym_amd.config import LFM25SamplingConfig
     from climbing_gym_amd.synthetic import LFM2_1P2B, random_prompts, random_state_dict
