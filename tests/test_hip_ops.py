@@ -484,11 +484,11 @@ def test_paged_slot_mapped_history_equals_dense_history(ops, fp8):
     assert torch.equal(paged, dense)
 
 
+@pytest.mark.parametrize("lengths", [[1, 7, 64, 65, 130, 33], [300, 1, 129, 513, 64, 128, 257]])   # up to 3 and up to 9 query blocks per sequence
 @pytest.mark.parametrize("dim,qh,kh", [(64, 32, 8), (64, 4, 2), (32, 4, 4), (128, 4, 1)])
 @torch.inference_mode()
-def test_varlen_prefill_attention_matches_causal_sdpa(ops, dim, qh, kh):
+def test_varlen_prefill_attention_matches_causal_sdpa(ops, dim, qh, kh, lengths):
     torch.manual_seed(11)
-    lengths = [1, 7, 64, 65, 130, 33]
     total = sum(lengths)
     q = torch.randn(total, qh, dim).bfloat16()
     k = torch.randn(total, kh, dim).bfloat16()
