@@ -884,7 +884,7 @@ template <> struct HalfMfma<_Float16> {
 // so softmax statistics never cross rows and P needs no relayout; the contraction order over the
 // 64 tokens of a tile is the same permutation on both operands.
 template <typename T, int D>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 prefill_attn_kernel(T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
                     const int32_t* __restrict__ cu, int QH, int KH, float scale_log2e) {
   typedef typename HalfMfma<T>::vec8 vec8;
