@@ -491,13 +491,20 @@ gemm_naive_kernel(void* out, const uint8_t* A, const uint8_t* W, const float* a_
 }
 
 struct TileInfo { int bm, bn, ks; };
-constexpr int kNumTiles = 23;
+constexpr int kNumTiles = 50;
 constexpr TileInfo kTiles[kNumTiles] = {{16, 64, 128}, {32, 64, 128}, {64, 64, 128}, {128, 64, 128}, {128, 128, 128},
                                         {64, 128, 128}, {128, 128, 128}, {64, 128, 128}, {128, 64, 128},
                                         {16, 64, 256}, {32, 64, 256}, {64, 64, 256},
                                         {32, 64, 128}, {64, 64, 128}, {128, 128, 128}, {32, 64, 256},
                                         {64, 64, 128}, {32, 64, 128}, {16, 64, 256}, {128, 64, 128}, {64, 128, 128},
-                                        {16, 64, 128}, {128, 64, 128}};
+                                        {16, 64, 128}, {128, 64, 128},
+                                        {64, 176, 128}, {64, 176, 128}, {64, 96, 128}, {64, 96, 128}, {256, 128, 128},
+                                        {256, 128, 128}, {64, 128, 128}, {128, 176, 128}, {128, 96, 128}, {64, 128, 128},
+                                        {32, 128, 128},
+                                        {64, 192, 128}, {64, 192, 128}, {128, 96, 128}, {64, 96, 128}, {64, 64, 128},
+                                        {64, 96, 128}, {128, 96, 128},
+                                        {128, 96, 256}, {64, 96, 256}, {128, 96, 128}, {128, 96, 256}, {64, 96, 256},
+                                        {32, 64, 128}, {32, 64, 256}, {32, 64, 256}, {64, 64, 256}};
 int64_t tile_steps(int tile, int64_t Kb) { return (Kb + kTiles[tile].ks - 1) / kTiles[tile].ks; }
 
 struct Plan { int tile, splits; };
@@ -531,6 +538,15 @@ Plan default_plan(int64_t M, int64_t N, int64_t Kb) {
     const int splits = (int)(512 / count(13));
     return {13, splits > 4 ? 4 : splits};
   }
+  // One tile per CU, as square as the output allows, with many waves: the K loop moves about 50 B/ns into a CU
+  // whatever the ring depth or step size, so the bytes a CU pulls decide (tile rows + columns, times K).
+  // 256 rows: N 11264 on 128x96 tiles of 16 waves 15.4 us against 19.4 on 64x64; N 6144 on 64x96 tiles of 8 waves
+  // 10.9 against 13.1; 512 rows, N 6144 on 128x96 tiles of 8 waves 15.2 against 17.7.
+  if (M > 128 && M <= 256 && steps <= 32) {
+    if (N % 96 == 0 && count(37) <= 256 && count(37) > 128) return {37, 1};
+    if (N >= 8192 && count(36) <= 256) return {36, 1};
+  }
+  if (M > 256 && M <= 512 && steps <= 32 && N % 96 == 0 && count(31) <= 256 && count(31) > 128) return {31, 1};
   if (count(6) >= 256) return {14, 1};                // 128x128, ring of 2
   if (count(2) >= 512) return {13, 1};                // 64x64, ring of 3
   // one round of 64x64 tiles over the 256 CUs beats two rounds of 32x64 (512 rows, N 2048: K 5632 16.8 us against
@@ -620,6 +636,33 @@ int gemm_entry(const char* name, void* out, const void* a, const float* as, cons
     TILE_(20, 64, 128, 2, 4, 128, 2);
     TILE_(21, 16, 64, 1, 4, 128, 4);
     TILE_(22, 128, 64, 2, 2, 128, 2);
+    TILE_(23, 64, 176, 4, 1, 128, 3);
+    TILE_(24, 64, 176, 4, 1, 128, 4);
+    TILE_(25, 64, 96, 2, 2, 128, 4);
+    TILE_(26, 64, 96, 2, 2, 128, 3);
+    TILE_(27, 256, 128, 4, 2, 128, 2);
+    TILE_(28, 256, 128, 4, 2, 128, 3);
+    TILE_(29, 64, 128, 2, 4, 128, 4);
+    TILE_(30, 128, 176, 4, 1, 128, 3);
+    TILE_(31, 128, 96, 4, 2, 128, 3);
+    TILE_(32, 64, 128, 2, 2, 128, 4);
+    TILE_(33, 32, 128, 2, 2, 128, 4);
+    TILE_(34, 64, 192, 2, 4, 128, 3);
+    TILE_(35, 64, 192, 4, 4, 128, 3);
+    TILE_(36, 128, 96, 8, 2, 128, 3);
+    TILE_(37, 64, 96, 4, 2, 128, 4);
+    TILE_(38, 64, 64, 4, 4, 128, 4);
+    TILE_(39, 64, 96, 4, 2, 128, 6);
+    TILE_(40, 128, 96, 4, 2, 128, 4);
+    TILE_(41, 128, 96, 8, 2, 256, 2);
+    TILE_(42, 64, 96, 4, 2, 256, 3);
+    TILE_(43, 128, 96, 8, 2, 128, 5);
+    TILE_(44, 128, 96, 4, 2, 256, 2);
+    TILE_(45, 64, 96, 2, 2, 256, 3);
+    TILE_(46, 32, 64, 2, 2, 128, 8);
+    TILE_(47, 32, 64, 2, 2, 256, 4);
+    TILE_(48, 32, 64, 2, 2, 256, 6);
+    TILE_(49, 64, 64, 2, 2, 256, 4);
   }
 #undef TILE_
   if (plan.splits > 1 && reduce)

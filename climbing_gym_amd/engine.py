@@ -290,15 +290,9 @@ class LFM25Engine:
         return hidden, residual
 
     def _head(self, hidden, residual, fp8, place=None):
+        """Final norm and the vocabulary projection; with `place` the product's rows land in `place.out`."""
         logits, _ = self._norm_linear(hidden, self.weights.embedding_norm_weight, residual, self.weights.lm_head_weight, fp8,
-                                      place if self.dtype == torch.bfloat16 or id(self.weights.lm_head_weight) in fp8 else None)
-        if place is not None and logits is not place.out:   # a product the placing GEMM does not cover (fp16/fp32 head)
-            if place.active is None and place.slots is None:
-                place.out[:logits.size(0)].copy_(logits)
-            else:
-                active = place.active if place.active is not None else torch.ones(logits.size(0), device=logits.device, dtype=torch.bool)
-                ops.scatter_logits(place.out, logits, place.slots, active)
-            return place.out
+                                      place)
         return logits
 
     # ------------------------------------------------------------------ decode step (one token per row)

@@ -263,13 +263,11 @@ class RowPlacement:
 
 def linear(x: torch.Tensor, weight: torch.Tensor, *, tile: int = -1, split_k: int = 0,
            place: Optional[RowPlacement] = None, defer_reduce: bool = False):
-    """lfm25_cuda_kernels.py:19-29: y = x W^T.  bf16 runs the MFMA kernel of this package; other dtypes
-    (only used by tests of the fp32 plumbing) go to the vendor GEMM.  With `place`, rows land in `place.out`.  With
-    `defer_reduce`, a product the plan splits along K comes back as a `SplitProduct` for `rms_norm` to reduce."""
-    if x.dtype != torch.bfloat16:
-        if place is not None:
-            raise ValueError("placed rows need a bf16 product")
-        return torch.nn.functional.linear(x, weight)
+    """lfm25_cuda_kernels.py:19-29: y = x W^T on the bf16 MFMA kernel of this package; any other dtype is refused
+    (there is no vendor-library path).  With `place`, rows land in `place.out`.  With `defer_reduce`, a product the
+    plan splits along K comes back as a `SplitProduct` for `rms_norm` to reduce."""
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise ValueError("linear runs in bfloat16 only: this package has no GEMM for other dtypes")
     _check(x, weight)
     m, k = _rows(x), x.size(-1)
     n = weight.size(0)
