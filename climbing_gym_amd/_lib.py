@@ -49,6 +49,7 @@ _SIGNATURES = {
     "lfm2_scatter_logits": "pppp" "llip",
     "lfm2_advance_positions": "pppp" "lp",
     "lfm2_sample": "ppppppp" "llfllip",
+    "lfm2_sample_static": "pppppp" "llfllip",
     "lfm2_sample_filtered": "pppppp" "llfifllip",
     "lfm2_head_logprobs": "ppppp" "lliip",
     "lfm2_record_sample": "ppppppppppppppp" "llllp",

@@ -4,6 +4,8 @@
 // used by compact decode batches.  Nothing here synchronises with the host.
 #include "lfm2_common.h"
 
+#include <mutex>
+
 namespace {
 
 #define DISPATCH_DTYPE(dtype, name, ...)                                               \
@@ -898,6 +900,52 @@ extern "C" int lfm2_sample(int64_t* tokens, float* logprobs, const void* logits,
                  hipLaunchKernelGGL(sample_finish_kernel<T>, dim3(B), dim3(256), 0, s, (const T*)logits, scratch, tokens,
                                     logprobs, seeds, steps, temperatures, seed, step, temperature, V, parts));
   LFM2_LAUNCH_CHECK();
+}
+
+// ---- the sampler for callers that cannot allocate: the tile statistics live in a file-scope device array ----------
+// One array per GPU (each device that loads this code object holds its own copy at its own address, until the process
+// ends).  Host code never passes the array's name to a kernel: the name is a host-side stand-in, the device address
+// comes from hipGetSymbolAddress, looked up once per device with that device current.
+constexpr int64_t kStaticTiles = 16384;                       // rows x 4096-column tiles one call may use
+static __device__ __align__(256) float scratch[kStaticTiles * 4];   // 256 KiB
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_static_mutex;
+float* g_static_scratch[kMaxDevices] = {};
+// Device address of `scratch` on the current device, or nullptr with the error text set.
+float* static_scratch() {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) {
+    lfm2_set_error("sample_static: no current device, or a device index above %d", kMaxDevices - 1);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_static_mutex);
+  if (g_static_scratch[device] == nullptr) {
+    float* ptr = nullptr;
+    const hipError_t status = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+    if (status != hipSuccess || ptr == nullptr) {
+      lfm2_set_error("sample_static: hipGetSymbolAddress failed: %s", hipGetErrorString(status));
+      return nullptr;
+    }
+    g_static_scratch[device] = ptr;
+  }
+  return g_static_scratch[device];
+}
+}  // namespace
+
+extern "C" int lfm2_sample_static(int64_t* tokens, float* logprobs, const void* logits, const int64_t* seeds,
+                                  const int64_t* steps, const float* temperatures, int64_t seed, int64_t step,
+                                  float temperature, int64_t B, int64_t V, int dtype, void* stream) {
+  LFM2_REQUIRE(B > 0 && V > 0, "sample_static: empty logits");
+  const int64_t tiles = B * ((V + kTile - 1) / kTile);
+  LFM2_REQUIRE(tiles <= kStaticTiles,
+               "sample_static: %ld rows x %ld tiles of 4096 columns = %ld tile records, the static scratch holds %ld "
+               "(use lfm2_sample with a caller-provided scratch)", (long)B, (long)((V + kTile - 1) / kTile), (long)tiles,
+               (long)kStaticTiles);
+  float* ptr = static_scratch();
+  if (ptr == nullptr) return LFM2_ERR_LAUNCH;
+  // pass 1 writes every record pass 2 reads, so nothing of the previous call's contents needs clearing
+  return lfm2_sample(tokens, logprobs, logits, ptr, seeds, steps, temperatures, seed, step, temperature, B, V, dtype, stream);
 }
 
 extern "C" int lfm2_sample_filtered(int64_t* tokens, float* logprobs, int32_t* kept_count, const void* logits,

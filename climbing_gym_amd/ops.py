@@ -473,6 +473,19 @@ def sample_logits(logits: torch.Tensor, *, temperature: float, seed: int, step: 
     return tokens, logprobs
 
 
+def sample_logits_static(logits: torch.Tensor, tokens: torch.Tensor, logprobs: torch.Tensor | None, *, temperature: float,
+                         seed: int, step: int):
+    """`sample_logits` into caller-provided outputs with no device allocation at all: the sampler's tile statistics
+    live in a fixed 256 KiB array inside the library (at most 16384 row-tiles of 4096 logits per call; calls that
+    overlap on one GPU race on it).  For callers that must not allocate; no counterpart in the reference."""
+    if logits.ndim != 2 or not logits.is_cuda or not logits.is_contiguous():
+        raise ValueError("sampling requires a contiguous 2D GPU logits tensor")
+    batch, vocab = logits.shape
+    call("lfm2_sample_static", tokens, logprobs, logits, None, None, None, int(seed) & 0x7FFFFFFFFFFFFFFF, int(step),
+         float(temperature), batch, vocab, _code(logits.dtype))
+    return tokens, logprobs
+
+
 class RowSampler:
     """lfm25_sampling.py:95-123: per-row seeds/steps/temperatures; returns buffers that are reused."""
 

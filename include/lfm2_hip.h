@@ -245,6 +245,17 @@ int lfm2_sample(int64_t* tokens, float* logprobs, const void* logits, float* scr
                 const int64_t* steps, const float* temperatures, int64_t seed, int64_t step, float temperature,
                 int64_t B, int64_t V, int dtype, void* stream);
 
+/* lfm2_sample without the scratch argument, for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): the tile statistics go to a file-scope device array
+ * of 256 KiB that each GPU holds until the process ends.  No counterpart in the reference.  It allocates nothing and
+ * calls nothing that allocates; B * ceil(V / 4096) must not exceed 16384 (e.g. 1024 rows of 65536 logits), larger
+ * calls are refused with LFM2_ERR_ARGUMENT.  Every call on a GPU shares that GPU's array: calls that overlap on one
+ * GPU (two streams) race; calls ordered on one stream do not, and nothing of an earlier call's contents is read.
+ * The first call on a device looks the array's address up (hipGetSymbolAddress) and must come outside a capture. */
+int lfm2_sample_static(int64_t* tokens, float* logprobs, const void* logits, const int64_t* seeds, const int64_t* steps,
+                       const float* temperatures, int64_t seed, int64_t step, float temperature, int64_t B, int64_t V,
+                       int dtype, void* stream);
+
 /* _sample + _apply_top_k_top_p of lfm25_engine.py:1574-1609,1759-1774 on the device: temperature,
  * top-k (ties with the k-th value kept), nucleus (rank 0 never dropped), then a Gumbel-max draw
  * from what is left.  kept_count int32[B] (may be NULL) reports the survivors. */
