@@ -50,7 +50,8 @@ _SIGNATURES = {
     "lfm2_advance_positions": "pppp" "lp",
     "lfm2_sample": "ppppppp" "llfllip",
     "lfm2_sample_static": "pppppp" "llfllip",
-    "lfm2_sample_filtered": "pppppp" "llfifllip",
+    "lfm2_sample_filtered": "ppppppppp" "llfifllip",
+    "lfm2_configure_rows": "p" "ll" "ppppppppppppp" "p",
     "lfm2_head_logprobs": "ppppp" "lliip",
     "lfm2_record_sample": "ppppppppppppppp" "llllp",
     "lfm2_record_head": "pppppp" "illp",

@@ -271,7 +271,14 @@ constexpr int kFT = 1024;  // threads of the filtered sampler
 template <typename T>
 __global__ void __launch_bounds__(kFT)
 sample_filtered_stream_kernel(const T* logits, int64_t* tokens, float* logprobs, int32_t* kept_count, const int64_t* seeds,
-                       const int64_t* steps, int64_t seed, int64_t step, float temperature, int top_k, float top_p, int64_t V) {
+                       const int64_t* steps, const float* temperatures, const int32_t* top_ks, const float* top_ps, int64_t seed,
+                       int64_t step, float temperature, int top_k, float top_p, int64_t V) {
+  if (temperatures) {   // per-row parameters: rows that ask for no filter (or are greedy) keep what the outputs hold
+    temperature = temperatures[blockIdx.x];
+    top_k = top_ks[blockIdx.x];
+    top_p = top_ps[blockIdx.x];
+    if (!(temperature > 0.f) || (top_k <= 0 && !(top_p < 1.0f))) return;
+  }
   __shared__ uint32_t h_cnt[256];
   __shared__ unsigned long long h_mass[256];
   __shared__ float s_f[kFT / 64];
@@ -484,7 +491,14 @@ struct Crossed { int bin; uint32_t count_above, count_at; unsigned long long mas
 template <typename T>
 __global__ void __launch_bounds__(kFT)
 sample_filtered_kernel(const T* logits, int64_t* tokens, float* logprobs, int32_t* kept_count, const int64_t* seeds,
-                       const int64_t* steps, int64_t seed, int64_t step, float temperature, int top_k, float top_p, int64_t V) {
+                       const int64_t* steps, const float* temperatures, const int32_t* top_ks, const float* top_ps, int64_t seed,
+                       int64_t step, float temperature, int top_k, float top_p, int64_t V) {
+  if (temperatures) {   // per-row parameters: rows that ask for no filter (or are greedy) keep what the outputs hold
+    temperature = temperatures[blockIdx.x];
+    top_k = top_ks[blockIdx.x];
+    top_p = top_ps[blockIdx.x];
+    if (!(temperature > 0.f) || (top_k <= 0 && !(top_p < 1.0f))) return;
+  }
   constexpr int EPV = 16 / sizeof(T), CHUNKS = kFV / EPV, WAVES = kFT / 64;
   __shared__ uint32_t h_cnt[kBins];
   __shared__ unsigned long long h_mass[kBins];
@@ -833,6 +847,34 @@ __global__ void record_sample_kernel(const int64_t* sampled, const float* logp, 
   input[row] = token;
 }
 
+// Per-row state of newly admitted requests (the state tensors of lfm25_session.py:150-165, set per request at
+// :244-262), all columns in one launch.  A spec is eight int64 words: slot, length limit, seed, emitted-token count
+// the random stream continues from, stop-automaton state, offset of the request's automaton in the flat stop table,
+// flags (bit 0: ignore EOS; bits 8..39: top_k), and temperature | top_p as two float bit patterns (low, high word).
+__global__ void configure_rows_kernel(const int64_t* specs, int64_t count, int64_t rows, int32_t* lengths, int32_t* limits,
+                                      int8_t* reasons, uint8_t* alive, uint8_t* pending, uint8_t* ignore_eos,
+                                      float* temperatures, int32_t* top_ks, float* top_ps, int64_t* seeds,
+                                      int64_t* rng_positions, int64_t* stop_states, int64_t* stop_offsets) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  const int64_t* spec = specs + i * 8;
+  const int64_t slot = spec[0];
+  if (slot < 0 || slot >= rows) return;
+  lengths[slot] = 0;
+  reasons[slot] = 0;
+  alive[slot] = 1;
+  pending[slot] = 0;
+  limits[slot] = (int32_t)spec[1];
+  seeds[slot] = spec[2];
+  rng_positions[slot] = spec[3];
+  stop_states[slot] = spec[4];
+  stop_offsets[slot] = spec[5];
+  ignore_eos[slot] = (uint8_t)(spec[6] & 1);
+  top_ks[slot] = (int32_t)((spec[6] >> 8) & 0xffffffffll);
+  temperatures[slot] = __uint_as_float((uint32_t)(spec[7] & 0xffffffffll));
+  top_ps[slot] = __uint_as_float((uint32_t)((uint64_t)spec[7] >> 32));
+}
+
 __global__ void record_head_kernel(const int64_t* ids, const float* probs, int32_t* out_ids, float* out_probs,
                                    const int32_t* lengths, const uint8_t* alive, int K, int64_t cap) {
   const int64_t row = blockIdx.x;
@@ -949,22 +991,41 @@ extern "C" int lfm2_sample_static(int64_t* tokens, float* logprobs, const void* 
 }
 
 extern "C" int lfm2_sample_filtered(int64_t* tokens, float* logprobs, int32_t* kept_count, const void* logits,
-                                    const int64_t* seeds, const int64_t* steps, int64_t seed, int64_t step,
+                                    const int64_t* seeds, const int64_t* steps, const float* temperatures,
+                                    const int32_t* top_ks, const float* top_ps, int64_t seed, int64_t step,
                                     float temperature, int top_k, float top_p, int64_t B, int64_t V, int dtype,
                                     void* stream) {
   LFM2_REQUIRE(B > 0 && V > 0, "sample_filtered: empty logits");
-  LFM2_REQUIRE(temperature > 0.f, "sample_filtered: temperature must be positive");
-  LFM2_REQUIRE(top_k >= 0 && top_p > 0.f && top_p <= 1.f, "sample_filtered: top_k >= 0 and top_p in (0,1] required");
+  LFM2_REQUIRE((temperatures == nullptr) == (top_ks == nullptr) && (temperatures == nullptr) == (top_ps == nullptr),
+               "sample_filtered: per-row temperatures, top_ks and top_ps go together");
+  if (temperatures == nullptr) {
+    LFM2_REQUIRE(temperature > 0.f, "sample_filtered: temperature must be positive");
+    LFM2_REQUIRE(top_k >= 0 && top_p > 0.f && top_p <= 1.f, "sample_filtered: top_k >= 0 and top_p in (0,1] required");
+  }
   LFM2_REQUIRE(V < (1ll << 31), "sample_filtered: vocabulary too large");
   LFM2_REQUIRE((seeds == nullptr) == (steps == nullptr), "sample_filtered: seeds and steps go together");
   DISPATCH_DTYPE(dtype, "sample_filtered",
                  if (V <= (int64_t)kFT * kFV)
                    hipLaunchKernelGGL(sample_filtered_kernel<T>, dim3(B), dim3(kFT), 0, (hipStream_t)stream, (const T*)logits,
-                                      tokens, logprobs, kept_count, seeds, steps, seed, step, temperature, top_k, top_p, V);
+                                      tokens, logprobs, kept_count, seeds, steps, temperatures, top_ks, top_ps, seed, step,
+                                      temperature, top_k, top_p, V);
                  else
                    hipLaunchKernelGGL(sample_filtered_stream_kernel<T>, dim3(B), dim3(kFT), 0, (hipStream_t)stream,
-                                      (const T*)logits, tokens, logprobs, kept_count, seeds, steps, seed, step, temperature,
-                                      top_k, top_p, V));
+                                      (const T*)logits, tokens, logprobs, kept_count, seeds, steps, temperatures, top_ks, top_ps,
+                                      seed, step, temperature, top_k, top_p, V));
+  LFM2_LAUNCH_CHECK();
+}
+
+extern "C" int lfm2_configure_rows(const int64_t* specs, int64_t count, int64_t rows, int32_t* lengths, int32_t* limits,
+                                   int8_t* reasons, uint8_t* alive, uint8_t* pending, uint8_t* ignore_eos,
+                                   float* temperatures, int32_t* top_ks, float* top_ps, int64_t* seeds,
+                                   int64_t* rng_positions, int64_t* stop_states, int64_t* stop_offsets, void* stream) {
+  LFM2_REQUIRE(count > 0 && rows > 0, "configure_rows: empty request list");
+  LFM2_REQUIRE(specs && lengths && limits && reasons && alive && pending && ignore_eos && temperatures && top_ks && top_ps &&
+               seeds && rng_positions && stop_states && stop_offsets, "configure_rows: a state column is missing");
+  hipLaunchKernelGGL(configure_rows_kernel, dim3(ceil_div(count, 128)), dim3(128), 0, (hipStream_t)stream, specs, count, rows,
+                     lengths, limits, reasons, alive, pending, ignore_eos, temperatures, top_ks, top_ps, seeds, rng_positions,
+                     stop_states, stop_offsets);
   LFM2_LAUNCH_CHECK();
 }
 

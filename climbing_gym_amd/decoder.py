@@ -137,13 +137,16 @@ class LFM25HIPDecoder:
         current.wait_stream(stream)
         torch.cuda.synchronize(device)
         graph = torch.cuda.CUDAGraph()
-        # torch.cuda.graph collects garbage before the capture begins; the cyclic collector must not run again until
-        # it ends: finalising an unreachable graph or stream of an earlier engine while this stream is capturing
-        # aborts the process
+        # Destroying a graph, a graph executable or a stream is one of the calls HIP forbids while a capture is open:
+        # under the default (global) capture mode any thread that makes one invalidates the capture and the runtime
+        # aborts the process.  Two sources of such calls exist here: the cyclic collector finalising an unreachable
+        # engine's graphs and streams in the middle of this capture (torch.cuda.graph collects once before the capture
+        # begins; the collector stays off until it ends), and another host thread dropping the last reference to such
+        # an object (thread-local capture mode confines the check to the capturing thread).
         collector_was_on = gc.isenabled()
         gc.disable()
         try:
-            with torch.cuda.graph(graph, stream=stream):
+            with torch.cuda.graph(graph, stream=stream, capture_error_mode="thread_local"):
                 step()
         finally:
             if collector_was_on:

@@ -501,10 +501,12 @@ class RowSampler:
         return self.tokens, self.logprobs
 
 
-def sample_filtered(logits, *, temperature: float, top_k: int, top_p: float, seed: int = 0, step: int = 0,
-                    seeds=None, steps=None, return_kept: bool = False, out=None):
+def sample_filtered(logits, *, temperature: float = 1.0, top_k: int = 0, top_p: float = 1.0, seed: int = 0, step: int = 0,
+                    seeds=None, steps=None, temperatures=None, top_ks=None, top_ps=None, return_kept: bool = False, out=None):
     """Device form of `_sample` + `_apply_top_k_top_p` (lfm25_engine.py:1574-1609, 1759-1774) for temperature > 0:
-    returns (tokens, raw log-probabilities[, survivors per row])."""
+    returns (tokens, raw log-probabilities[, survivors per row]).  With per-row `temperatures`, `top_ks` (int32) and
+    `top_ps` every row has its own parameters, and rows that ask for no filter or for greedy decoding are left as `out`
+    holds them."""
     if logits.ndim != 2 or not logits.is_cuda:
         raise ValueError("sampling requires a 2D GPU logits tensor")
     logits = logits.contiguous()
@@ -513,8 +515,9 @@ def sample_filtered(logits, *, temperature: float, top_k: int, top_p: float, see
         torch.empty(batch, device=logits.device, dtype=torch.long),
         torch.empty(batch, device=logits.device, dtype=torch.float32))
     kept = torch.empty(batch, device=logits.device, dtype=torch.int32) if return_kept else None
-    call("lfm2_sample_filtered", tokens, logprobs, kept, logits, seeds, steps, int(seed) & 0x7FFFFFFFFFFFFFFF,
-         int(step), float(temperature), int(top_k), float(top_p), batch, vocab, _code(logits.dtype))
+    call("lfm2_sample_filtered", tokens, logprobs, kept, logits, seeds, steps, temperatures, top_ks, top_ps,
+         int(seed) & 0x7FFFFFFFFFFFFFFF, int(step), float(temperature), int(top_k), float(top_p), batch, vocab,
+         _code(logits.dtype))
     return (tokens, logprobs, kept) if return_kept else (tokens, logprobs)
 
 
@@ -535,6 +538,14 @@ def record_sample(sampled, logp, tokens, logprobs, lengths, limits, reasons, ali
     call("lfm2_record_sample", sampled, logp, tokens, logprobs, lengths, limits, reasons, alive, pending, input_tokens,
          stop_states, stop_offsets, stop_table, ignore_eos, rng_positions, int(eos), int(vocab), int(cap),
          sampled.numel())
+
+
+def configure_rows(specs, table) -> None:
+    """Per-row session state of newly admitted requests in one launch (lfm25_session.py:150-165, 244-262): `specs` is
+    int64 [count, 8] on the device (see `lfm2_configure_rows`), `table` the object that owns the state columns."""
+    call("lfm2_configure_rows", specs, specs.size(0), table.lengths.numel(), table.lengths, table.limits, table.reasons,
+         table.alive, table.pending, table.ignore_eos, table.temperatures, table.top_ks, table.top_ps, table.seeds,
+         table.rng_positions, table.stop_states, table.stop_offsets)
 
 
 def record_head(ids, probs, out_ids, out_probs, lengths, alive, k: int, cap: int):

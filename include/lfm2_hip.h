@@ -258,11 +258,14 @@ int lfm2_sample_static(int64_t* tokens, float* logprobs, const void* logits, con
 
 /* _sample + _apply_top_k_top_p of lfm25_engine.py:1574-1609,1759-1774 on the device: temperature,
  * top-k (ties with the k-th value kept), nucleus (rank 0 never dropped), then a Gumbel-max draw
- * from what is left.  kept_count int32[B] (may be NULL) reports the survivors. */
+ * from what is left.  kept_count int32[B] (may be NULL) reports the survivors.
+ * temperatures float[B], top_ks int32[B], top_ps float[B] (all three or none) give every row its own parameters and
+ * replace the scalars; a row whose parameters ask for no filter (top_k 0 and top_p 1) or for greedy decoding
+ * (temperature 0) is then skipped and its outputs keep their contents (the sampler for those rows is lfm2_sample). */
 int lfm2_sample_filtered(int64_t* tokens, float* logprobs, int32_t* kept_count, const void* logits,
-                         const int64_t* seeds, const int64_t* steps, int64_t seed, int64_t step,
-                         float temperature, int top_k, float top_p, int64_t B, int64_t V, int dtype,
-                         void* stream);
+                         const int64_t* seeds, const int64_t* steps, const float* temperatures, const int32_t* top_ks,
+                         const float* top_ps, int64_t seed, int64_t step, float temperature, int top_k, float top_p,
+                         int64_t B, int64_t V, int dtype, void* stream);
 
 /* _head_logprobs of lfm25_sampling.py:126-149: out[b,j] = values[b,j] - logZ(b). */
 int lfm2_head_logprobs(float* out, const void* logits, const int64_t* selected, const float* logprobs,
@@ -274,6 +277,15 @@ int lfm2_record_sample(const int64_t* sampled, const float* logp, int64_t* token
                        uint8_t* pending, int64_t* input, int64_t* stop_states, const int64_t* stop_offsets,
                        const int32_t* stop_table, const uint8_t* ignore_eos, int64_t* rng_positions,
                        int64_t eos, int64_t V, int64_t cap, int64_t B, void* stream);
+/* The per-row state of newly admitted session requests (the state tensors of lfm25_session.py:150-165 as they are set
+ * per request at :244-262) written in one launch: specs int64[count, 8] = slot, length limit, seed, random-stream
+ * position, stop-automaton state, stop-table offset, flags (bit 0 ignore EOS, bits 8..39 top_k), temperature | top_p
+ * (float bit patterns, low | high word).  Row `slot` of every column is set; length and finish reason become 0, the
+ * row alive and not pending.  Specs whose slot is outside [0, rows) are ignored. */
+int lfm2_configure_rows(const int64_t* specs, int64_t count, int64_t rows, int32_t* lengths, int32_t* limits,
+                        int8_t* reasons, uint8_t* alive, uint8_t* pending, uint8_t* ignore_eos, float* temperatures,
+                        int32_t* top_ks, float* top_ps, int64_t* seeds, int64_t* rng_positions, int64_t* stop_states,
+                        int64_t* stop_offsets, void* stream);
 /* _record_head of lfm25_session.py:22-31. */
 int lfm2_record_head(const int64_t* ids, const float* probs, int32_t* out_ids, float* out_probs,
                      const int32_t* lengths, const uint8_t* alive, int K, int64_t cap, int64_t B, void* stream);

@@ -237,6 +237,9 @@ class OracleEngine:
         self.QH, self.KH, self.D = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
         self.scale = self.D ** -0.5
         self.cos, self.sin = rope_tables(self.D, cfg.rope_theta, self.max_model_len)
+        # tests may set this to a list: every layer's input hidden state is then appended as
+        # ("prefill" | "decode", layer index, tensor) -- the `return_hidden` idea of lfm25_engine.py:1097-1098 per layer
+        self.hidden_trace = None
 
     # ---- cache
     def empty_cache(self, slots: int, cap: int) -> OracleCache:
@@ -284,7 +287,9 @@ class OracleEngine:
         pos = torch.arange(T)
         cos, sin = self.cos[pos].view(1, T, 1, -1), self.sin[pos].view(1, T, 1, -1)
         h = F.embedding(ids, self.embed)
-        for L in self.layers:
+        for index, L in enumerate(self.layers):
+            if self.hidden_trace is not None:
+                self.hidden_trace.append(("prefill", index, h.clone()))
             x = rms_norm(h, L.operator_norm, self.cfg.norm_eps)
             if L.kind == "attn":
                 q, k, v = self._qkv_split(L, x, fused_ok=False)
@@ -347,7 +352,9 @@ class OracleEngine:
         n = slots.numel()
         cos, sin = self.cos[pos].unsqueeze(1), self.sin[pos].unsqueeze(1)
         h = F.embedding(tokens.long(), self.embed)
-        for L in self.layers:
+        for index, L in enumerate(self.layers):
+            if self.hidden_trace is not None:
+                self.hidden_trace.append(("decode", index, h.clone()))
             x = rms_norm(h, L.operator_norm, self.cfg.norm_eps)
             if L.kind == "attn":
                 q, k, v = self._qkv_split(L, x, fused_ok=True)
@@ -377,6 +384,8 @@ class OracleEngine:
             h = h + y
             h = h + self._mlp(L, rms_norm(h, L.ffn_norm, self.cfg.norm_eps))
         cache.seq_lens[slots] += 1
+        if self.hidden_trace is not None:
+            self.hidden_trace.append(("decode", len(self.layers), h.clone()))
         return self._lin(rms_norm(h, self.final_norm, self.cfg.norm_eps), self.head, "head")
 
     # ---- sampling (lfm25_engine.py:1574-1609)

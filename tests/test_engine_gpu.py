@@ -92,9 +92,12 @@ def test_tiny_model_greedy_tokens_and_logits_match_cpu_engine():
     cache, first = cpu_bf16.prefill(prompts, cap=192)
     cpu_trace = [first.float()] + [cpu_bf16.append_tokens(cache, torch.arange(4), want_tokens[:, i]).float() for i in range(63)]
     cpu_worst = max((a - b).abs().max().item() for a, b in zip(cpu_trace, trace))
-    print(f"bf16 logits vs fp32 CPU engine: GPU {worst:.3e}, CPU engine in bf16 {cpu_worst:.3e}")
-    # 2e-2 max-abs, or what the reference algorithm itself loses when run in bf16 on the CPU if that is larger
-    assert worst <= max(2e-2, 1.1 * cpu_worst), f"bf16 logits differ from the CPU engine by {worst}"
+    direct = max((a - b).abs().max().item() for a, b in zip(got, cpu_trace))
+    print(f"bf16 logits vs fp32 CPU engine: GPU {worst:.3e}, CPU engine in bf16 {cpu_worst:.3e}; GPU vs CPU engine in bf16 {direct:.3e}")
+    # the stated 2e-2 max-abs against the CPU engine run in the path's own arithmetic (bf16), over all 64 steps; against
+    # the fp32 CPU engine, 2e-2 or what that arithmetic itself loses on the CPU if that is larger
+    assert direct <= 2e-2, f"bf16 logits differ from the CPU engine in bf16 by {direct}"
+    assert worst <= max(2e-2, 1.1 * cpu_worst), f"bf16 logits differ from the fp32 CPU engine by {worst}"
     decided = 0
     for step, (mine, ref) in enumerate(zip(got, trace)):
         top2 = ref.topk(2).values
@@ -159,8 +162,11 @@ def test_fp8_logits_stay_within_tolerance_of_cpu_engine(flags, parts):
         # With 3 mantissa bits and 256-wide rows, W8A8 rounding alone moves these logits by more than 6e-2
         # (`inherent`), and two emulations that differ only in activation precision are as far apart from each
         # other.  The HIP path must be no further from the fp32 engine than the CPU emulation is.
+        # The HIP path must be as close to the emulating CPU engine as that emulation is to the fp32 engine (two
+        # emulations that differ in one rounding are that far apart), and no further from fp32 than the emulation is.
+        assert worst <= 1.1 * inherent
         assert to_fp32 <= 1.25 * inherent + 2e-2
-        assert rms(got, trace) <= 1.25 * rms(trace, trace_fp32) + 1e-3
+        assert rms(got, trace) <= rms(trace, trace_fp32) and rms(got, trace_fp32) <= 1.1 * rms(trace, trace_fp32)
     assert entry.cache.fp8 == bool(flags.get("fp8_kv"))
     n = len(engine._cuda_decoder.fp8_weights)
     assert n == (8 if flags.get("fp8_mlp") else 0) + (1 if flags.get("fp8_lm_head") else 0) + (8 if flags.get("fp8_operators") else 0)
@@ -195,7 +201,7 @@ def test_model_width_layers_at_a_few_rows_match_the_cpu_engine(flags, parts):
     inherent = max((a - b).abs().max().item() for a, b in zip(trace, trace_fp32))
     print(f"{parts or 'bf16'}: GPU vs CPU engine {worst:.3e}; GPU vs fp32 CPU {to_fp32:.3e}; emulated CPU vs fp32 CPU {inherent:.3e}")
     if parts:
-        assert worst <= 6e-2 or to_fp32 <= 1.25 * inherent + 2e-2
+        assert worst <= inherent and to_fp32 <= 1.25 * inherent + 2e-2
     else:
         # 2e-2, or what the same algorithm loses in bf16 on the CPU when that is larger (6e-2 at these widths)
         cpu_bf16 = O.OracleEngine(ocfg, state, torch.bfloat16, max_model_len=128)
@@ -381,6 +387,92 @@ def test_filtered_sampling_in_generate_is_deterministic_and_stays_in_the_support
     greedy = engine.generate(*prompts, repeats=1, sampling=replace(sampling, top_k=1, top_p=1.0))
     argmax = engine.generate(*prompts, repeats=1, sampling=replace(sampling, temperature=0.0, top_k=0, top_p=1.0))
     assert torch.equal(greedy.token_ids, argmax.token_ids)
+
+
+@torch.inference_mode()
+def test_repetition_penalty_in_sample_and_generate_follows_the_cpu_engine():
+    """lfm25_engine.py:1777-1790 applied before the draw (:1587-1597), seen-token mask from the prompt's unique tokens
+    plus every emitted token (:933-961, :806-808).  `_sample` against the oracle on random logits; then a greedy
+    generation whose every step is replayed on the fp32 CPU engine with the same mask bookkeeping."""
+    engine, ocfg, state = _engine()
+    torch.manual_seed(8)
+    logits = (torch.randn(6, 257) * 3).bfloat16()
+    seen = torch.rand(6, 257) < 0.3
+    seen[:, logits.float().argmax(-1)] = True            # the unpenalised winners are all penalised
+    for penalty in (1.0, 1.4, 0.6):
+        sampling = LFM25SamplingConfig(temperature=0.0, repetition_penalty=penalty)
+        tokens, raw = engine._sample(logits.to(DEV), sampling, step=0, seen_token_mask=seen.to(DEV))
+        want_tokens, want_raw = O.OracleEngine.sample(None, logits.float(), temperature=0.0, seen=seen, penalty=penalty)
+        assert torch.equal(tokens.cpu(), want_tokens)
+        torch.testing.assert_close(raw.cpu(), want_raw, atol=3e-6, rtol=0)
+    assert not torch.equal(O.OracleEngine.sample(None, logits.float(), seen=seen, penalty=1.4)[0], logits.float().argmax(-1))
+
+    engine.enable_cuda_graphs(max_graphs=1)
+    prompts = [[1, 5, 9, 5], [3, 4]]
+    sampling = LFM25SamplingConfig(temperature=0.0, max_new_tokens=10, ignore_eos=True, repetition_penalty=1.5)
+    out = engine.generate(*_flat(prompts), repeats=1, sampling=sampling)
+    plain = engine.generate(*_flat(prompts), repeats=1, sampling=replace(sampling, repetition_penalty=1.0))
+    assert not torch.equal(out.token_ids, plain.token_ids)
+    oracle = O.OracleEngine(ocfg, state, torch.float32, max_model_len=256)
+    for row, prompt in enumerate(prompts):
+        cache, row_logits = oracle.prefill([prompt], cap=32)
+        mask = torch.zeros(1, 257, dtype=torch.bool)
+        mask[0, prompt] = True
+        for step, token in enumerate(out.token_ids[row, 0].tolist()):
+            penalised = O.repetition_penalty(row_logits.float(), mask, 1.5)[0]
+            assert penalised.max().item() - penalised[token].item() <= 4e-2, f"row {row} step {step}"
+            assert abs(penalised.log_softmax(-1)[token].item() - out.logprobs[row, 0, step].item()) <= 2e-2
+            mask[0, token] = True
+            row_logits = oracle.append_tokens(cache, torch.arange(1), torch.tensor([token]))
+
+
+def test_graphs_can_be_dropped_and_recaptured_while_garbage_is_collected():
+    """Engines and graphs that die while a later capture is running (the cyclic collector finalising an old graph or
+    stream during capture aborted the process; `_capture` keeps the collector off for the capture's duration):
+    engines are built, used, dropped without cleanup and re-captured, from two host threads taking turns, with
+    reference cycles that only the cyclic collector can free.  Runs in a child process with a time limit so that an
+    abort cannot take the test session with it (tests/helpers/native_graph_recapture.py of the reference)."""
+    import subprocess
+    import sys
+    import textwrap
+    program = textwrap.dedent("""
+        import gc, sys, threading
+        import torch
+        sys.path.insert(0, ROOT)
+        from climbing_gym_amd.config import LFM2Config, LFM25SamplingConfig
+        from climbing_gym_amd.engine import LFM25Engine, flatten_token_batches
+        from climbing_gym_amd.synthetic import random_state_dict
+        shape = dict(hidden=128, mlp_hidden=192, layer_types=("conv", "full_attention"), q_heads=4, kv_heads=2, vocab=257)
+        cfg = LFM2Config(vocab_size=257, hidden_size=128, mlp_hidden_size=192, num_hidden_layers=2, num_attention_heads=4,
+                         num_key_value_heads=2, max_position_embeddings=256, layer_types=shape["layer_types"])
+        state = random_state_dict(**shape, seed=1)
+        sampling = LFM25SamplingConfig(temperature=0.0, max_new_tokens=4, ignore_eos=True)
+        prompts = flatten_token_batches([[1, 2, 3], [4, 5]])
+        lock, outputs = threading.Lock(), []
+
+        def worker(rounds):
+            for i in range(rounds):
+                with lock, torch.inference_mode():
+                    engine = LFM25Engine.from_state_dict(cfg, state, device="cuda", max_model_len=64)
+                    engine.enable_cuda_graphs(max_graphs=2, fp8_mlp=bool(i % 2), fp8_kv=bool(i % 2))
+                    outputs.append(engine.generate(*prompts, repeats=1, sampling=sampling).token_ids.cpu())
+                    engine.generate(*flatten_token_batches([[1, 2, 3, 4, 5, 6], [7], [8, 9]]), repeats=1, sampling=sampling)
+                    engine.cycle = engine          # only the cyclic collector can free this engine and its graphs
+                    del engine
+                if i == rounds // 2:
+                    gc.collect()
+
+        threads = [threading.Thread(target=worker, args=(4,)) for _ in range(2)]
+        for t in threads: t.start()
+        for t in threads: t.join()
+        gc.collect()
+        torch.cuda.synchronize()
+        same = [o for i, o in enumerate(outputs) if i % 2 == 0]
+        assert len(outputs) == 8 and all(torch.equal(o.view(-1)[:1], outputs[0].view(-1)[:1]) for o in same)
+        print("RECAPTURE_OK", len(outputs))
+    """).replace("ROOT", repr(str(__import__("pathlib").Path(__file__).resolve().parents[1])))
+    done = subprocess.run([sys.executable, "-c", program], capture_output=True, text=True, timeout=280)
+    assert done.returncode == 0 and "RECAPTURE_OK 8" in done.stdout, done.stdout[-2000:] + done.stderr[-4000:]
 
 
 # ------------------------------------------------------------------------------------------------ sessions
@@ -582,6 +674,21 @@ class _ByteTokenizer:
         return bytes(int(i) % 256 for i in ids).decode("latin-1")
 
 
+def _assert_greedy_rollout_follows_cpu_engine(oracle, prompt_ids, token_ids, logprobs, tie=4e-2, atol=2e-2):
+    """A greedy completion checked step by step against the fp32 CPU engine fed the same history: each chosen token is
+    the CPU engine's argmax or within `tie` of it, and each recorded log-probability is the CPU engine's raw
+    log-softmax of that token within `atol`.  Returns how many steps chose the CPU engine's own argmax."""
+    cache, logits = oracle.prefill([list(prompt_ids)], cap=len(prompt_ids) + len(token_ids) + 1)
+    exact = 0
+    for step, (token, logprob) in enumerate(zip(token_ids, logprobs)):
+        row = logits[0].float()
+        assert row.max().item() - row[token].item() <= tie, f"step {step}: token {token} is not the CPU engine's choice"
+        exact += int(row.argmax().item() == token)
+        assert abs(row.log_softmax(-1)[token].item() - logprob) <= atol, f"step {step}: log-probability differs"
+        logits = oracle.append_tokens(cache, torch.arange(1), torch.tensor([token]))
+    return exact
+
+
 @torch.inference_mode()
 def test_async_adapter_runs_batches_and_chains_on_the_hip_engine():
     """generate_many gives what a direct engine.generate of the same prompts gives; a two-phase chain whose second
@@ -590,7 +697,8 @@ def test_async_adapter_runs_batches_and_chains_on_the_hip_engine():
     import asyncio
     from climbing_gym_amd.async_engine import LFM25AsyncInferenceEngine
     from climbing_gym_amd.inference_config import InferenceEngineConfig, SamplingConfig
-    engine, _, _ = _engine()
+    engine, ocfg, state = _engine()
+    oracle = O.OracleEngine(ocfg, state, torch.float32, max_model_len=256)
     engine.enable_cuda_graphs(max_graphs=2)
     adapter = LFM25AsyncInferenceEngine.from_components(engine=engine, tokenizer=_ByteTokenizer(),
                                                         config=InferenceEngineConfig(model_path="", seed=3), max_batch_size=8)
@@ -601,6 +709,9 @@ def test_async_adapter_runs_batches_and_chains_on_the_hip_engine():
                              sampling=LFM25SamplingConfig(temperature=0.0, max_new_tokens=12, ignore_eos=True))
     for row, result in enumerate(results):
         assert result.token_ids == tuple(direct.token_ids[row, 0].cpu().tolist())
+        chosen = _assert_greedy_rollout_follows_cpu_engine(oracle, prompts[row].encode("latin-1"), result.token_ids,
+                                                           result.completion_logprobs)
+        assert chosen >= 10
         assert result.outputs[0].finish_reason == "length" and len(result.completion_logprobs) == 12
         assert result.text == _ByteTokenizer().decode(result.token_ids)
 
@@ -622,7 +733,8 @@ def test_async_adapter_runs_batches_and_chains_on_the_hip_engine():
 @torch.inference_mode()
 def test_rollout_runner_collects_groups_through_the_adapter_on_the_hip_engine():
     """The runner's requests (rollout/runner.py:272-305) go through the adapter's queue into batched generate calls of
-    the HIP engine: every trajectory carries the engine's ids and logprobs for its prompt, greedy rollouts of one
+    the HIP engine: every trajectory carries, for its prompt, the greedy ids and raw log-probabilities the fp32 CPU
+    engine gives for the same history (and what a direct engine.generate gives), greedy rollouts of one
     prompt are identical (so with dynamic sampling off the flat groups are kept), and the coordinator parks nothing
     it should not and pushes weights through the adapter."""
     import asyncio
@@ -630,7 +742,8 @@ def test_rollout_runner_collects_groups_through_the_adapter_on_the_hip_engine():
     from climbing_gym_amd.async_engine import LFM25AsyncInferenceEngine
     from climbing_gym_amd.inference_config import InferenceEngineConfig, SamplingConfig
     from climbing_gym_amd.rollout import DirectHarness, RolloutConfig, RolloutRunner, RolloutRunnerConfig
-    engine, _, _ = _engine()
+    engine, ocfg, state = _engine()
+    oracle = O.OracleEngine(ocfg, state, torch.float32, max_model_len=256)
     engine.enable_cuda_graphs(max_graphs=2)
     adapter = LFM25AsyncInferenceEngine.from_components(engine=engine, tokenizer=_ByteTokenizer(),
                                                         config=InferenceEngineConfig(model_path="", seed=3), max_batch_size=8)
@@ -663,5 +776,8 @@ def test_rollout_runner_collects_groups_through_the_adapter_on_the_hip_engine():
         assert turn.completion_token_ids == tuple(direct.token_ids[row, 0].cpu().tolist())
         assert len(turn.completion_logprobs) == 10 and turn.finish_reason == "length"
         assert item.final_response == _ByteTokenizer().decode(turn.completion_token_ids)
+        # the trajectory against the CPU engine itself: ids and log-probabilities, step by step
+        assert _assert_greedy_rollout_follows_cpu_engine(oracle, turn.prompt_token_ids, turn.completion_token_ids,
+                                                         turn.completion_logprobs) >= 8
     adapter.close()
     engine.disable_cuda_graphs()

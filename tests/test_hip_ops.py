@@ -129,12 +129,18 @@ def test_fused_activation_quantization_matches_separate_kernels_and_oracle(ops, 
     actual, actual_scales, summed = ops.rms_norm_fp8(dx, dw, 1e-5, dr)
     assert torch.equal(summed, expected_sum) and torch.equal(actual_scales, scales)
     assert torch.equal(actual.view(torch.uint8), expected.view(torch.uint8))
+    # the quantising half is bit-exact: the oracle's row quantisation of the very values the norm kernel produced
+    oq, oscale = O.k_quantize_rows(normalized.cpu())
+    assert torch.equal(actual_scales.cpu(), oscale) and torch.equal(actual.cpu().view(torch.uint8), oq.view(torch.uint8))
+    # end to end against the oracle the only freedom is the order of the norm's fp32 sum of squares, which moves a
+    # normalised value across a bf16 boundary in well under 1 % of the elements; a row's scale differs only when that
+    # happens to the row's largest element, and then by one bf16 step
     oq, oscale, _ = O.k_rms_norm_fp8(x, weight, 1e-5, residual)
     torch.testing.assert_close(actual_scales.cpu(), oscale, rtol=2 ** -7, atol=0)
     same_scale = actual_scales.cpu() == oscale
-    assert same_scale.float().mean() > 0.8
     mismatch = (actual.cpu().view(torch.uint8) != oq.view(torch.uint8))[same_scale].float().mean().item()
-    assert mismatch < 5e-3
+    print(f"width {width}: rows with the oracle's scale {int(same_scale.sum())}/17, differing e4m3 codes in those rows {mismatch:.2e}")
+    assert same_scale.sum() >= 16 and mismatch < 1e-3
     projected = torch.randn(17, 2 * width).bfloat16()
     expected, scales = ops.quantize_rows(ops.swiglu(projected.to(DEV)))
     actual, actual_scales = ops.swiglu_fp8(projected.to(DEV))
@@ -877,3 +883,47 @@ def test_bf16_split_k_partials_reduce_inside_the_following_norm(ops):
     expected, got = ops.rms_norm_fp8(whole, norm_w, 1e-5, residual), ops.rms_norm_fp8(deferred, norm_w, 1e-5, residual)
     assert torch.equal(got[0].view(torch.uint8), expected[0].view(torch.uint8)) and torch.equal(got[1], expected[1])
     assert isinstance(ops.linear(act[:, :2048].contiguous(), weight[:, :2048].contiguous(), defer_reduce=True), torch.Tensor)
+
+
+# ------------------------------------------------------------------------------------------------ rounding points
+def _rounding_cases():
+    import json, os
+    return json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "rounding_cases.json")))
+
+
+@torch.inference_mode()
+def test_kernels_round_where_the_reference_kernels_round(ops):
+    """The fixtures of tests/golden/rounding_cases.json: inputs on which one rounding point of
+    lfm25_cuda_kernels.py:32-140 decides the bf16 result (the sum, the normalised value, the SwiGLU activation, b*x,
+    each tap product and their sum, the QK-norm stages, the table entries and both RoPE products).  The HIP kernels
+    must give `expected`, never `without`."""
+    cases = _rounding_cases()
+    bf = lambda values: torch.tensor(values, dtype=torch.float32).to(torch.bfloat16).to(DEV)
+    for name in ("rms_add", "rms_norm"):
+        case = cases[name]
+        out, summed = ops.rms_norm(bf([case["x"]]), bf(case["weight"]), case["eps"], bf([case["residual"]]))
+        assert out.float().cpu()[0].tolist() == case["expected"], name
+        assert summed.float().cpu()[0].tolist() == case["summed"], name
+        q, scales, _ = ops.rms_norm_fp8(bf([case["x"]]), bf(case["weight"]), case["eps"], bf([case["residual"]]))
+        oq, oscale = O.k_quantize_rows(torch.tensor([case["expected"]]).bfloat16())
+        assert torch.equal(scales.cpu(), oscale) and torch.equal(q.cpu().view(torch.uint8), oq.view(torch.uint8)), name
+    case = cases["swiglu_act"]
+    row = bf([[case["gate"]] * 8 + [case["up"]] * 8])
+    assert ops.swiglu(row).float().cpu()[0].tolist() == [case["expected"]] * 8
+    for name in ("conv_bx", "conv_p0", "conv_p1", "conv_p2", "conv_sum"):
+        case = cases[name]
+        channels = 8
+        state = bf([[case["state"]] * channels])
+        bcx = bf([[case["b"]] * channels + [case["c"]] * channels + [case["x"]] * channels])
+        out = ops.conv_update(bcx, bf([case["weight"]] * channels), state)
+        assert out.float().cpu()[0].tolist() == [case["expected"]] * channels, name
+        assert state.float().cpu()[0].tolist() == [case["new_state"]] * channels, name
+    for name in ("qk_norm", "qk_weight", "qk_table", "qk_left", "qk_right"):
+        case = cases[name]
+        head, weight = bf(case["x"]), bf(case["weight"])
+        cos = torch.tensor([case["cos"]], dtype=torch.float32, device=DEV)
+        sin = torch.tensor([case["sin"]], dtype=torch.float32, device=DEV)
+        x = torch.cat((head, head, torch.zeros(64, dtype=torch.bfloat16, device=DEV)))[None].contiguous()
+        q, k, v = ops.prepare_qkv(x, weight, weight, cos, sin, torch.zeros(1, dtype=torch.int32, device=DEV), 1, 1, 64, case["eps"])
+        assert q.float().cpu().flatten().tolist() == case["expected"], name
+        assert k.float().cpu().flatten().tolist() == case["expected"], name
