@@ -42,6 +42,8 @@ def parse_args():
     p.add_argument("--cpu-seqs", type=int, default=4, help="sequences of the workload the CPU baseline runs (0 = skip)")
     p.add_argument("--cpu-steps", type=int, default=96)
     p.add_argument("--attn-samples", type=int, default=20, help="timed launches of the decode-attention kernel per layer")
+    p.add_argument("--mid-job-advance", type=int, default=2048,
+                   help="second timed point: the same batch with every context this many tokens longer (0 = skip)")
     p.add_argument("--top-k", type=int, default=0, help="top-k filter of the sampler (0: full support)")
     p.add_argument("--top-p", type=float, default=1.0, help="top-p filter of the sampler (1: off)")
     p.add_argument("--workload", choices=("decode", "attention", "gemm", "prefill", "serve"), default="decode",
@@ -347,22 +349,25 @@ def time_decode_attention(engine, session, samples):
     quantized = bool(cache.fp8 and attention_ops and id(attention_ops[0].out_weight) in engine._fp8()
                      and -(-cfg.num_attention_heads // 16) * -(-cfg.head_dim // 64) <= 4)
     stream = torch.cuda.current_stream()
-    total_ms, launches = 0.0, 0
-    for layer in range(cache.k_cache.size(0)):
-        args = (q, cache.k_cache[layer], cache.v_cache[layer],
-                None if cache.k_scales is None else cache.k_scales[layer],
-                None if cache.v_scales is None else cache.v_scales[layer], positions)
-        ops.attend(*args, active=active, scale=engine._scaling, schedule=schedule, quantized=quantized)  # warm
-        # one pair of events per call: a marker between two calls also keeps the next call's first waves from
-        # starting under the tail of this one, which a kernel trace would count twice
-        marks = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(samples)]
-        for begin, end in marks:
-            begin.record(stream)
-            ops.attend(*args, active=active, scale=engine._scaling, schedule=schedule, quantized=quantized)
-            end.record(stream)
-        marks[-1][1].synchronize()
-        total_ms += sum(begin.elapsed_time(end) for begin, end in marks)
-        launches += samples
+    layers = cache.k_cache.size(0)
+    call_args = [(q, cache.k_cache[layer], cache.v_cache[layer],
+                  None if cache.k_scales is None else cache.k_scales[layer],
+                  None if cache.v_scales is None else cache.v_scales[layer], positions) for layer in range(layers)]
+    run = lambda args: ops.attend(*args, active=active, scale=engine._scaling, schedule=schedule, quantized=quantized)
+    for args in call_args:
+        run(args)   # warm
+    # consecutive calls walk the layers' caches as the decode step does, so every call streams its history from HBM
+    # (six layers' histories do not fit the memory-side cache); one pair of events per call: the marker between two
+    # calls also keeps the next call's first waves from starting under the tail of this one, which a kernel trace
+    # would count twice
+    marks = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(samples * layers)]
+    for index, (begin, end) in enumerate(marks):
+        begin.record(stream)
+        run(call_args[index % layers])
+        end.record(stream)
+    marks[-1][1].synchronize()
+    total_ms = sum(begin.elapsed_time(end) for begin, end in marks)
+    launches = len(marks)
     tokens = int((positions.long() + 1).sum())
     kv_token = cfg.num_key_value_heads * cfg.head_dim * 2 * (1 if cache.fp8 else 2) + (cfg.num_key_value_heads * 2 * 4 if cache.fp8 else 0)
     bytes_per_call = tokens * kv_token + 2 * rows * cfg.num_attention_heads * cfg.head_dim * 2
@@ -503,6 +508,7 @@ def main():
         session.admit(prompts, sampling)
         torch.cuda.synchronize()
         prefill_s = time.perf_counter() - t0
+        prefill_plan = dict(engine.last_prefill)
         session.poll(steps=max(args.warmup, 1))
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -511,14 +517,40 @@ def main():
         elapsed = time.perf_counter() - t0
         assert not finished, "no sequence may finish inside the timed region"
         attn_s, attn_bytes, ctx_tokens = time_decode_attention(engine, session, args.attn_samples)
+        kv_token = 6 * (attn_bytes - 2 * args.batch * 32 * 64 * 2) // max(ctx_tokens, 1)
+        # the same batch later in the job: every row's context longer by `--mid-job-advance` tokens (the cache is
+        # written by the steps that follow; what the history holds does not change what the step costs)
+        mid = None
+        if args.mid_job_advance > 0:
+            session.entry.cache.seq_lens.add_(args.mid_job_advance)
+            session.poll(steps=2)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            finished = session.poll(steps=args.steps)
+            torch.cuda.synchronize()
+            mid_elapsed = time.perf_counter() - t0
+            assert not finished, "no sequence may finish inside the timed region"
+            mid_attn_s, mid_attn_bytes, mid_tokens = time_decode_attention(engine, session, max(args.attn_samples // 2, 2))
+            mid = (mid_elapsed, mid_attn_s, mid_attn_bytes, mid_tokens)
         calibration_copy()
         gemms = time_gemms(engine) if fp8_requested(args) else None
-        kv_token = 6 * (attn_bytes - 2 * args.batch * 32 * 64 * 2) // max(ctx_tokens, 1)
     fp8 = args.precision == "fp8"
     weights = sum(w.numel() for w in set(engine.weights.linear_matrices())) * (1 if fp8 else 2)
-    step_bytes = weights + ctx_tokens * kv_token + args.batch * 122880 * 2 + args.batch * cfg.vocab_size * 2 * 2
+    fixed_bytes = weights + args.batch * 122880 * 2 + args.batch * cfg.vocab_size * 2 * 2
+    step_bytes = fixed_bytes + ctx_tokens * kv_token
     ms_per_step = elapsed / args.steps * 1000
     achieved = attn_bytes / attn_s / 1e9
+    mid_job = None
+    if mid is not None:
+        mid_elapsed, mid_attn_s, mid_attn_bytes, mid_tokens = mid
+        mid_ms = mid_elapsed / args.steps * 1000
+        mid_bytes = fixed_bytes + mid_tokens * kv_token
+        mid_job = {"context_tokens": mid_tokens, "ms_per_step": round(mid_ms, 4),
+                   "tok_per_s": round(args.batch * args.steps / mid_elapsed, 1), "step_algorithmic_bytes": mid_bytes,
+                   "step_hbm_fraction": round(mid_bytes / (mid_ms / 1000) / 1e9 / HBM_PEAK_GBS, 4),
+                   "attention_us_per_call": round(mid_attn_s * 1e6, 2),
+                   "attention_GBps": round(mid_attn_bytes / mid_attn_s / 1e9, 1),
+                   "attention_frac": round(mid_attn_bytes / mid_attn_s / 1e9 / HBM_PEAK_GBS, 4)}
     line = {
         "metric": "decode output tok/s @256 ragged seqs, LFM2.5-1.2B FP8; % HBM roofline",
         "value": round(args.batch * args.steps / elapsed, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
@@ -530,8 +562,10 @@ def main():
                                f"{'' if args.top_k == 0 and args.top_p == 1.0 else f', top-k {args.top_k}, top-p {args.top_p}'}, "
                                f"max_model_len {args.max_model_len}, HIP-graph decode step",
                    "context_tokens": ctx_tokens, "prefill_tok_per_s": round(sum(map(len, prompts)) / prefill_s, 1),
+                   "prefill_chunks": prefill_plan.get("chunks"), "prefill_chunk_fill": round(prefill_plan.get("fill", 0.0), 4),
                    "gemm": gemms, "step_algorithmic_bytes": step_bytes,
-                   "step_hbm_fraction": round(step_bytes / (ms_per_step / 1000) / 1e9 / HBM_PEAK_GBS, 4)},
+                   "step_hbm_fraction": round(step_bytes / (ms_per_step / 1000) / 1e9 / HBM_PEAK_GBS, 4),
+                   "mid_job": mid_job},
         "roofline": {"kernel": "decode_attn_mfma_kernel + decode_combine_row_kernel (one ragged GQA decode-attention call, e4m3 KV, rows quantised for the W8A8 out projection as in the decode step)"
                                if fp8 else "decode_attn_mfma_kernel + decode_combine_row_kernel (one ragged GQA decode-attention call, bf16 KV)",
                      "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",

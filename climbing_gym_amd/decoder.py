@@ -204,20 +204,19 @@ class LFM25HIPDecoder:
         return CompactDecodeGraph(graph, slots, (tokens, positions, active))
 
     def _select_graph(self, entry: _DecodeGraph, live_slots):
-        """Smallest power-of-two compute batch (>= 16) that holds the live rows (lfm25_cuda.py:194-209)."""
-        maximum = entry.input_tokens.numel()
-        if not self.adaptive_batching or maximum <= 16:
-            return entry.graph, maximum
-        size = 16
-        while size < len(live_slots):
-            size *= 2
-        if size >= maximum:
-            return entry.graph, maximum
-        if size not in entry.compact_graphs:
-            entry.compact_graphs[size] = self.capture_compact(entry, size)
-        compact = entry.compact_graphs[size]
-        compact.set_slots(live_slots)
-        return compact.graph, size
+        """(graph, compute rows) for the rows that are live: with adaptive batching the smallest power of two that holds
+        them, 16 at least, as a compact graph over the same cache; the full graph when that is no smaller than it
+        (lfm25_cuda.py:194-209)."""
+        rows = entry.input_tokens.numel()
+        if self.adaptive_batching:
+            width = max(16, 1 << max(len(live_slots) - 1, 0).bit_length())
+            if width < rows:
+                compact = entry.compact_graphs.get(width)
+                if compact is None:
+                    compact = entry.compact_graphs[width] = self.capture_compact(entry, width)
+                compact.set_slots(live_slots)
+                return compact.graph, width
+        return entry.graph, rows
 
     # ------------------------------------------------------------------ generate
     @torch.inference_mode()

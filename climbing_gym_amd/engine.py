@@ -5,8 +5,8 @@ Public surface and argument meaning follow the reference's `LFM25Engine`
 by design and do not change results beyond GEMM rounding:
 
 * prefill runs a *packed* (varlen) batch through the same fused kernels as decode instead of a
-  right-padded batch through eager torch ops; the chunk planner that bounds a prefill by
-  `max_prefill_tokens` is the reference's (lfm25_engine.py:646-665), so chunks are the same;
+  right-padded batch through eager torch ops; `max_prefill_tokens` (lfm25_engine.py:646-665) bounds the real
+  tokens of a chunk, since a packed chunk has no padding to count;
 * the engine only exists on the GPU in bf16: there is no eager CPU path in this package.
 """
 from __future__ import annotations
@@ -73,8 +73,9 @@ class LFM25GenerationOutput:
 
 
 def plan_prefill_chunks(lengths: Sequence[int], budget: int):
-    """Contiguous groups (start, end, padded width) with (count * longest) <= budget; a group always takes
-    its first prompt (lfm25_engine.py:646-665)."""
+    """The reference's planner for right-padded chunks: contiguous groups (start, end, padded width) with
+    (count * longest) <= budget; a group always takes its first prompt (lfm25_engine.py:646-665).  This engine packs
+    its chunks and plans them with `plan_packed_chunks`; the padded rule is kept for callers that size padded batches."""
     groups, start, total = [], 0, len(lengths)
     while start < total:
         end, width = start, 0
@@ -84,6 +85,21 @@ def plan_prefill_chunks(lengths: Sequence[int], budget: int):
                 break
             width, end = widest, end + 1
         groups.append((start, end, width))
+        start = end
+    return groups
+
+
+def plan_packed_chunks(lengths: Sequence[int], budget: int):
+    """Contiguous groups (start, end) of whole prompts whose token counts add up to at most `budget`; a group always
+    takes its first prompt.  A packed (varlen) chunk carries no padding, so the budget of lfm25_engine.py:646-665 is
+    spent on real tokens: with prompts of 256 to 2048 tokens a 4096-token chunk holds about 3500 instead of 2660."""
+    groups, start, total = [], 0, len(lengths)
+    while start < total:
+        end, used = start + 1, lengths[start]
+        while end < total and used + lengths[end] <= budget:
+            used += lengths[end]
+            end += 1
+        groups.append((start, end))
         start = end
     return groups
 
@@ -126,6 +142,7 @@ class LFM25Engine:
         self._scaling = cfg.head_dim ** -0.5
         self._cuda_decoder = None
         self.policy_version = 0
+        self.last_prefill: dict = {}   # chunk count, tokens and fill of the latest prefill() call
         # fp32 rotary tables [max_model_len, D/2] (lfm25_engine.py:1004-1012)
         inv = 1.0 / (cfg.rope_theta ** (torch.arange(0, cfg.head_dim, 2, dtype=torch.float32, device=self.device) / cfg.head_dim))
         angles = torch.arange(self.max_model_len, dtype=torch.float32, device=self.device)[:, None] * inv[None, :]
@@ -355,28 +372,20 @@ class LFM25Engine:
         return logits
 
     # ------------------------------------------------------------------ prefill
-    def _prefill_packed(self, cache: LFM25HybridCache, tokens, lengths: Sequence[int], fp8, lengths_device=None):
-        """Forward a packed batch of whole prompts into cache rows 0..n-1; returns next-token logits [n, V].
-        `lengths_device` (int32 on the device, the same numbers as `lengths`) lets a caller with many chunks copy all
-        lengths to the device once: a host-to-device copy per chunk waits for the stream and stops the host from
-        running ahead of the GPU."""
+    def _prefill_packed(self, cache: LFM25HybridCache, tokens, lengths: Sequence[int], fp8, lengths_device, slots, logits_out):
+        """Forward a packed batch of whole prompts; sequence i goes to cache slot `slots[i]` (int32 on the device) and
+        its next-token logits to row `slots[i]` of `logits_out`.  `lengths_device` holds the same numbers as `lengths`
+        on the device: a caller with many chunks copies all lengths once, because a host-to-device copy per chunk waits
+        for the stream and stops the host from running ahead of the GPU."""
         cfg = self.config
         count, total, longest = len(lengths), int(sum(lengths)), int(max(lengths))
-        if count > cache.max_slots:
-            raise RuntimeError("cache slot capacity exceeded")
         if longest > cache.max_seq_len:
             raise RuntimeError("cache capacity exceeded")
         if longest > self.max_model_len:
             raise RuntimeError("position exceeds engine max_model_len")
-        if lengths_device is None:
-            cu_host = torch.zeros(count + 1, dtype=torch.int32)
-            cu_host[1:] = torch.tensor(lengths, dtype=torch.int32).cumsum(0)
-            cu = cu_host.to(self.device)
-        else:
-            cu = torch.zeros(count + 1, device=self.device, dtype=torch.int32)
-            cu[1:] = lengths_device.cumsum(0)
+        cu = torch.zeros(count + 1, device=self.device, dtype=torch.int32)
+        cu[1:] = lengths_device.cumsum(0)
         seq_of_token, positions = ops.build_token_map(cu, total)
-        slots = torch.arange(count, device=self.device, dtype=torch.int32)
 
         def attention_op(op, qkv):
             q, k, v = ops.prepare_qkv(qkv, op.q_norm_weight, op.k_norm_weight, self._rope_cos, self._rope_sin, positions,
@@ -393,36 +402,49 @@ class LFM25Engine:
 
         hidden, residual = self._backbone(tokens, attention_op, conv_op, fp8)
         last = (cu[1:] - 1).long()
-        logits = self._head(hidden.index_select(0, last), residual.index_select(0, last), fp8)
-        cache.seq_lens[:count].copy_(cu[1:] - cu[:-1])
-        return logits
+        # the head projection places each sequence's logits in its slot's row of the destination
+        self._head(hidden.index_select(0, last), residual.index_select(0, last), fp8, ops.RowPlacement(logits_out, slots))
+        cache.seq_lens.index_copy_(0, slots.long(), lengths_device)
 
     @torch.inference_mode()
     def prefill(self, input_ids, cu_seqlens, max_seqlen: int, *, max_cache_len: int | None = None,
                 cache: LFM25HybridCache | None = None, max_prefill_tokens: int | None = None,
-                logits_buffer: torch.Tensor | None = None) -> LFM25PrefixBatch:
+                logits_buffer: torch.Tensor | None = None, slots: Sequence[int] | None = None) -> LFM25PrefixBatch:
+        """Prefill whole prompts (lfm25_engine.py:605-684) as packed chunks of at most `max_prefill_tokens` real tokens.
+        Without `slots`, prompt i fills cache slot i of a cache with exactly that many slots, as in the reference.
+        With `slots` (distinct slot indices, one per prompt) the prompts go to those slots of a larger cache and their
+        logits to the same rows of `logits_buffer` ([cache slots, vocab]); the other slots are not touched."""
         input_ids = input_ids.to(device=self.device, dtype=torch.long).reshape(-1)
-        cu_host = cu_seqlens.to(device="cpu", dtype=torch.long).reshape(-1)
-        if cu_host.numel() < 2:
+        bounds = cu_seqlens.to(device="cpu", dtype=torch.long).reshape(-1)
+        if bounds.numel() < 2:
             raise ValueError("cu_seqlens must contain at least [0, total_tokens]")
-        if int(cu_host[0]) != 0:
+        if int(bounds[0]) != 0:
             raise ValueError("cu_seqlens must start at 0")
-        if int(cu_host[-1]) != int(input_ids.numel()):
+        if int(bounds[-1]) != int(input_ids.numel()):
             raise ValueError("cu_seqlens[-1] must equal input_ids.numel()")
-        lengths = (cu_host[1:] - cu_host[:-1]).tolist()
+        offsets = bounds.tolist()
+        lengths = [b - a for a, b in zip(offsets[:-1], offsets[1:])]
         if min(lengths) <= 0:
             raise ValueError("empty prompts are not supported")
         if max(lengths) > int(max_seqlen):
             raise ValueError("max_seqlen is smaller than at least one prompt")
+        if max_prefill_tokens is not None and max_prefill_tokens <= 0:
+            raise ValueError("max_prefill_tokens must be positive")
         count = len(lengths)
         cache_len = int(max_cache_len or max_seqlen)
         if cache is None:
+            if slots is not None:
+                raise ValueError("slots address an existing cache")
             cache = self._empty_cache(max_slots=count, max_seq_len=cache_len)
-        elif cache.max_slots != count or cache.max_seq_len < cache_len:
+        elif cache.max_seq_len < cache_len or (slots is None and cache.max_slots != count):
             raise ValueError("destination cache does not fit the prompt batch")
-        if max_prefill_tokens is not None and max_prefill_tokens <= 0:
-            raise ValueError("max_prefill_tokens must be positive")
-        shape = (count, self.config.vocab_size)
+        if slots is None:
+            slot_list = list(range(count))
+        else:
+            slot_list = [int(slot) for slot in slots]
+            if len(slot_list) != count or len(set(slot_list)) != count or min(slot_list) < 0 or max(slot_list) >= cache.max_slots:
+                raise ValueError("slots must be distinct cache slots, one per prompt")
+        shape = (cache.max_slots, self.config.vocab_size)
         if logits_buffer is None:
             logits_out = torch.empty(shape, device=self.device, dtype=self.dtype)
         else:
@@ -431,18 +453,21 @@ class LFM25Engine:
             logits_out = logits_buffer
         budget = MAX_PACKED_TOKENS if max_prefill_tokens is None else min(int(max_prefill_tokens), MAX_PACKED_TOKENS)
         fp8 = self._fp8()
-        offsets = cu_host.tolist()
-        lengths_device = torch.tensor(lengths, dtype=torch.int32).to(self.device)
+        # one upload for the whole call: lengths and destination slots
+        meta = torch.tensor([lengths, slot_list], dtype=torch.int32).to(self.device)
+        lengths_device, slots_device = meta[0], meta[1]
+        plan = plan_packed_chunks(lengths, budget)
         in_flight = []   # the host stays at most two chunks (a few hundred launches) ahead of the GPU
-        for start, end, _ in plan_prefill_chunks(lengths, budget):
-            logits = self._prefill_packed(cache.rows(start, end), input_ids[offsets[start]:offsets[end]], lengths[start:end], fp8,
-                                          lengths_device[start:end])
-            logits_out[start:end].copy_(logits)
+        for start, end in plan:
+            self._prefill_packed(cache, input_ids[offsets[start]:offsets[end]], lengths[start:end], fp8,
+                                 lengths_device[start:end], slots_device[start:end], logits_out)
             marker = torch.cuda.Event()
             marker.record()
             in_flight.append(marker)
             if len(in_flight) > 2:
                 in_flight.pop(0).synchronize()
+        self.last_prefill = {"chunks": len(plan), "tokens": offsets[-1], "budget": budget,
+                             "fill": offsets[-1] / (len(plan) * budget)}
         return LFM25PrefixBatch(cache, logits_out, lengths_device, input_ids)
 
     # ------------------------------------------------------------------ fork / decode_step
@@ -547,9 +572,9 @@ class LFM25Engine:
         result = [()] * len(sequences)
         order = sorted(range(len(sequences)), key=lambda i: len(sequences[i]))
         lengths = [len(sequences[i]) for i in order]
-        for start, end, width in plan_prefill_chunks(lengths, min(int(max_prefill_tokens), MAX_PACKED_TOKENS)):
+        for start, end in plan_packed_chunks(lengths, min(int(max_prefill_tokens), MAX_PACKED_TOKENS)):
             group = order[start:end]
-            cache = self._empty_cache(max_slots=len(group), max_seq_len=width)
+            cache = self._empty_cache(max_slots=len(group), max_seq_len=max(lengths[start:end]))
             tokens = torch.tensor([t for i in group for t in sequences[i]], device=self.device, dtype=torch.long)
             hidden = self._prefill_hidden(cache, tokens, [len(sequences[i]) for i in group], fp8)
             rows, targets, base = [], [], 0

@@ -1,19 +1,26 @@
-"""Continuous batching over one graph entry: admit, poll, resume, release, fork, snapshot.
+"""Continuous batching over one captured decode step: the stand-in for `LFM25GenerationSession`
+(lfm25_session.py:109-533) with its public methods, argument meanings, error texts and statistics keys.
 
-Mirrors `LFM25GenerationSession` of the reference (lfm25_session.py:109-533).  Row lifecycle: a finished
-request keeps every token except its last sampled one in the KV/conv cache; `pending[row]` says that
-token still has to be consumed.  The first step after `admit` leaves a fresh row inactive, so the sampler
-reads the prefill logits kept in the entry's logits buffer.
+How this one is built:
 
-All per-token state (lengths, limits, finish reasons, stop automaton state, RNG positions) lives in device
-tensors updated by the record kernel; the host reads `reasons` once per poll.
+* the per-row device state is one struct of tensors (`_RowTable`); an admission writes all of its rows with one
+  upload and one kernel (`lfm2_configure_rows`), whatever the number of requests;
+* a slot is a small host record (`_Slot`) with a generation counter; a continuation handle is valid while it is the
+  record's current lease, so "stale", "consumed" and "other session" are one comparison;
+* the flag "this row still owes the model its last sampled token" IS the graph's activity mask: the record kernel
+  writes it, the next replay reads it, and no copy runs between the two;
+* a whole admission is one packed prefill, whichever slots are free: the prefill kernels scatter every sequence to its
+  slot, so fragmented free slots cost nothing;
+* every row is drawn by the full-support sampler; rows that ask for top-k / top-p (an extension: the reference's
+  sessions refuse them, lfm25_session.py:217-218) are then redrawn by the filtered sampler with their own
+  temperature, k and p, so a request's tokens never depend on what its neighbours asked for.
 
-Beyond the reference, rows may use temperature/top-k/top-p sampling as long as every filtered row of the
-session shares one (top_k, top_p) pair; the draw then comes from the on-device filtered sampler.
+A finished request keeps every token except its last sampled one in the KV/conv cache; resuming it feeds that token
+(and any new suffix) one position per replay under a per-row mask.
 """
 from __future__ import annotations
 
-from contextlib import contextmanager
+import struct
 from dataclasses import dataclass
 from typing import Sequence
 
@@ -29,11 +36,13 @@ STAT_KEYS = ("prefilled_tokens", "resumed_prefix_tokens", "appended_tokens", "ad
              "decode_steps", "slot_refills", "peak_live_slots", "decode_row_steps", "reserved_row_steps",
              "adaptive_graph_captures", "forked_requests", "copied_prefix_tokens", "snapshot_prefilled_tokens",
              "snapshot_count", "peak_snapshots", "peak_snapshot_bytes")
+_SEED_MASK = (1 << 63) - 1
 
 
+# ---------------------------------------------------------------------------------------------- what callers hold
 @dataclass(frozen=True)
 class LFM25ContinuationHandle:
-    """Single-use lease on one session slot; invalid after release or close."""
+    """Single-use lease on one session slot; invalid after release, resume or close."""
     session: object
     slot: int
     version: int
@@ -52,466 +61,507 @@ class LFM25SessionResult:
 
 @dataclass(frozen=True)
 class LFM25PrefixSnapshot:
-    """Opaque immutable lease; the tensors belong to the session that made it."""
+    """Opaque immutable lease on a stored prefix; the tensors stay with the session that made it."""
     session: object
     identity: int
     policy_version: int
     prefix_token_ids: tuple
 
 
+# ---------------------------------------------------------------------------------------------- host-side records
 @dataclass
-class _Snapshot:
+class _Slot:
+    generation: int = 0                    # bumped every time the slot is configured or given back
+    prompt: tuple | None = None
+    sampling: LFM25SamplingConfig | None = None
+    lease: LFM25ContinuationHandle | None = None   # set once the result has been handed out
+    used_before: bool = False
+
+    @property
+    def busy(self) -> bool:
+        return self.prompt is not None
+
+    @property
+    def running(self) -> bool:
+        return self.prompt is not None and self.lease is None
+
+
+@dataclass
+class _StoredPrefix:
     lease: LFM25PrefixSnapshot
     cache: LFM25HybridCache
     logits: torch.Tensor
-    pending_token: int | None
-    seed: int
-    rng_position: int
-    stop_state: int
+    pending_token: int | None = None
+    seed: int = 0
+    rng_position: int = 0
+    stop_state: int = 0
+
+    def nbytes(self) -> int:
+        return self.cache.nbytes() + self.logits.numel() * self.logits.element_size()
 
 
-@dataclass
-class _Request:
-    prompt: tuple
-    sampling: LFM25SamplingConfig
-    version: int
-    delivered: bool = False
-    handle: LFM25ContinuationHandle | None = None
+class _RowTable:
+    """Device state of the session's rows, one column per field (the tensors of lfm25_session.py:150-165 plus the
+    per-row filter parameters)."""
+
+    def __init__(self, rows: int, new_tokens: int, head: int, pending: torch.Tensor, device):
+        column = lambda dtype: torch.zeros(rows, device=device, dtype=dtype)
+        self.lengths, self.limits, self.top_ks = column(torch.int32), column(torch.int32), column(torch.int32)
+        self.seeds, self.rng_positions = column(torch.int64), column(torch.int64)
+        self.stop_states, self.stop_offsets = column(torch.int64), column(torch.int64)
+        self.reasons = column(torch.int8)
+        self.alive, self.ignore_eos = column(torch.bool), column(torch.bool)
+        self.temperatures, self.top_ps = column(torch.float32), column(torch.float32)
+        self.pending = pending.zero_()     # the decode graph's activity mask
+        self.tokens = torch.empty((rows, new_tokens), device=device, dtype=torch.long)
+        self.logprobs = torch.empty((rows, new_tokens), device=device, dtype=torch.float32)
+        self.head_ids = torch.empty((rows, new_tokens, head), device=device, dtype=torch.int32) if head else None
+        self.head_logprobs = torch.empty((rows, new_tokens, head), device=device, dtype=torch.float32) if head else None
+        self.device = device
+
+    @staticmethod
+    def spec(slot: int, sampling: LFM25SamplingConfig, stop_offset: int, rng_position: int, stop_state: int) -> list:
+        """The eight words `lfm2_configure_rows` reads for one request."""
+        floats = struct.unpack("<q", struct.pack("<ff", float(sampling.temperature), float(sampling.top_p)))[0]
+        flags = int(bool(sampling.ignore_eos)) | (int(sampling.top_k if sampling.filtered else 0) << 8)
+        return [slot, sampling.max_new_tokens, sampling.seed & _SEED_MASK, rng_position, stop_state, stop_offset, flags, floats]
+
+    def write(self, specs: list) -> None:
+        ops.configure_rows(torch.tensor(specs, dtype=torch.int64).to(self.device), self)
+
+    def retire(self, slot: int) -> None:
+        self.alive[slot] = False
+        self.pending[slot] = False
 
 
+class _StopTables:
+    """One flat int32 table: entries 0..V-1 are the automaton that never stops; each distinct (stop table, stop ids)
+    pair appends its states x V entries, with stop ids marked 65536 in every state (lfm25_session.py:228-241)."""
+
+    def __init__(self, vocab: int, device):
+        self.vocab, self.device = vocab, device
+        self.flat = torch.zeros(vocab, device=device, dtype=torch.int32)
+        self._known: dict = {}
+
+    def offset(self, sampling: LFM25SamplingConfig) -> int:
+        if sampling.stop_table is None and not sampling.stop_token_ids:
+            return 0
+        key = (id(sampling.stop_table), tuple(sampling.stop_token_ids))
+        found = self._known.get(key)
+        if found is None:
+            states = (torch.zeros((1, self.vocab), dtype=torch.int32, device=self.device) if sampling.stop_table is None
+                      else sampling.stop_table.to(self.device).clone())
+            if sampling.stop_token_ids:
+                states[:, list(sampling.stop_token_ids)] = 65536
+            found = (self.flat.numel(), sampling.stop_table)   # holding the table keeps its id() from being reused
+            self.flat = torch.cat((self.flat, states.reshape(-1)))
+            self._known[key] = found
+        return found[0]
+
+
+class _PhaseClock:
+    """Optional GPU timing of the session's phases with event pairs, read once at the end."""
+
+    def __init__(self, enabled: bool):
+        self.enabled, self.spans = enabled, []
+
+    def __call__(self, phase: str):
+        return _PhaseSpan(self, phase)
+
+    def totals(self) -> dict:
+        if self.spans:
+            self.spans[-1][2].synchronize()
+        out: dict = {}
+        for phase, begin, end in self.spans:
+            out[f"{phase}_gpu_seconds"] = out.get(f"{phase}_gpu_seconds", 0.0) + begin.elapsed_time(end) / 1000
+        return out
+
+
+class _PhaseSpan:
+    def __init__(self, clock: _PhaseClock, phase: str):
+        self.clock, self.phase = clock, phase
+
+    def __enter__(self):
+        if self.clock.enabled:
+            self.begin = torch.cuda.Event(enable_timing=True)
+            self.begin.record()
+
+    def __exit__(self, *_):
+        if self.clock.enabled:
+            end = torch.cuda.Event(enable_timing=True)
+            end.record()
+            self.clock.spans.append((self.phase, self.begin, end))
+
+
+# ---------------------------------------------------------------------------------------------- the session
 class LFM25GenerationSession:
     @torch.inference_mode()
     def __init__(self, decoder, *, max_batch_size: int, max_new_tokens: int, cache_len: int | None = None,
                  behavior_topk: int = 0, profile_timings: bool = False):
         if decoder._active_session is not None:
             raise RuntimeError("A native generation session is already open")
-        if type(max_batch_size) is not int or max_batch_size <= 0:
-            raise ValueError("max_batch_size must be a positive integer")
-        if type(max_new_tokens) is not int or max_new_tokens <= 0:
-            raise ValueError("max_new_tokens must be a positive integer")
+        for name, value in (("max_batch_size", max_batch_size), ("max_new_tokens", max_new_tokens)):
+            if type(value) is not int or value <= 0:
+                raise ValueError(f"{name} must be a positive integer")
         engine = decoder.engine
         vocab = engine.config.vocab_size
         if type(behavior_topk) is not int or not 0 <= behavior_topk <= min(128, vocab):
             raise ValueError('behavior_topk must be an integer between 0 and min(vocab, 128)')
         self.decoder, self.engine = decoder, engine
         self.batch_size, self.max_new_tokens, self.behavior_topk = max_batch_size, max_new_tokens, behavior_topk
-        self.entry = decoder._get_graph(max_batch_size, cache_len or engine.max_model_len, masked=True)
-        self.entry.active.zero_()
-        self.entry.cache.seq_lens.zero_()
-        self.requests: list = [None] * max_batch_size
-        self.versions = [0] * max_batch_size
-        self.closed = False
         self.policy_version = engine.policy_version
-        self.profile_timings = profile_timings
-        self._snapshots: dict = {}
-        self._snapshot_ids = 0
-        self._events: list = []
-        self._filter = None  # (top_k, top_p) shared by filtered rows
-        device = engine.device
-        col = lambda dtype, fill=0: torch.full((max_batch_size,), fill, device=device, dtype=dtype)
-        self.lengths, self.limits = col(torch.int32), col(torch.int32)
-        self.rng_positions, self.seeds = col(torch.int64), col(torch.int64)
-        self.reasons = col(torch.int8)
-        self.alive, self.pending, self.ignore_eos = col(torch.bool), col(torch.bool), col(torch.bool)
-        self.temperatures = col(torch.float32)
-        self.stop_states, self.stop_offsets = col(torch.int64), col(torch.int64)
-        self.tokens = torch.empty((max_batch_size, max_new_tokens), device=device, dtype=torch.long)
-        self.logprobs = torch.empty((max_batch_size, max_new_tokens), device=device, dtype=torch.float32)
-        self.head_ids = (torch.empty((max_batch_size, max_new_tokens, behavior_topk), device=device, dtype=torch.int32)
-                         if behavior_topk else None)
-        self.head_logprobs = torch.empty_like(self.head_ids, dtype=torch.float32) if behavior_topk else None
+        self.closed = False
+        self.entry = decoder._get_graph(max_batch_size, cache_len or engine.max_model_len, masked=True)
+        self.entry.cache.seq_lens.zero_()
+        self.rows = _RowTable(max_batch_size, max_new_tokens, behavior_topk, self.entry.active, engine.device)
+        self.slots = [_Slot() for _ in range(max_batch_size)]
+        self.stops = _StopTables(vocab, engine.device)
         self.sampler = ops.RowSampler(self.entry.logits)
-        self.stop_table = torch.zeros(vocab, device=device, dtype=torch.int32)
-        self._stop_tables: dict = {}
-        self.stats = {key: 0 for key in STAT_KEYS}
+        self.clock = _PhaseClock(profile_timings)
+        self._stored: dict = {}
+        self._stored_ids = 0
+        self._filtered_rows: set = set()
+        self.stats: dict = dict.fromkeys(STAT_KEYS, 0)
         self.stats["decode_batches"] = {}
         decoder._active_session = self
 
-    # ------------------------------------------------------------------ guards
-    def _check_open(self):
-        if self.closed or self.decoder._active_session is not self or self.engine._cuda_decoder is not self.decoder:
+    # ------------------------------------------------------------------ state checks
+    def _require_open(self) -> None:
+        mine = self.decoder._active_session is self and self.engine._cuda_decoder is self.decoder
+        if self.closed or not mine:
             raise RuntimeError("Native generation session is closed")
         if self.engine.policy_version != self.policy_version:
             raise ValueError('Session cache belongs to another policy version')
 
-    @contextmanager
-    def _timed(self, phase):
-        if not self.profile_timings:
-            yield
-            return
-        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        begin.record()
-        try:
-            yield
-        finally:
-            end.record()
-            self._events.append((phase, begin, end))
+    def timing_stats(self) -> dict:
+        """GPU seconds per phase (`prefill`, `cache_copy`, `append`), resolved once, outside the hot loop."""
+        return self.clock.totals()
 
-    def timing_stats(self):
-        """GPU seconds per phase, resolved once at the end (outside the hot loop)."""
-        if self._events:
-            self._events[-1][2].synchronize()
-        totals: dict = {}
-        for phase, begin, end in self._events:
-            key = phase + '_gpu_seconds'
-            totals[key] = totals.get(key, 0.0) + begin.elapsed_time(end) / 1000
-        return totals
+    def _violations(self, prompt, sampling: LFM25SamplingConfig):
+        """(broken, message) for every rule a request must meet, in checking order; evaluated lazily, so a later rule
+        may rely on the earlier ones."""
+        vocab, table = self.engine.config.vocab_size, sampling.stop_table
+        yield not prompt, "Empty prompts are not supported"
+        yield sampling.behavior_topk > self.behavior_topk, "Request behavior head exceeds the session reservation"
+        # three C-level passes over the ids instead of a Python loop
+        yield (set(map(type, prompt)) != {int} or min(prompt) < 0 or max(prompt) >= vocab), "Prompt token outside the model vocabulary"
+        yield sampling.max_new_tokens > self.max_new_tokens, "Request exceeds the session generation buffer"
+        yield (len(prompt) + sampling.max_new_tokens > self.entry.cache.max_seq_len), "Request exceeds reserved session context capacity"
+        yield (sampling.repetition_penalty != 1.0,
+               "Sessions support greedy, full-support and top-k/top-p sampling without repetition penalties")
+        yield (bool(sampling.stop_token_sequences),
+               "Sessions use stop_token_ids or stop_table; encode string stops with build_stop_table")
+        yield any(not 0 <= token < vocab for token in sampling.stop_token_ids), "Stop token outside the model vocabulary"
+        yield (table is not None and (table.ndim != 2 or table.size(1) != vocab or table.dtype != torch.int32),
+               "stop_table must be an int32 state-by-vocabulary table")
 
-    def _validate(self, prompt, sampling):
-        vocab = self.engine.config.vocab_size
-        if sampling.behavior_topk > self.behavior_topk:
-            raise ValueError('Request behavior head exceeds the session reservation')
-        if not prompt:
-            raise ValueError("Empty prompts are not supported")
-        if set(map(type, prompt)) != {int} or min(prompt) < 0 or max(prompt) >= vocab:   # C-level passes over the ids
-            raise ValueError("Prompt token outside the model vocabulary")
-        if len(prompt) + sampling.max_new_tokens > self.entry.cache.max_seq_len:
-            raise ValueError("Request exceeds reserved session context capacity")
-        if sampling.max_new_tokens > self.max_new_tokens:
-            raise ValueError("Request exceeds the session generation buffer")
-        if sampling.repetition_penalty != 1.0:
-            raise ValueError("Sessions support greedy/full-support/filtered sampling without repetition penalties")
-        if sampling.filtered and self._filter not in (None, (sampling.top_k, sampling.top_p)):
-            raise ValueError("Filtered rows of one session must share top_k and top_p")
-        if sampling.stop_token_sequences:
-            raise ValueError("Sessions use stop_token_ids or stop_table; encode string stops with build_stop_table")
-        if any(not 0 <= t < vocab for t in sampling.stop_token_ids):
-            raise ValueError("Stop token outside the model vocabulary")
-        table = sampling.stop_table
-        if table is not None and (table.ndim != 2 or table.size(1) != vocab or table.dtype != torch.int32):
-            raise ValueError("stop_table must be an int32 state-by-vocabulary table")
+    def _validate(self, prompt, sampling: LFM25SamplingConfig) -> None:
+        for broken, message in self._violations(prompt, sampling):
+            if broken:
+                raise ValueError(message)
 
-    def _stop_offset(self, sampling) -> int:
-        """Offset of the request's automaton inside the flat table; entry 0..V-1 is the empty automaton."""
-        if sampling.stop_table is None and not sampling.stop_token_ids:
-            return 0
-        key = (id(sampling.stop_table), sampling.stop_token_ids)
-        if key not in self._stop_tables:
-            vocab, device = self.engine.config.vocab_size, self.engine.device
-            table = (torch.zeros((1, vocab), dtype=torch.int32, device=device) if sampling.stop_table is None
-                     else sampling.stop_table.to(device).clone())
-            if sampling.stop_token_ids:
-                table[:, list(sampling.stop_token_ids)] = 65536
-            offset = self.stop_table.numel()
-            self.stop_table = torch.cat((self.stop_table, table.reshape(-1)))
-            self._stop_tables[key] = (offset, sampling.stop_table)  # keep the source alive: ids must stay unique
-        return self._stop_tables[key][0]
+    def _claim(self, wanted, count: int, purpose: str) -> list:
+        """`count` free slots: the lowest ones, or exactly the requested ones."""
+        if wanted is None:
+            chosen = [i for i, slot in enumerate(self.slots) if not slot.busy][:count]
+        else:
+            chosen = [int(i) for i in wanted]
+        ok = (len(chosen) == count and len(set(chosen)) == count
+              and all(0 <= i < self.batch_size and not self.slots[i].busy for i in chosen))
+        if not ok:
+            raise ValueError(f"{purpose} requires distinct free session slots")
+        return chosen
 
-    def _configure(self, slot, prompt, sampling, *, rng_position=0, stop_state=0):
-        self._configure_many([(slot, prompt, sampling)], rng_position=rng_position, stop_state=stop_state)
+    def _start(self, work, *, carried=None) -> None:
+        """Make (slot, prompt, sampling) the running request of each slot: host records, then every device column of
+        every row in one launch.  `carried[slot]` = (random-stream position, stop state) for rows that keep them."""
+        specs = []
+        for index, prompt, sampling in work:
+            slot = self.slots[index]
+            slot.generation += 1
+            slot.prompt, slot.sampling, slot.lease, slot.used_before = tuple(prompt), sampling, None, True
+            (self._filtered_rows.add if sampling.filtered else self._filtered_rows.discard)(index)
+            position, stop_state = (0, 0) if carried is None else carried[index]
+            specs.append(_RowTable.spec(index, sampling, self.stops.offset(sampling), position, stop_state))
+        self.rows.write(specs)
+        self.stats["peak_live_slots"] = max(self.stats["peak_live_slots"], sum(slot.busy for slot in self.slots))
 
-    def _configure_many(self, work, *, rng_position=0, stop_state=0):
-        """Per-row state of newly admitted (slot, prompt, sampling) requests: one indexed write per state tensor for
-        the whole group (a write per row and tensor is eleven tiny launches per request)."""
-        for slot, prompt, sampling in work:
-            self.versions[slot] += 1
-            self.requests[slot] = _Request(tuple(prompt), sampling, self.versions[slot])
-            if sampling.filtered:
-                self._filter = (sampling.top_k, sampling.top_p)
-        samplings = [sampling for _, _, sampling in work]
-        columns = ((self.lengths, [0] * len(work)), (self.reasons, [0] * len(work)),
-                   (self.stop_states, [stop_state] * len(work)), (self.rng_positions, [rng_position] * len(work)),
-                   (self.limits, [s.max_new_tokens for s in samplings]),
-                   (self.seeds, [s.seed & 0x7FFFFFFFFFFFFFFF for s in samplings]),
-                   (self.temperatures, [s.temperature for s in samplings]), (self.ignore_eos, [s.ignore_eos for s in samplings]),
-                   (self.stop_offsets, [self._stop_offset(s) for s in samplings]), (self.alive, [True] * len(work)),
-                   (self.pending, [False] * len(work)))
-        if len(work) == 1:
-            slot = work[0][0]
-            for tensor, values in columns:
-                tensor[slot] = values[0]
-            return
-        index = torch.tensor([slot for slot, _, _ in work], dtype=torch.long).to(self.lengths.device)
-        for tensor, values in columns:
-            tensor[index] = torch.tensor(values, dtype=tensor.dtype).to(tensor.device)
-
-    def _free_slots(self):
-        return [i for i, r in enumerate(self.requests) if r is None]
-
-    def _live_count(self):
-        return sum(r is not None for r in self.requests)
-
-    def _pick_slots(self, slots, count, what):
-        free = self._free_slots()
-        slots = list(free[:count] if slots is None else slots)
-        if len(slots) != count or len(set(slots)) != len(slots) or any(s not in free for s in slots):
-            raise ValueError(f"{what} requires distinct free session slots")
-        return slots
+    def _graph_for(self, rows):
+        known = len(self.entry.compact_graphs)
+        graph, width = self.decoder._select_graph(self.entry, rows)
+        self.stats["adaptive_graph_captures"] += len(self.entry.compact_graphs) - known
+        return graph, width
 
     # ------------------------------------------------------------------ admission
     @torch.inference_mode()
     def admit(self, prompts: Sequence[Sequence[int]], samplings: Sequence[LFM25SamplingConfig], *,
               slots: Sequence[int] | None = None) -> list:
-        self._check_open()
+        self._require_open()
         if len(prompts) != len(samplings):
             raise ValueError("One sampling configuration is required per prompt")
-        slots = self._pick_slots(slots, len(prompts), "Admission")
-        work = sorted(zip(slots, prompts, samplings), key=lambda item: item[0])
-        for _, prompt, sampling in work:
+        chosen = self._claim(slots, len(prompts), "Admission")
+        for prompt, sampling in zip(prompts, samplings):
             self._validate(prompt, sampling)
-        # runs of consecutive slots prefill straight into views of the session cache
-        begin = 0
-        while begin < len(work):
-            end = begin + 1
-            while end < len(work) and work[end][0] == work[end - 1][0] + 1:
-                end += 1
-            first, last = work[begin][0], work[end - 1][0] + 1
-            flat = flatten_token_batches([list(p) for _, p, _ in work[begin:end]], device=self.engine.device)
-            with self._timed('prefill'):
-                self.engine.prefill(*flat, cache=self.entry.cache.rows(first, last),
-                                    max_prefill_tokens=self.decoder.max_prefill_tokens,
-                                    logits_buffer=self.entry.logits[first:last])
-            begin = end
-        for slot, prompt, sampling in work:
-            self.stats['slot_refills'] += int(self.versions[slot] > 0)
-            self.stats['prefilled_tokens'] += len(prompt)
-            self.stats['admitted_requests'] += 1
-        self._configure_many(work)
-        self.stats['peak_live_slots'] = max(self.stats['peak_live_slots'], self._live_count())
-        return slots
+        if not chosen:
+            return chosen
+        refills = sum(self.slots[i].used_before for i in chosen)
+        flat, bounds, longest = flatten_token_batches(prompts, device=self.engine.device)
+        with self.clock("prefill"):
+            # one packed prefill for the whole admission: each sequence lands in its own slot of the session cache
+            self.engine.prefill(flat, bounds, longest, cache=self.entry.cache, slots=chosen, logits_buffer=self.entry.logits,
+                                max_prefill_tokens=self.decoder.max_prefill_tokens)
+        self.stats["slot_refills"] += refills
+        self.stats["prefilled_tokens"] += int(flat.numel())
+        self.stats["admitted_requests"] += len(chosen)
+        self._start(list(zip(chosen, prompts, samplings)))
+        return chosen
 
-    # ------------------------------------------------------------------ snapshots and forks
-    def _remember(self, prompt, cache, logits, pending_token=None, seed=0, rng_position=0, stop_state=0):
-        self._snapshot_ids += 1
-        lease = LFM25PrefixSnapshot(self, self._snapshot_ids, self.policy_version, tuple(prompt))
-        self._snapshots[lease.identity] = _Snapshot(lease, cache, logits, pending_token, seed, rng_position, stop_state)
-        held = sum(s.cache.nbytes() + s.logits.numel() * s.logits.element_size() for s in self._snapshots.values())
-        self.stats['snapshot_count'] += 1
-        self.stats['peak_snapshots'] = max(self.stats['peak_snapshots'], len(self._snapshots))
-        self.stats['peak_snapshot_bytes'] = max(self.stats['peak_snapshot_bytes'], held)
-        return lease
+    # ------------------------------------------------------------------ stored prefixes
+    def _store(self, prefix: _StoredPrefix) -> LFM25PrefixSnapshot:
+        self._stored[prefix.lease.identity] = prefix
+        self.stats["snapshot_count"] += 1
+        self.stats["peak_snapshots"] = max(self.stats["peak_snapshots"], len(self._stored))
+        self.stats["peak_snapshot_bytes"] = max(self.stats["peak_snapshot_bytes"], sum(p.nbytes() for p in self._stored.values()))
+        return prefix.lease
+
+    def _new_lease(self, tokens) -> LFM25PrefixSnapshot:
+        self._stored_ids += 1
+        return LFM25PrefixSnapshot(self, self._stored_ids, self.policy_version, tuple(tokens))
+
+    def _lookup(self, snapshot: LFM25PrefixSnapshot) -> _StoredPrefix:
+        self._require_open()
+        if snapshot.policy_version != self.engine.policy_version:
+            raise ValueError('Snapshot belongs to another policy version')
+        stored = self._stored.get(snapshot.identity) if snapshot.session is self else None
+        if stored is None or stored.lease is not snapshot:
+            raise ValueError('Snapshot is released or belongs to another session')
+        return stored
 
     @torch.inference_mode()
     def prefill_snapshot(self, prompt: Sequence[int]) -> LFM25PrefixSnapshot:
-        """Prefill one exact prefix once under the current weights."""
-        self._check_open()
+        """Prefill one exact prefix once under the current weights, outside the session's slots."""
+        self._require_open()
         prompt = tuple(prompt)
         self._validate(prompt, LFM25SamplingConfig(max_new_tokens=1))
         cache = self.engine._empty_cache(max_slots=1, max_seq_len=len(prompt), fp8_kv=self.entry.cache.fp8)
-        with self._timed('prefill'):
-            prefix = self.engine.prefill(*flatten_token_batches([list(prompt)], device=self.engine.device), cache=cache,
-                                         max_prefill_tokens=self.decoder.max_prefill_tokens)
-        self.stats['prefilled_tokens'] += len(prompt)
-        self.stats['snapshot_prefilled_tokens'] += len(prompt)
-        return self._remember(prompt, cache, prefix.next_token_logits)
+        with self.clock("prefill"):
+            done = self.engine.prefill(*flatten_token_batches([prompt], device=self.engine.device), cache=cache,
+                                       max_prefill_tokens=self.decoder.max_prefill_tokens)
+        self.stats["prefilled_tokens"] += len(prompt)
+        self.stats["snapshot_prefilled_tokens"] += len(prompt)
+        return self._store(_StoredPrefix(self._new_lease(prompt), cache, done.next_token_logits))
 
     @torch.inference_mode()
     def snapshot(self, handle: LFM25ContinuationHandle) -> LFM25PrefixSnapshot:
-        """Copy the valid KV bytes/scales, conv state, logits and the pending token of a delivered row."""
-        request = self._request_for(handle)
-        length = len(handle.prefix_token_ids) - 1
-        if int(self.entry.cache.seq_lens[handle.slot]) != length:
+        """Copy a delivered row: the valid part of its KV bytes and scales, its conv state, its logits and the token it
+        still owes the model."""
+        slot = self._leased(handle)
+        cached = len(handle.prefix_token_ids) - 1
+        if int(self.entry.cache.seq_lens[handle.slot]) != cached:
             raise ValueError('Cached position does not match the pending-token prefix')
-        with self._timed('cache_copy'):
-            src = self.entry.cache.rows(handle.slot, handle.slot + 1)
-            part = lambda t: None if t is None else t[:, :, :length].clone()
-            cache = LFM25HybridCache(part(src.k_cache), part(src.v_cache), src.conv_state.clone(), src.seq_lens.clone(),
-                                     part(src.k_scales), part(src.v_scales))
+        with self.clock("cache_copy"):
+            row = self.entry.cache.rows(handle.slot, handle.slot + 1)
+            history = [None if t is None else t[:, :, :cached].clone() for t in (row.k_cache, row.v_cache, row.k_scales, row.v_scales)]
+            copy = LFM25HybridCache(history[0], history[1], row.conv_state.clone(), row.seq_lens.clone(), history[2], history[3])
             logits = self.entry.logits[handle.slot:handle.slot + 1].clone()
-        return self._remember(handle.prefix_token_ids, cache, logits, handle.prefix_token_ids[-1], request.sampling.seed,
-                              int(self.rng_positions[handle.slot]), int(self.stop_states[handle.slot]))
+        state = self.rows
+        return self._store(_StoredPrefix(self._new_lease(handle.prefix_token_ids), copy, logits, handle.prefix_token_ids[-1],
+                                         slot.sampling.seed, int(state.rng_positions[handle.slot]), int(state.stop_states[handle.slot])))
 
-    def _snapshot_for(self, snapshot):
-        self._check_open()
-        if snapshot.policy_version != self.engine.policy_version:
-            raise ValueError('Snapshot belongs to another policy version')
-        state = self._snapshots.get(snapshot.identity)
-        if snapshot.session is not self or state is None or state.lease is not snapshot:
-            raise ValueError('Snapshot is released or belongs to another session')
-        return state
+    def release_snapshot(self, snapshot: LFM25PrefixSnapshot) -> None:
+        del self._stored[self._lookup(snapshot).lease.identity]
 
     @torch.inference_mode()
     def fork(self, snapshot: LFM25PrefixSnapshot, samplings: Sequence[LFM25SamplingConfig], *,
              slots: Sequence[int] | None = None) -> list:
-        """Start independent children of a snapshot in free rows without any prefill."""
-        state = self._snapshot_for(snapshot)
-        slots = self._pick_slots(slots, len(samplings), "Fork")
+        """Start independent children of a stored prefix in free slots without any prefill."""
+        stored = self._lookup(snapshot)
+        chosen = self._claim(slots, len(samplings), "Fork")
         for sampling in samplings:
             self._validate(snapshot.prefix_token_ids, sampling)
-        length = state.cache.max_seq_len
-        with self._timed('cache_copy'):
-            for slot in slots:
-                dst = self.entry.cache.rows(slot, slot + 1)
-                for target, source in ((dst.k_cache, state.cache.k_cache), (dst.v_cache, state.cache.v_cache),
-                                       (dst.k_scales, state.cache.k_scales), (dst.v_scales, state.cache.v_scales)):
-                    if target is not None:
-                        _copy_bytes(target[:, :, :length], source)
-                dst.conv_state.copy_(state.cache.conv_state)
-                dst.seq_lens.copy_(state.cache.seq_lens)
-                self.entry.logits[slot].copy_(state.logits[0])
-        if slots and state.pending_token is not None:
-            # the snapshot's last sampled token is not in the cache yet: consume it once in every child
-            with self._timed('append'):
-                keep = self.entry.input_tokens.clone()
-                self.entry.input_tokens[slots] = state.pending_token
-                self.entry.active.zero_()
-                self.entry.active[slots] = True
-                self._select_graph(slots)[0].replay()
-                self.entry.input_tokens.copy_(keep)
-        for slot, sampling in zip(slots, samplings):
-            self.stats['slot_refills'] += int(self.versions[slot] > 0)
-            self._configure(slot, snapshot.prefix_token_ids, sampling)
-        self.stats['forked_requests'] += len(slots)
-        self.stats['copied_prefix_tokens'] += length * len(slots)
-        self.stats['peak_live_slots'] = max(self.stats['peak_live_slots'], self._live_count())
-        return slots
-
-    def release_snapshot(self, snapshot: LFM25PrefixSnapshot) -> None:
-        self._snapshot_for(snapshot)
-        del self._snapshots[snapshot.identity]
+        if not chosen:
+            return chosen
+        cached = stored.cache.max_seq_len
+        where = torch.tensor(chosen, device=self.engine.device)
+        target, source = self.entry.cache, stored.cache
+        with self.clock("cache_copy"):
+            for mine, theirs in ((target.k_cache, source.k_cache), (target.v_cache, source.v_cache),
+                                 (target.k_scales, source.k_scales), (target.v_scales, source.v_scales)):
+                if mine is not None:   # bytes as they are (an e4m3 cache is never dequantised), broadcast over the children
+                    _raw(mine)[:, where, :cached] = _raw(theirs)
+            target.conv_state[:, where] = source.conv_state
+            target.seq_lens[where] = source.seq_lens
+            self.entry.logits[where] = stored.logits
+        if stored.pending_token is not None:
+            # the stored row's last sampled token is not in the cache yet: every child consumes it once
+            with self.clock("append"):
+                self._feed({index: [stored.pending_token] for index in chosen})
+        self.stats["slot_refills"] += sum(self.slots[i].used_before for i in chosen)
+        self.stats["forked_requests"] += len(chosen)
+        self.stats["copied_prefix_tokens"] += cached * len(chosen)
+        self._start([(index, snapshot.prefix_token_ids, sampling) for index, sampling in zip(chosen, samplings)])
+        return chosen
 
     # ------------------------------------------------------------------ continuation
-    def _request_for(self, handle):
-        self._check_open()
+    def _leased(self, handle: LFM25ContinuationHandle) -> _Slot:
+        self._require_open()
         if handle.session is not self or not 0 <= handle.slot < self.batch_size:
             raise ValueError("Continuation handle belongs to another session")
-        request = self.requests[handle.slot]
-        if request is None or request.version != handle.version or not request.delivered or request.handle is not handle:
+        slot = self.slots[handle.slot]
+        if slot.lease is not handle or slot.generation != handle.version:
             raise ValueError("Continuation handle is stale or already consumed")
-        return request
+        return slot
 
-    def _select_graph(self, slots):
-        before = len(self.entry.compact_graphs)
-        graph, size = self.decoder._select_graph(self.entry, slots)
-        self.stats['adaptive_graph_captures'] += len(self.entry.compact_graphs) - before
-        return graph, size
+    def _feed(self, queues: dict) -> None:
+        """Append tokens to cached rows: `queues[slot]` is consumed one position per replay while the other rows sit
+        out; their own pending flags and next inputs are put back afterwards."""
+        depth = max(map(len, queues.values()))
+        plan = torch.full((depth, self.batch_size), -1, dtype=torch.long)
+        for index, tokens in queues.items():
+            plan[:len(tokens), index] = torch.tensor(tokens, dtype=torch.long)
+        plan = plan.to(self.engine.device)
+        feeding = plan >= 0
+        owed_tokens, owed_flags = self.entry.input_tokens.clone(), self.rows.pending.clone()
+        graph, _ = self._graph_for(sorted(queues))
+        for step in range(depth):
+            self.entry.input_tokens.copy_(plan[step].clamp_min(0))
+            self.rows.pending.copy_(feeding[step])
+            graph.replay()
+        self.entry.input_tokens.copy_(owed_tokens)
+        self.rows.pending.copy_(owed_flags)
 
     @torch.inference_mode()
     def resume(self, handles: Sequence[LFM25ContinuationHandle], prompts: Sequence[Sequence[int]],
                samplings: Sequence[LFM25SamplingConfig], *, preserve_rng: bool = False) -> None:
-        """Continue delivered rows from an exact extension of their cached prefix: the pending token and the new
-        suffix are appended one token per replay with per-row masks."""
+        """Continue delivered rows from an exact extension of what they hold: the owed token and the new suffix are
+        appended under per-row masks, then the rows run again.  `preserve_rng` keeps the random stream's position and
+        the stop automaton's state (an internal pause of the same request)."""
         if not len(handles) == len(prompts) == len(samplings):
             raise ValueError("One prompt and sampling configuration is required per handle")
-        if len({h.slot for h in handles}) != len(handles):
+        if len({handle.slot for handle in handles}) != len(handles):
             raise ValueError("Cannot resume a handle twice")
-        appends, carried = [], []
+        queues, carried = {}, {}
         for handle, prompt, sampling in zip(handles, prompts, samplings):
-            request = self._request_for(handle)
+            slot = self._leased(handle)
             self._validate(prompt, sampling)
-            prefix = handle.prefix_token_ids
-            if tuple(prompt[:len(prefix)]) != prefix:
+            held = handle.prefix_token_ids
+            if tuple(prompt[:len(held)]) != held:
                 raise ValueError("Continuation requires the exact cached token prefix")
-            if preserve_rng and (tuple(prompt) != prefix or sampling.seed != request.sampling.seed
-                                 or sampling.stop_table is not request.sampling.stop_table
-                                 or sampling.stop_token_ids != request.sampling.stop_token_ids):
-                raise ValueError('Internal pauses must preserve the exact context, seed and stop rules')
-            carried.append((int(self.rng_positions[handle.slot]), int(self.stop_states[handle.slot])) if preserve_rng else (0, 0))
-            appends.append((handle.slot, (prefix[-1], *prompt[len(prefix):])))
-        if not appends:
+            if preserve_rng:
+                before = slot.sampling
+                if (len(prompt) != len(held) or sampling.seed != before.seed or sampling.stop_table is not before.stop_table
+                        or sampling.stop_token_ids != before.stop_token_ids):
+                    raise ValueError('Internal pauses must preserve the exact context, seed and stop rules')
+            queues[handle.slot] = [held[-1], *prompt[len(held):]]
+        if not queues:
             return
-        width = max(len(t) for _, t in appends)
-        feed = torch.zeros((width, self.batch_size), dtype=torch.long)
-        mask = torch.zeros((width, self.batch_size), dtype=torch.bool)
-        for slot, toks in appends:
-            feed[:len(toks), slot] = torch.tensor(toks)
-            mask[:len(toks), slot] = True
-        feed, mask = feed.to(self.engine.device), mask.to(self.engine.device)
-        keep = self.entry.input_tokens.clone()  # other live rows still owe their own pending tokens
-        graph, _ = self._select_graph([slot for slot, _ in appends])
-        for i in range(width):
-            self.entry.input_tokens.copy_(feed[i])
-            self.entry.active.copy_(mask[i])
-            graph.replay()
-        self.entry.input_tokens.copy_(keep)
-        for handle, prompt, sampling, (position, stop_state) in zip(handles, prompts, samplings, carried):
-            self._configure(handle.slot, prompt, sampling, rng_position=position, stop_state=stop_state)
-            self.stats['resumed_prefix_tokens'] += len(handle.prefix_token_ids) - 1
-            self.stats['appended_tokens'] += len(prompt) - len(handle.prefix_token_ids) + 1
-            self.stats['resumed_requests'] += 1
+        if preserve_rng:
+            positions, states = self.rows.rng_positions.cpu().tolist(), self.rows.stop_states.cpu().tolist()
+            carried = {index: (positions[index], states[index]) for index in queues}
+        with self.clock("append"):
+            self._feed(queues)
+        for handle, prompt in zip(handles, prompts):
+            self.stats["resumed_prefix_tokens"] += len(handle.prefix_token_ids) - 1
+            self.stats["appended_tokens"] += len(prompt) - len(handle.prefix_token_ids) + 1
+        self.stats["resumed_requests"] += len(handles)
+        self._start([(handle.slot, prompt, sampling) for handle, prompt, sampling in zip(handles, prompts, samplings)],
+                    carried=carried or None)
 
     # ------------------------------------------------------------------ the hot loop
-    def _sample(self):
-        logits = self.entry.logits
-        if self._filter is None:
-            return self.sampler.sample(logits, self.seeds, self.rng_positions, self.temperatures)
-        # one shared (top_k, top_p); temperature is per request but must be positive for filtered rows
-        top_k, top_p = self._filter
-        temperature = max(r.sampling.temperature for r in self.requests if r is not None and r.sampling.filtered)
-        return ops.sample_filtered(logits, temperature=temperature, top_k=top_k, top_p=top_p, seeds=self.seeds,
-                                   steps=self.rng_positions, out=(self.sampler.tokens, self.sampler.logprobs))
+    def _draw(self):
+        state = self.rows
+        tokens, logprobs = self.sampler.sample(self.entry.logits, state.seeds, state.rng_positions, state.temperatures)
+        if self._filtered_rows:   # rows with top-k / top-p are redrawn with their own parameters; the others are skipped
+            ops.sample_filtered(self.entry.logits, seeds=state.seeds, steps=state.rng_positions, temperatures=state.temperatures,
+                                top_ks=state.top_ks, top_ps=state.top_ps, out=(tokens, logprobs))
+        return tokens, logprobs
 
     @torch.inference_mode()
     def poll(self, *, steps: int | None = None) -> list:
-        self._check_open()
+        """Run `steps` decode steps (default: the decoder's finish-check interval) and hand out what finished."""
+        self._require_open()
         steps = self.decoder.finish_check_interval if steps is None else steps
         if type(steps) is not int or steps <= 0:
             raise ValueError("steps must be a positive integer")
-        live = [i for i, r in enumerate(self.requests) if r is not None and not r.delivered]
-        if not live:
+        running = [index for index, slot in enumerate(self.slots) if slot.running]
+        if not running:
             return []
-        graph, batch = self._select_graph(live)
-        cfg = self.engine.config
+        graph, width = self._graph_for(running)
+        state, config = self.rows, self.engine.config
         for _ in range(steps):
-            self.entry.active.copy_(self.pending)
-            graph.replay()
-            sampled, logp = self._sample()
+            graph.replay()       # consumes the owed token of every row whose pending flag is set
+            tokens, logprobs = self._draw()
             if self.behavior_topk:
-                ids, probs = ops.behavior_topk(self.entry.logits, sampled, logp, self.behavior_topk)
-                ops.record_head(ids, probs, self.head_ids, self.head_logprobs, self.lengths, self.alive,
+                ids, values = ops.behavior_topk(self.entry.logits, tokens, logprobs, self.behavior_topk)
+                ops.record_head(ids, values, state.head_ids, state.head_logprobs, state.lengths, state.alive,
                                 self.behavior_topk, self.max_new_tokens)
-            ops.record_sample(sampled, logp, self.tokens, self.logprobs, self.lengths, self.limits, self.reasons, self.alive,
-                              self.pending, self.entry.input_tokens, self.stop_states, self.stop_offsets, self.stop_table,
-                              self.ignore_eos, self.rng_positions, cfg.eos_token_id, cfg.vocab_size, self.max_new_tokens)
-        self.stats['decode_steps'] += steps
-        self.stats['decode_row_steps'] += batch * steps
-        self.stats['reserved_row_steps'] += self.batch_size * steps
-        hist = self.stats['decode_batches']
-        hist[str(batch)] = hist.get(str(batch), 0) + steps
-        reasons = self.reasons.cpu().tolist()
-        done = [i for i in live if reasons[i]]
-        if not done:
+            ops.record_sample(tokens, logprobs, state.tokens, state.logprobs, state.lengths, state.limits, state.reasons,
+                              state.alive, state.pending, self.entry.input_tokens, state.stop_states, state.stop_offsets,
+                              self.stops.flat, state.ignore_eos, state.rng_positions, config.eos_token_id, config.vocab_size,
+                              self.max_new_tokens)
+        self.stats["decode_steps"] += steps
+        self.stats["decode_row_steps"] += width * steps
+        self.stats["reserved_row_steps"] += self.batch_size * steps
+        histogram = self.stats["decode_batches"]
+        histogram[str(width)] = histogram.get(str(width), 0) + steps
+        return self._hand_out(running)
+
+    def _hand_out(self, running) -> list:
+        """Results of the running rows that now carry a finish code (one device read for the codes, one per column for
+        the finished rows only)."""
+        codes = self.rows.reasons.cpu().tolist()
+        finished = [index for index in running if codes[index]]
+        if not finished:
             return []
-        index = torch.tensor(done, device=self.engine.device)
-        lengths = self.lengths[index].cpu().tolist()
-        longest = max(lengths)
-        tokens = self.tokens[:, :longest].index_select(0, index).cpu().tolist()
-        logprobs = self.logprobs[:, :longest].index_select(0, index).cpu().tolist()
+        state = self.rows
+        where = torch.tensor(finished, device=self.engine.device)
+        counts = state.lengths[where].cpu().tolist()
+        span = max(counts)
+        token_rows = state.tokens[where, :span].cpu().tolist()
+        logprob_rows = state.logprobs[where, :span].cpu().tolist()
         results = []
-        for slot, length, ids, probs in zip(done, lengths, tokens, logprobs):
-            request = self.requests[slot]
-            request.delivered = True
-            ids = tuple(ids[:length])
-            request.handle = LFM25ContinuationHandle(self, slot, request.version, request.prompt + ids)
-            k = request.sampling.behavior_topk
-            head = BehaviorTopK(self.head_ids[slot, :length, :k].cpu(), self.head_logprobs[slot, :length, :k].cpu()) if k else None
-            results.append(LFM25SessionResult(request.handle, request.prompt, ids,
-                                              tuple(probs[:length]) if request.sampling.return_logprobs else None,
-                                              reasons[slot], head))
+        for index, count, ids, values in zip(finished, counts, token_rows, logprob_rows):
+            slot = self.slots[index]
+            ids = tuple(ids[:count])
+            slot.lease = LFM25ContinuationHandle(self, index, slot.generation, slot.prompt + ids)
+            head = None
+            if slot.sampling.behavior_topk:
+                k = slot.sampling.behavior_topk
+                head = BehaviorTopK(state.head_ids[index, :count, :k].cpu(), state.head_logprobs[index, :count, :k].cpu())
+            results.append(LFM25SessionResult(slot.lease, slot.prompt, ids,
+                                              tuple(values[:count]) if slot.sampling.return_logprobs else None,
+                                              codes[index], head))
         return results
 
     @torch.inference_mode()
     def release(self, handle: LFM25ContinuationHandle) -> None:
-        self._request_for(handle)
-        slot = handle.slot
-        self.requests[slot] = None
-        self.versions[slot] += 1
-        self.alive[slot] = False
-        self.pending[slot] = False
-        self.entry.cache.seq_lens[slot] = 0
-        if not any(r is not None and r.sampling.filtered for r in self.requests):
-            self._filter = None
+        """Give a delivered row's slot back."""
+        slot = self._leased(handle)
+        slot.generation += 1
+        slot.prompt = slot.sampling = slot.lease = None
+        self._filtered_rows.discard(handle.slot)
+        self.rows.retire(handle.slot)
+        self.entry.cache.seq_lens[handle.slot] = 0
 
-    def close(self):
+    def close(self) -> None:
         if self.closed:
             return
         self.closed = True
-        self.requests = [None] * self.batch_size
-        self._snapshots.clear()
+        for slot in self.slots:
+            slot.generation += 1
+            slot.prompt = slot.sampling = slot.lease = None
+        self._stored.clear()
         if self.decoder._active_session is self:
             self.decoder._active_session = None
 
     def __enter__(self):
-        self._check_open()
+        self._require_open()
         return self
 
     def __exit__(self, *_):
         self.close()
 
 
-def _copy_bytes(target: torch.Tensor, source: torch.Tensor) -> None:
-    """Copy without dequantising: one-byte element types go through a uint8 view."""
-    if target.element_size() == 1:
-        target.view(torch.uint8).copy_(source.view(torch.uint8))
-    else:
-        target.copy_(source)
+def _raw(tensor: torch.Tensor) -> torch.Tensor:
+    """One-byte element types as uint8, so that indexed copies move e4m3 codes as they are."""
+    return tensor.view(torch.uint8) if tensor.element_size() == 1 else tensor

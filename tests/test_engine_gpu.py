@@ -605,19 +605,35 @@ def test_adaptive_batching_compact_graphs_leave_resident_rows_untouched():
 
 
 @torch.inference_mode()
-def test_session_filtered_sampling_extension():
+def test_session_rows_keep_their_own_sampling_whatever_their_neighbours_ask_for():
+    """Top-k / top-p rows in a session (an extension: lfm25_session.py:217-218 refuses them) next to greedy and
+    full-support rows: every request's tokens are those of the same request alone in a session, in any slot, and rows
+    with different k, p and temperature coexist."""
     engine, _, _ = _engine()
     engine.enable_cuda_graphs(max_graphs=1)
-    s = LFM25SamplingConfig(temperature=1.0, top_k=4, top_p=0.95, seed=11, max_new_tokens=7, ignore_eos=True)
-    outs = []
-    for slots in ([0, 1], [1, 0]):
-        with engine.generation_session(max_batch_size=2, max_new_tokens=7, cache_len=32) as session:
-            session.admit([[1, 2, 3], [1, 4]], [s, replace(s, seed=12)], slots=slots)
-            with pytest.raises(ValueError, match="share top_k"):
-                session._validate([1], replace(s, top_k=9))
-            res = {r.prompt_token_ids: r.token_ids for r in session.poll(steps=8)}
-            outs.append(res)
-    assert outs[0] == outs[1]
+    base = LFM25SamplingConfig(temperature=1.0, seed=11, max_new_tokens=7, ignore_eos=True)
+    requests = [([1, 2, 3], replace(base, top_k=4, top_p=0.95)),           # filtered
+                ([1, 4], replace(base, temperature=0.0)),                   # greedy
+                ([1, 5, 6], replace(base, seed=12)),                        # full support
+                ([1, 7], replace(base, temperature=0.7, top_k=9, seed=13)),  # filtered, other k and temperature
+                ([1, 8, 8], replace(base, top_p=0.5, seed=14))]             # nucleus only
+
+    def run(items, slots=None):
+        with engine.generation_session(max_batch_size=5, max_new_tokens=7, cache_len=32) as session:
+            session.admit([p for p, _ in items], [s for _, s in items], slots=slots)
+            return {r.prompt_token_ids: (r.token_ids, r.logprobs) for r in session.poll(steps=8)}
+
+    together = run(requests)
+    shuffled = run(requests, slots=[4, 2, 0, 1, 3])
+    assert together == shuffled and len(together) == 5
+    for prompt, sampling in requests:
+        alone = run([(prompt, sampling)])
+        assert alone[tuple(prompt)] == together[tuple(prompt)], f"{sampling} changed next to other requests"
+    # the greedy row is the argmax sequence, the top-k row stays inside a top-1 run when k = 1
+    greedy = engine.generate(*_flat([[1, 4]]), repeats=1, sampling=replace(base, temperature=0.0))
+    assert list(together[(1, 4)][0]) == greedy.token_ids[0, 0].tolist()
+    top1 = run([([1, 4], replace(base, top_k=1))])
+    assert top1[(1, 4)][0] == together[(1, 4)][0]
 
 
 @torch.inference_mode()
