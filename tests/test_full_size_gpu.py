@@ -221,6 +221,44 @@ def test_full_model_graph_replay_equals_eager_step_and_chunked_prefill_equals_wh
 
 
 @torch.inference_mode()
+def test_all_bf16_session_at_256_sequences_graph_equals_eager_and_repeats(big_model):
+    """Config 4's batch: the all-bf16 engine (bf16 linears, bf16 KV cache) with 256 concurrent ragged sequences at
+    temperature 1 through one session.  The captured step and the same step launched kernel by kernel give the same
+    tokens and log-probabilities, a second run repeats them, and the first tokens are draws from the prefill logits of
+    an independent prefill of the same prompts (raw log-probability of each first token within 1e-5)."""
+    engine, ocfg, _ = big_model
+    from climbing_gym_amd.config import LFM25SamplingConfig
+    from climbing_gym_amd.engine import flatten_token_batches
+    g = torch.Generator().manual_seed(8)
+    prompts = [torch.randint(0, ocfg.vocab_size, (int(n),), generator=g).tolist() for n in torch.randint(24, 97, (256,), generator=g)]
+    sampling = [LFM25SamplingConfig(temperature=1.0, seed=500 + i, max_new_tokens=6, ignore_eos=True) for i in range(256)]
+
+    def run(capture):
+        engine.enable_cuda_graphs(max_graphs=1, max_prefill_tokens=4096, capture=capture)
+        with engine.generation_session(max_batch_size=256, max_new_tokens=6, cache_len=128) as session:
+            assert not session.entry.cache.fp8 and not engine._cuda_decoder.fp8_weights
+            session.admit(prompts, sampling)
+            results = sorted(session.poll(steps=7), key=lambda r: r.handle.slot)
+            stats = dict(session.stats)
+        engine.disable_cuda_graphs()
+        return results, stats
+
+    graph, stats = run(True)
+    eager, _ = run(False)
+    again, _ = run(True)
+    assert len(graph) == 256 and stats["decode_steps"] == 7 and stats["decode_batches"] == {"256": 7}
+    for a, b, c in zip(graph, eager, again):
+        assert a.token_ids == b.token_ids == c.token_ids and len(a.token_ids) == 6 and a.finish_reason == 3
+        assert a.logprobs == b.logprobs == c.logprobs
+    engine.enable_cuda_graphs(max_graphs=1, max_prefill_tokens=1 << 20, capture=False)
+    prefix = engine.prefill(*flatten_token_batches(prompts))
+    first = torch.tensor([r.token_ids[0] for r in graph], device=DEV)
+    want = prefix.next_token_logits.float().log_softmax(-1).gather(1, first[:, None])[:, 0].cpu()
+    engine.disable_cuda_graphs()
+    torch.testing.assert_close(torch.tensor([r.logprobs[0] for r in graph]), want, atol=3e-2, rtol=0)
+
+
+@torch.inference_mode()
 def test_filtered_sampling_session_at_512_sequences_is_repeatable_and_stays_in_support(big_model):
     """Config 5: FP8 everywhere, 512 concurrent ragged sequences (prompts uniform in [512, 4096]), top-k 50 /
     top-p 0.95 at temperature 1 with fixed seeds, sequences admitted and retired as they finish."""
