@@ -20,6 +20,7 @@ DTYPE_CODE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 _SIGNATURES = {
     "lfm2_embedding": "ppplllip",
     "lfm2_rms_norm": "ppppp" "llfip",
+    "lfm2_embedding_rms_norm": "ppppppp" "lllfip",
     "lfm2_rms_norm_fp8": "pppppp" "llfip",
     "lfm2_swiglu": "ppllip",
     "lfm2_swiglu_fp8": "pppllip",
@@ -43,6 +44,7 @@ _SIGNATURES = {
     "lfm2_store_kv_packed": "ppppppppp" "liillliip",
     "lfm2_decode_attention": "pppppppppp" "lipp" "liiillllfiippp",
     "lfm2_decode_schedule": "pppp" "lp",
+    "lfm2_decode_begin": "pppppppp" "lp",
     "lfm2_prefill_attention": "ppppp" "lliiifip",
     "lfm2_build_token_map": "ppp" "llp",
     "lfm2_gather_inputs": "ppppppp" "lp",
@@ -54,6 +56,7 @@ _SIGNATURES = {
     "lfm2_configure_rows": "p" "ll" "ppppppppppppp" "p",
     "lfm2_head_logprobs": "ppppp" "lliip",
     "lfm2_record_sample": "ppppppppppppppp" "llllp",
+    "lfm2_sample_record": "pppppppppppppppppppp" "llllip",
     "lfm2_record_head": "pppppp" "illp",
 }
 _INT64_RESULT = {

@@ -605,8 +605,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
 // One counting sweep over the rows gives the classes' sizes, a second one places the rows: in each, a thread's rank
 // within its class comes from a wave scan and the waves' totals.
 constexpr int kSchedClasses = 9;   // full chunks, then partial chunks of 8 (512-token chunks only), 7, ... 1 tiles
-__global__ void __launch_bounds__(1024)
-decode_schedule_kernel(int32_t* schedule, const int32_t* positions, const uint8_t* active, const int32_t* slot_ids, int B) {
+__device__ __forceinline__ void
+schedule_rows(int32_t* schedule, const int32_t* positions, const uint8_t* active, const int32_t* slot_ids, int B) {
   __shared__ int wave_total[kSchedClasses][16];
   __shared__ int class_base[kSchedClasses + 1];   // where each class starts; running, during the second sweep
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -716,6 +716,38 @@ decode_schedule_kernel(int32_t* schedule, const int32_t* positions, const uint8_
     }
     __syncthreads();
   }
+}
+
+__global__ void __launch_bounds__(1024)
+decode_schedule_kernel(int32_t* schedule, const int32_t* positions, const uint8_t* active, const int32_t* slot_ids, int B) {
+  schedule_rows(schedule, positions, active, slot_ids, B);
+}
+
+// The head of a decode step in one launch: the rows' inputs (through the slot map of a compact batch when `slots` is
+// given: _gather_inputs of lfm25_batching.py:11-22), the positions the step's layers use (a snapshot of the lengths),
+// the lengths advanced for the rows that take part (lfm25_cuda.py:185-186, lfm25_batching.py:35-46: nothing else of the
+// step reads the lengths, so advancing them first changes nothing), and the attention work list.  Row b is handled by
+// thread b % 1024 in every sweep, so a thread only reads back what it wrote itself.
+__global__ void __launch_bounds__(1024)
+decode_begin_kernel(int32_t* schedule, int32_t* positions_out, int64_t* tokens_out, uint8_t* mask_out, int32_t* lengths,
+                    const int64_t* input, const uint8_t* active, const int32_t* slots, int B) {
+  for (int b = threadIdx.x; b < B; b += 1024) {
+    int pos;
+    if (slots) {
+      const int slot = slots[b];
+      const bool valid = slot >= 0;
+      const bool on = valid && active[slot];
+      pos = valid ? lengths[slot] : 0;
+      tokens_out[b] = valid ? input[slot] : 0;
+      mask_out[b] = on;
+      if (on) lengths[slot] = pos + 1;
+    } else {
+      pos = lengths[b];
+      if (!active || active[b]) lengths[b] = pos + 1;
+    }
+    positions_out[b] = pos;
+  }
+  schedule_rows(schedule, positions_out, slots ? mask_out : active, slots, B);
 }
 
 // Merge the chunk partials of one (row, query head); inactive or empty rows give zeros.
@@ -1116,6 +1148,17 @@ extern "C" int lfm2_decode_schedule(int32_t* schedule, const int32_t* positions,
   LFM2_REQUIRE(B > 0 && schedule && positions, "decode_schedule: bad arguments");
   hipLaunchKernelGGL(decode_schedule_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, schedule, positions, active,
                      slot_ids, (int)B);
+  LFM2_LAUNCH_CHECK();
+}
+
+extern "C" int lfm2_decode_begin(int32_t* schedule, int32_t* positions_out, int64_t* tokens_out, uint8_t* mask_out,
+                                 int32_t* lengths, const int64_t* input, const uint8_t* active, const int32_t* slots,
+                                 int64_t B, void* stream) {
+  LFM2_REQUIRE(B > 0 && schedule && positions_out && lengths, "decode_begin: bad arguments");
+  LFM2_REQUIRE(slots == nullptr || (tokens_out && mask_out && input && active),
+               "decode_begin: a slot map needs the input tokens, the slots' activity flags and the two row outputs");
+  hipLaunchKernelGGL(decode_begin_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, schedule, positions_out, tokens_out,
+                     mask_out, lengths, input, active, slots, (int)B);
   LFM2_LAUNCH_CHECK();
 }
 

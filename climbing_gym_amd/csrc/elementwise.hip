@@ -104,6 +104,10 @@ struct SplitInput {
   const float* w_scales;  // [H]
   int64_t stride;         // M * H
   int splits;
+  // With `tokens` set (no residual) `x` is an embedding table [vocab, H]: the row's input is the table row of its token
+  // (ids clamped into the table like lfm2_embedding), and that row is also written to `summed`, the residual stream.
+  const int64_t* tokens = nullptr;
+  int64_t vocab = 0;
 };
 
 template <typename T, int NV, bool ADD, bool FP8>
@@ -113,7 +117,15 @@ rms_norm_kernel(T* out, uint8_t* q, float* scales, T* summed, const T* x, const 
   __shared__ float red[kRowWaves];
   const int64_t row = blockIdx.x;
   constexpr int N = Vec<T>::N;
-  x += row * H;
+  const bool gather = !ADD && split.tokens != nullptr;
+  if (gather) {
+    int64_t tok = split.tokens[row];
+    tok = tok < 0 ? 0 : (tok >= split.vocab ? split.vocab - 1 : tok);
+    x += tok * H;
+    summed += row * H;
+  } else {
+    x += row * H;
+  }
   if (ADD) { res += row * H; summed += row * H; }
   if (FP8) q += row * H; else out += row * H;
 
@@ -137,6 +149,7 @@ rms_norm_kernel(T* out, uint8_t* q, float* scales, T* summed, const T* x, const 
           for (int e = 0; e < N; ++e) v[j][e] = round_to<T>(split.w_scales ? (v[j][e] * sa) * split.w_scales[i + e] : v[j][e]);
         } else {
           load_vec<T>(x + i, v[j]);
+          if (gather) store_vec<T>(summed + i, v[j]);
         }
         if (ADD) {
           float r[N];
@@ -190,7 +203,7 @@ rms_norm_kernel(T* out, uint8_t* q, float* scales, T* summed, const T* x, const 
     float ss = 0.f;
     for (int64_t i = threadIdx.x; i < H; i += kRowThreads) {
       const float a = value(i);
-      if (ADD) summed[i] = Elem<T>::store(a);
+      if (ADD || gather) summed[i] = Elem<T>::store(a);
       ss += a * a;
     }
     ss = block_sum<kRowWaves>(ss, red);
@@ -260,6 +273,22 @@ extern "C" int lfm2_rms_norm_fp8(uint8_t* q, float* scales, void* summed, const 
   hipStream_t s = (hipStream_t)stream;
   DISPATCH_DTYPE(dtype, if (residual) launch_rms<T, true, true>(nullptr, q, scales, summed, x, weight, residual, M, H, eps, s);
                  else launch_rms<T, false, true>(nullptr, q, scales, nullptr, x, weight, nullptr, M, H, eps, s));
+  LFM2_LAUNCH_CHECK();
+}
+
+extern "C" int lfm2_embedding_rms_norm(void* out, uint8_t* q, float* scales, void* hidden, const void* table,
+                                       const int64_t* tokens, const void* weight, int64_t M, int64_t H, int64_t V, float eps,
+                                       int dtype, void* stream) {
+  LFM2_REQUIRE(M > 0 && H > 0 && V > 0, "embedding_rms_norm: empty shape");
+  LFM2_REQUIRE(hidden && table && tokens && weight, "embedding_rms_norm: a required pointer is null");
+  LFM2_REQUIRE((q == nullptr) == (scales == nullptr) && (q == nullptr) != (out == nullptr),
+               "embedding_rms_norm: either out, or q with scales");
+  SplitInput gather{nullptr, nullptr, nullptr, 0, 0};
+  gather.tokens = tokens;
+  gather.vocab = V;
+  hipStream_t s = (hipStream_t)stream;
+  DISPATCH_DTYPE(dtype, if (q) launch_rms<T, false, true>(nullptr, q, scales, hidden, table, weight, nullptr, M, H, eps, s, gather);
+                 else launch_rms<T, false, false>(out, nullptr, nullptr, hidden, table, weight, nullptr, M, H, eps, s, gather));
   LFM2_LAUNCH_CHECK();
 }
 

@@ -126,6 +126,33 @@ sample_partial_kernel(const T* logits, float* scratch, const float* temperatures
   }
 }
 
+// The per-row record step of lfm25_session.py:34-56 for one row and its freshly drawn token: token and raw
+// log-probability into the row's buffers, stop automaton, finish code, flags, next input, random-stream position.
+// `tokens == nullptr` means "no record": the sampler then only returns its draw.
+struct RecordArgs {
+  int64_t* tokens; float* logprobs; int32_t* lengths; const int32_t* limits; int8_t* reasons; uint8_t* alive;
+  uint8_t* pending; int64_t* input; int64_t* stop_states; const int64_t* stop_offsets; const int32_t* stop_table;
+  const uint8_t* ignore_eos; int64_t* rng_positions; int64_t eos, V, cap;
+};
+__device__ __forceinline__ void record_row(const RecordArgs& r, int64_t row, int64_t token, float logp) {
+  if (!r.alive[row]) return;
+  const int32_t length = r.lengths[row];
+  r.tokens[row * r.cap + length] = token;
+  r.logprobs[row * r.cap + length] = logp;
+  const int32_t value = r.stop_table[r.stop_offsets[row] + r.stop_states[row] * r.V + token];
+  r.stop_states[row] = value & 65535;
+  int8_t reason = 0;
+  if (token == r.eos && !r.ignore_eos[row]) reason = 1;
+  else if (value >= 65536) reason = 2;
+  else if (length + 1 >= r.limits[row]) reason = 3;
+  r.lengths[row] = length + 1;
+  r.rng_positions[row] += 1;
+  r.reasons[row] = reason;
+  r.alive[row] = reason == 0;
+  r.pending[row] = reason == 0;
+  r.input[row] = token;
+}
+
 // Pass 2, one workgroup per row: merge the tiles, then read one tile again.  Greedy rows take the first column
 // that holds the maximum, in the first tile that has it.  The others pick the tile and then the column where the
 // cumulative mass passes u * total (tiles and columns in index order; the last column with mass if rounding pushes
@@ -134,7 +161,7 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 sample_finish_kernel(const T* logits, const float* scratch, int64_t* tokens, float* logprobs, const int64_t* seeds,
                      const int64_t* steps, const float* temperatures, int64_t seed, int64_t step, float temperature,
-                     int64_t V, int parts) {
+                     int64_t V, int parts, RecordArgs record) {
   __shared__ TileStat s_stat[4];
   __shared__ float s_tile_mass[256];
   __shared__ float s_wave[4];
@@ -252,7 +279,9 @@ sample_finish_kernel(const T* logits, const float* scratch, int64_t* tokens, flo
     float chosen = x[0];
 #pragma unroll
     for (int i = 1; i < 16; ++i) chosen = token - col0 == i ? x[i] : chosen;
-    if (logprobs) logprobs[row] = chosen - (mx + logf(total));
+    const float logp = chosen - (mx + logf(total));
+    if (logprobs) logprobs[row] = logp;
+    if (record.tokens) record_row(record, row, token, logp);
   }
 }
 
@@ -940,7 +969,31 @@ extern "C" int lfm2_sample(int64_t* tokens, float* logprobs, const void* logits,
                  hipLaunchKernelGGL(sample_partial_kernel<T>, dim3(parts, B), dim3(256), 0, s, (const T*)logits, scratch,
                                     temperatures, temperature, V, parts);
                  hipLaunchKernelGGL(sample_finish_kernel<T>, dim3(B), dim3(256), 0, s, (const T*)logits, scratch, tokens,
-                                    logprobs, seeds, steps, temperatures, seed, step, temperature, V, parts));
+                                    logprobs, seeds, steps, temperatures, seed, step, temperature, V, parts, RecordArgs{}));
+  LFM2_LAUNCH_CHECK();
+}
+
+extern "C" int lfm2_sample_record(int64_t* sampled, float* logp, const void* logits, float* scratch, const int64_t* seeds,
+                                  const int64_t* steps, const float* temperatures, int64_t* tokens, float* logprobs,
+                                  int32_t* lengths, const int32_t* limits, int8_t* reasons, uint8_t* alive, uint8_t* pending,
+                                  int64_t* input, int64_t* stop_states, const int64_t* stop_offsets,
+                                  const int32_t* stop_table, const uint8_t* ignore_eos, int64_t* rng_positions, int64_t eos,
+                                  int64_t cap, int64_t B, int64_t V, int dtype, void* stream) {
+  LFM2_REQUIRE(B > 0 && V > 0 && cap > 0, "sample_record: bad shape");
+  LFM2_REQUIRE(B <= 65535, "sample_record: more than 65535 rows");
+  LFM2_REQUIRE(V <= 256ll * kTile, "sample_record: vocabulary above 1048576");
+  LFM2_REQUIRE(sampled && logp && logits && scratch && seeds && steps && temperatures && tokens && logprobs && lengths &&
+               limits && reasons && alive && pending && input && stop_states && stop_offsets && stop_table && ignore_eos &&
+               rng_positions, "sample_record: a required pointer is null");
+  const int parts = ceil_div(V, kTile);
+  const RecordArgs record{tokens, logprobs, lengths, limits, reasons, alive, pending, input, stop_states, stop_offsets,
+                          stop_table, ignore_eos, rng_positions, eos, V, cap};
+  hipStream_t s = (hipStream_t)stream;
+  DISPATCH_DTYPE(dtype, "sample_record",
+                 hipLaunchKernelGGL(sample_partial_kernel<T>, dim3(parts, B), dim3(256), 0, s, (const T*)logits, scratch,
+                                    temperatures, 0.f, V, parts);
+                 hipLaunchKernelGGL(sample_finish_kernel<T>, dim3(B), dim3(256), 0, s, (const T*)logits, scratch, sampled, logp,
+                                    seeds, steps, temperatures, 0, 0, 0.f, V, parts, record));
   LFM2_LAUNCH_CHECK();
 }
 

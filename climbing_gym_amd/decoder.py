@@ -116,9 +116,9 @@ class LFM25HIPDecoder:
         self.fp8_weights.clear()
 
     # ------------------------------------------------------------------ capture
-    def _forward(self, cache, tokens, active=None, *, slot_ids=None, positions=None, logits_out=None):
+    def _forward(self, cache, tokens, active=None, *, slot_ids=None, positions=None, logits_out=None, gather=None):
         return self.engine._decode_forward(cache, tokens, active, slot_ids=slot_ids, positions=positions, fp8=self.fp8_weights,
-                                           logits_out=logits_out)
+                                           logits_out=logits_out, gather=gather)
 
     def _capture(self, step, before_warmup=None):
         """Two warm-up launches, then record `step` into a HIP graph on the decoder's capture stream."""
@@ -197,8 +197,9 @@ class LFM25HIPDecoder:
         active = torch.zeros(batch_size, device=device, dtype=torch.bool)
 
         def step():
-            ops.gather_inputs(tokens, positions, active, entry.input_tokens, entry.cache.seq_lens, entry.active, slots)
-            self._forward(entry.cache, tokens, active, slot_ids=slots, positions=positions, logits_out=entry.logits)
+            # the rows' tokens, positions and activity flags are gathered from the slots by the step's first launch
+            self._forward(entry.cache, tokens, active, slot_ids=slots, positions=positions, logits_out=entry.logits,
+                          gather=(entry.input_tokens, entry.active))
 
         graph = self._capture(step)
         return CompactDecodeGraph(graph, slots, (tokens, positions, active))

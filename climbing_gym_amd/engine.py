@@ -250,17 +250,27 @@ class LFM25Engine:
     def _fp8(self):
         return self._cuda_decoder.fp8_weights if self._cuda_decoder is not None else {}
 
-    def _norm_linear(self, x, norm_weight, residual, weight, fp8, place=None):
-        """residual-add + RMSNorm feeding a projection; W8A8 when the projection has an e4m3 copy.  `place`
-        (an `ops.RowPlacement`) sends the product's rows into an existing buffer."""
-        packed = fp8.get(id(weight))
-        if packed is not None:
+    def _normed(self, x, norm_weight, residual, weight, fp8):
+        """residual-add + RMSNorm in front of the projection `weight`: (projection input, new residual).  The input is
+        (e4m3 rows, per-row scales) when the projection has an e4m3 copy, a tensor otherwise."""
+        if id(weight) in fp8:
             q, scales, residual = ops.rms_norm_fp8(x, norm_weight, self.config.norm_eps, residual)
-            return packed.linear_quantized(q, scales, dtype=self.dtype, place=place), residual
+            return (q, scales), residual
         if isinstance(x, ops.SplitProduct) and residual is None:
             x = x.materialize()
-        normed, residual = ops.rms_norm(x, norm_weight, self.config.norm_eps, residual)
-        return ops.linear(normed, weight, place=place), residual
+        return ops.rms_norm(x, norm_weight, self.config.norm_eps, residual)
+
+    def _project(self, normed, weight, fp8, place=None):
+        """The projection of what `_normed` returned; `place` (an `ops.RowPlacement`) sends the product's rows into an
+        existing buffer."""
+        packed = fp8.get(id(weight))
+        if packed is not None:
+            return packed.linear_quantized(normed[0], normed[1], dtype=self.dtype, place=place)
+        return ops.linear(normed, weight, place=place)
+
+    def _norm_linear(self, x, norm_weight, residual, weight, fp8, place=None):
+        normed, residual = self._normed(x, norm_weight, residual, weight, fp8)
+        return self._project(normed, weight, fp8, place), residual
 
     def _linear(self, x, weight, fp8):
         """Out projection of an operator; `x` is a tensor or, from a fused producer, (e4m3 rows, scales)."""
@@ -271,32 +281,33 @@ class LFM25Engine:
 
     def _backbone(self, tokens, attention_op, conv_op, fp8, *, defer_reduce=False, projecting_attention_op=None):
         """Embedding and all layers with the fused residual chain of lfm25_cuda.py:134-184: every RMSNorm also adds
-        the previous block's output into the running residual.  Returns (last MLP output, residual).  With
-        `defer_reduce` (decode) a split-K down projection hands its partial sums to the next norm.
-        `projecting_attention_op(op, packed, rows_q, row_scales)` (decode), when it takes the layer (returns something),
-        runs the W8A8 QKV projection itself, with the head preparation and the KV append as the product's epilogue."""
-        hidden = ops.embedding(tokens, self.weights.embed_tokens)
-        residual = None
-        for layer in self.weights.layers:
+        the previous block's output into the running residual; the first norm, which has nothing to add, runs in the
+        launch that gathers the embedding rows.  Returns (last MLP output, residual).  With `defer_reduce` (decode) a
+        split-K down projection hands its partial sums to the next norm.  `projecting_attention_op(op, packed, rows_q,
+        row_scales)` (decode), when it takes the layer (returns something), runs the W8A8 QKV projection itself, with the
+        head preparation and the KV append as the product's epilogue."""
+        layers = self.weights.layers
+        if not layers:
+            return ops.embedding(tokens, self.weights.embed_tokens), None
+        operator_weight = lambda layer: layer.attention.qkv_weight if layer.attention is not None else layer.conv.in_weight
+        normed, residual = ops.embedding_rms_norm(tokens, self.weights.embed_tokens, layers[0].operator_norm_weight,
+                                                  self.config.norm_eps, fp8=id(operator_weight(layers[0])) in fp8)
+        hidden = None
+        for index, layer in enumerate(layers):
+            if index:
+                normed, residual = self._normed(hidden, layer.operator_norm_weight, residual, operator_weight(layer), fp8)
             if layer.attention is not None:
                 op = layer.attention
                 packed = fp8.get(id(op.qkv_weight))
                 attended = None
                 if projecting_attention_op is not None and packed is not None:
-                    rows_q, row_scales, summed = ops.rms_norm_fp8(hidden, layer.operator_norm_weight, self.config.norm_eps, residual)
-                    attended = projecting_attention_op(op, packed, rows_q, row_scales)
-                    if attended is None:   # shape not covered: the plain projection of the rows just quantised
-                        qkv = packed.linear_quantized(rows_q, row_scales, dtype=self.dtype)
-                        attended = attention_op(op, qkv)
-                    residual = summed
-                else:
-                    qkv, residual = self._norm_linear(hidden, layer.operator_norm_weight, residual, op.qkv_weight, fp8)
-                    attended = attention_op(op, qkv)
+                    attended = projecting_attention_op(op, packed, normed[0], normed[1])
+                if attended is None:   # no fused projection for this shape: the plain one, then the head preparation
+                    attended = attention_op(op, self._project(normed, op.qkv_weight, fp8))
                 mixed = self._linear(attended, op.out_weight, fp8)
             else:
                 op = layer.conv
-                bcx, residual = self._norm_linear(hidden, layer.operator_norm_weight, residual, op.in_weight, fp8)
-                mixed = self._linear(conv_op(op, bcx), op.out_weight, fp8)
+                mixed = self._linear(conv_op(op, self._project(normed, op.in_weight, fp8)), op.out_weight, fp8)
             gate_up, residual = self._norm_linear(mixed, layer.ffn_norm_weight, residual, layer.w13_weight, fp8)
             down = fp8.get(id(layer.w2_weight))
             if down is not None:
@@ -314,17 +325,28 @@ class LFM25Engine:
 
     # ------------------------------------------------------------------ decode step (one token per row)
     def _decode_forward(self, cache: LFM25HybridCache, tokens, active=None, *, slot_ids=None, positions=None, fp8=None,
-                        logits_out=None):
+                        logits_out=None, gather=None):
         """One token for every row (lfm25_cuda.py:128-192).  Rows index cache slots directly, or through `slot_ids`
         (then `positions` are the rows' lengths and -1 marks padding).  With `logits_out` ([slots, vocab]) the head
         projection writes the live rows' logits there (row -> its slot) and the other rows keep theirs: the
         `_scatter_logits` step of lfm25_batching.py:99-101 without a copy."""
         cfg = self.config
         fp8 = self._fp8() if fp8 is None else fp8
-        positions = cache.seq_lens if positions is None else positions
         rows = tokens.numel()
-        # the attention layers of one step see the same lengths: build the work list of the attention kernel once
-        schedule = ops.decode_schedule(positions, active, slot_ids, capacity=cache.max_seq_len)
+        # The attention layers of one step see the same lengths: the work list of the attention kernel is built once.
+        # When the step owns its rows' bookkeeping (rows are the cache's slots, or a compact batch gathered from them:
+        # `gather` = (the slots' input tokens, the slots' activity flags)) the same launch snapshots the positions,
+        # gathers the inputs and advances the lengths; otherwise the caller's positions are used and the lengths are
+        # advanced at the end.
+        advance_after = False
+        if positions is None:
+            positions, schedule = ops.decode_begin(cache.seq_lens, active, capacity=cache.max_seq_len)
+        elif gather is not None:
+            positions, schedule = ops.decode_begin(cache.seq_lens, capacity=cache.max_seq_len,
+                                                   gather=(gather[0], gather[1], slot_ids, tokens, positions, active))
+        else:
+            schedule = ops.decode_schedule(positions, active, slot_ids, capacity=cache.max_seq_len)
+            advance_after = True
 
         def attention_op(op, qkv):
             # QK norm + RoPE with the new token's keys and values written straight into the cache, then attention over
@@ -368,7 +390,8 @@ class LFM25Engine:
                                           projecting_attention_op=projecting_attention_op)
         place = None if logits_out is None else ops.RowPlacement(logits_out, slot_ids, active)
         logits = self._head(hidden, residual, fp8, place)
-        ops.advance_positions(cache.seq_lens, positions, slot_ids, active)
+        if advance_after:
+            ops.advance_positions(cache.seq_lens, positions, slot_ids, active)
         return logits
 
     # ------------------------------------------------------------------ prefill

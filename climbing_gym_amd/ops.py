@@ -50,6 +50,25 @@ def embedding(tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
     return out.view(*tokens.shape, table.size(1))
 
 
+def embedding_rms_norm(tokens: torch.Tensor, table: torch.Tensor, weight: torch.Tensor, eps: float, *, fp8: bool):
+    """`embedding` followed by the step's first norm, which has no residual (lfm25_cuda.py:134-137), as one launch:
+    returns (norm output, hidden) or, with `fp8`, ((e4m3 rows, scales), hidden); `hidden` is the embedding itself."""
+    _check(tokens, table, weight)
+    flat = tokens.reshape(-1).to(torch.long)
+    rows, width = flat.numel(), table.size(1)
+    hidden = torch.empty((rows, width), device=table.device, dtype=table.dtype)
+    if fp8:
+        q = torch.empty((rows, width), device=table.device, dtype=FP8)
+        scales = torch.empty(rows, device=table.device, dtype=torch.float32)
+        call("lfm2_embedding_rms_norm", None, q, scales, hidden, table, flat, weight, rows, width, table.size(0), float(eps),
+             _code(table.dtype))
+        return (q, scales), hidden
+    out = torch.empty_like(hidden)
+    call("lfm2_embedding_rms_norm", out, None, None, hidden, table, flat, weight, rows, width, table.size(0), float(eps),
+         _code(table.dtype))
+    return out, hidden
+
+
 def rms_norm(x, weight: torch.Tensor, eps: float, residual: torch.Tensor | None = None):
     """lfm25_cuda_kernels.py:47-55: returns (norm(x+residual)*w, x+residual); `summed is x` without residual.
     `x` may be a `SplitProduct` (then a residual is required and the projection's reduce pass runs inside the norm)."""
@@ -381,6 +400,25 @@ def decode_schedule(positions, active=None, slot_ids=None, *, capacity: int):
     return schedule
 
 
+def decode_begin(lengths, active=None, *, capacity: int, gather=None):
+    """The head of a decode step in one launch: returns (positions, schedule) where `positions` is a snapshot of the
+    rows' cache lengths for the step's layers and `schedule` the attention work list; the lengths of the rows that take
+    part are advanced by one (nothing else of the step reads them).  `gather` = (input tokens [slots], activity
+    flags [slots], slot map int32 [rows], tokens out int64 [rows], positions out int32 [rows], mask out bool [rows])
+    makes the rows a compact batch over the slots (`gather_inputs` of lfm25_batching.py:11-22 in the same launch)."""
+    if gather is None:
+        rows = lengths.numel()
+        positions = torch.empty(rows, device=lengths.device, dtype=torch.int32)
+        schedule = torch.empty(query("lfm2_decode_schedule_size", rows, int(capacity)), device=lengths.device, dtype=torch.int32)
+        call("lfm2_decode_begin", schedule, positions, None, None, lengths, None, active, None, rows)
+        return positions, schedule
+    input_tokens, slot_active, slots, tokens, positions, mask = gather
+    rows = slots.numel()
+    schedule = torch.empty(query("lfm2_decode_schedule_size", rows, int(capacity)), device=lengths.device, dtype=torch.int32)
+    call("lfm2_decode_begin", schedule, positions, tokens, mask, lengths, input_tokens, slot_active, slots, rows)
+    return positions, schedule
+
+
 def attend(q, k_cache, v_cache, k_scales, v_scales, positions, *, active=None, scale=None, config=None,
            slot_ids=None, window=0, block_table=None, page=16, schedule=None, quantized=False):
     """lfm25_fp8_kv.py:138-167 (e4m3 history + scales) and flash_attn_with_kvcache of lfm25_cuda.py:156-165
@@ -499,6 +537,17 @@ class RowSampler:
         call("lfm2_sample", self.tokens, self.logprobs, logits, self.scratch, seeds, steps, temperatures, 0, 0, 1.0,
              self.batch, self.vocab, _code(logits.dtype))
         return self.tokens, self.logprobs
+
+
+def sample_and_record(sampler: RowSampler, logits, table, input_tokens, stop_table, eos: int, cap: int):
+    """`RowSampler.sample` with the session's per-row seeds, positions and temperatures followed by `record_sample` of
+    the draw (lfm25_session.py:469-482), the record done by the sampler's last launch.  `table` owns the per-row state
+    columns; returns the sampler's reused (tokens, logprobs) buffers."""
+    call("lfm2_sample_record", sampler.tokens, sampler.logprobs, logits, sampler.scratch, table.seeds, table.rng_positions,
+         table.temperatures, table.tokens, table.logprobs, table.lengths, table.limits, table.reasons, table.alive,
+         table.pending, input_tokens, table.stop_states, table.stop_offsets, stop_table, table.ignore_eos,
+         table.rng_positions, int(eos), int(cap), sampler.batch, sampler.vocab, _code(logits.dtype))
+    return sampler.tokens, sampler.logprobs
 
 
 def sample_filtered(logits, *, temperature: float = 1.0, top_k: int = 0, top_p: float = 1.0, seed: int = 0, step: int = 0,

@@ -488,8 +488,13 @@ class LFM25GenerationSession:
             return []
         graph, width = self._graph_for(running)
         state, config = self.rows, self.engine.config
+        fused_record = not self._filtered_rows and not self.behavior_topk
         for _ in range(steps):
             graph.replay()       # consumes the owed token of every row whose pending flag is set
+            if fused_record:     # no redraw and no behaviour head between the draw and its record: one launch less
+                ops.sample_and_record(self.sampler, self.entry.logits, state, self.entry.input_tokens, self.stops.flat,
+                                      config.eos_token_id, self.max_new_tokens)
+                continue
             tokens, logprobs = self._draw()
             if self.behavior_topk:
                 ids, values = ops.behavior_topk(self.entry.logits, tokens, logprobs, self.behavior_topk)

@@ -58,6 +58,12 @@ int lfm2_rms_norm_split(void* out, void* summed, const float* partial, int split
                         const float* w_scales, const void* weight, const void* residual, int64_t M, int64_t H, float eps,
                         int dtype, void* stream);
 
+/* F.embedding followed by the first layer's norm (lfm25_cuda.py:134-137: the first rms_norm of a step has no
+ * residual) in one launch: hidden [M,H] receives the embedding rows (the residual stream), and either out [M,H]
+ * (rms_norm) or q uint8[M,H] with scales float[M] (rms_norm_fp8) their norm.  Same bytes as the two launches. */
+int lfm2_embedding_rms_norm(void* out, uint8_t* q, float* scales, void* hidden, const void* table, const int64_t* tokens,
+                            const void* weight, int64_t M, int64_t H, int64_t V, float eps, int dtype, void* stream);
+
 /* swiglu of lfm25_cuda_kernels.py:58-72.  x [M,2I] (gate first) -> out [M,I]. */
 int lfm2_swiglu(void* out, const void* x, int64_t M, int64_t I, int dtype, void* stream);
 
@@ -207,6 +213,14 @@ int64_t lfm2_decode_attention_workspace(int64_t B, int QH, int D, int64_t capaci
 int lfm2_decode_schedule(int32_t* schedule, const int32_t* positions, const uint8_t* active, const int32_t* slot_ids,
                          int64_t B, void* stream);
 int64_t lfm2_decode_schedule_size(int64_t B, int64_t capacity);
+/* The head of a decode step in one launch (lfm25_cuda.py:128-133,185-186; with `slots`, lfm25_batching.py:11-22,35-46):
+ * positions_out int32[B] = the rows' cache lengths before the step (row b's own slot, or slot slots[b]); the lengths
+ * of the rows that take part advanced by one; the work list of lfm2_decode_schedule for those positions; and, with
+ * `slots` (int32[B], -1 = padding), tokens_out int64[B] and mask_out uint8[B] gathered from input int64[slots] and
+ * active uint8[slots] as lfm2_gather_inputs does.  Without `slots`, `active` is per row and may be NULL (all rows).
+ * Equal to lfm2_gather_inputs + lfm2_decode_schedule before the layers and lfm2_advance_positions after them. */
+int lfm2_decode_begin(int32_t* schedule, int32_t* positions_out, int64_t* tokens_out, uint8_t* mask_out, int32_t* lengths,
+                      const int64_t* input, const uint8_t* active, const int32_t* slots, int64_t B, void* stream);
 
 /* flash_attn_func(causal=True) of lfm25_engine.py:1415-1417 in varlen form: q [T,QH,D], k,v [T,KH,D]
  * packed by cu_seqlens int32[nseq+1]; out [T,QH,D]. */
@@ -277,6 +291,16 @@ int lfm2_record_sample(const int64_t* sampled, const float* logp, int64_t* token
                        uint8_t* pending, int64_t* input, int64_t* stop_states, const int64_t* stop_offsets,
                        const int32_t* stop_table, const uint8_t* ignore_eos, int64_t* rng_positions,
                        int64_t eos, int64_t V, int64_t cap, int64_t B, void* stream);
+/* lfm2_sample with per-row seeds, steps and temperatures, followed by lfm2_record_sample of its draw, in the sampler's
+ * own launches (lfm25_session.py:469-482: RowSampler.sample, then _record_sample): sampled int64[B] and logp float[B]
+ * receive the draw as from lfm2_sample; the record arguments are those of lfm2_record_sample.  `steps` may be the
+ * same array as `rng_positions`: a row's step is read before its position is advanced. */
+int lfm2_sample_record(int64_t* sampled, float* logp, const void* logits, float* scratch, const int64_t* seeds,
+                       const int64_t* steps, const float* temperatures, int64_t* tokens, float* logprobs, int32_t* lengths,
+                       const int32_t* limits, int8_t* reasons, uint8_t* alive, uint8_t* pending, int64_t* input,
+                       int64_t* stop_states, const int64_t* stop_offsets, const int32_t* stop_table,
+                       const uint8_t* ignore_eos, int64_t* rng_positions, int64_t eos, int64_t cap, int64_t B, int64_t V,
+                       int dtype, void* stream);
 /* The per-row state of newly admitted session requests (the state tensors of lfm25_session.py:150-165 as they are set
  * per request at :244-262) written in one launch: specs int64[count, 8] = slot, length limit, seed, random-stream
  * position, stop-automaton state, stop-table offset, flags (bit 0 ignore EOS, bits 8..39 top_k), temperature | top_p

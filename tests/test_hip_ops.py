@@ -927,3 +927,105 @@ def test_kernels_round_where_the_reference_kernels_round(ops):
         q, k, v = ops.prepare_qkv(x, weight, weight, cos, sin, torch.zeros(1, dtype=torch.int32, device=DEV), 1, 1, 64, case["eps"])
         assert q.float().cpu().flatten().tolist() == case["expected"], name
         assert k.float().cpu().flatten().tolist() == case["expected"], name
+
+
+# ------------------------------------------------------------------------------------------------ fused launches
+@pytest.mark.parametrize("fp8", (False, True))
+@torch.inference_mode()
+def test_embedding_fused_into_the_first_norm_equals_the_two_launches(ops, fp8):
+    torch.manual_seed(21)
+    vocab, width = 1000, 2048
+    table = torch.randn(vocab, width, device=DEV).bfloat16()
+    weight = torch.randn(width, device=DEV).bfloat16()
+    tokens = torch.randint(0, vocab, (37,), device=DEV)
+    tokens[3], tokens[4] = -5, vocab + 9          # out-of-range ids are clamped into the table, as `embedding` does
+    hidden = ops.embedding(tokens, table)
+    fused, fused_hidden = ops.embedding_rms_norm(tokens, table, weight, 1e-5, fp8=fp8)
+    assert torch.equal(fused_hidden, hidden)
+    if fp8:
+        q, scales, _ = ops.rms_norm_fp8(hidden, weight, 1e-5)
+        assert torch.equal(fused[0].view(torch.uint8), q.view(torch.uint8)) and torch.equal(fused[1], scales)
+    else:
+        assert torch.equal(fused, ops.rms_norm(hidden, weight, 1e-5)[0])
+    narrow = torch.randn(50, 36, device=DEV).bfloat16()     # a width without 16-byte rows takes the scalar form
+    out, kept = ops.embedding_rms_norm(tokens[:5] % 50, narrow, weight[:36].contiguous(), 1e-5, fp8=False)
+    again = ops.embedding(tokens[:5] % 50, narrow)
+    assert torch.equal(kept, again) and torch.equal(out, ops.rms_norm(again, weight[:36].contiguous(), 1e-5)[0])
+
+
+@torch.inference_mode()
+def test_decode_begin_equals_gather_schedule_and_advance(ops):
+    """The step's first launch against the three it replaces: the same positions, gathered inputs, work list and
+    advanced lengths, for rows that are the cache's slots (with and without a mask) and for a compact batch."""
+    torch.manual_seed(23)
+    rows, capacity = 300, 8192
+    lengths = torch.randint(0, 4000, (rows,), dtype=torch.int32, device=DEV)
+    for active in (None, torch.rand(rows, device=DEV) < 0.7):
+        want_lengths = lengths.clone()
+        want_schedule = ops.decode_schedule(want_lengths, active, None, capacity=capacity)
+        ops.advance_positions(want_lengths, want_lengths.clone(), None, active)
+        got_lengths = lengths.clone()
+        positions, schedule = ops.decode_begin(got_lengths, active, capacity=capacity)
+        assert torch.equal(positions, lengths) and torch.equal(got_lengths, want_lengths)
+        used = 4 + 4 * rows + 4 * int(schedule[0])     # header (pair count, chunk size, two unused words), rows, pairs
+        assert torch.equal(schedule[:2], want_schedule[:2]) and torch.equal(schedule[4:used], want_schedule[4:used])
+    compact = 64
+    slots = torch.full((compact,), -1, dtype=torch.int32, device=DEV)
+    slots[:40] = torch.randperm(rows, device=DEV)[:40].to(torch.int32)
+    slot_active = torch.rand(rows, device=DEV) < 0.8
+    inputs = torch.randint(0, 65536, (rows,), device=DEV)
+    t0, p0, m0 = (torch.zeros(compact, device=DEV, dtype=d) for d in (torch.long, torch.int32, torch.bool))
+    want_lengths = lengths.clone()
+    ops.gather_inputs(t0, p0, m0, inputs, want_lengths, slot_active, slots)
+    want_schedule = ops.decode_schedule(p0, m0, slots, capacity=capacity)
+    ops.advance_positions(want_lengths, p0, slots, m0)
+    t1, p1, m1 = (torch.full((compact,), 7, device=DEV).to(d) for d in (torch.long, torch.int32, torch.bool))
+    got_lengths = lengths.clone()
+    positions, schedule = ops.decode_begin(got_lengths, capacity=capacity, gather=(inputs, slot_active, slots, t1, p1, m1))
+    assert positions is p1 and torch.equal(t1, t0) and torch.equal(p1, p0) and torch.equal(m1, m0)
+    assert torch.equal(got_lengths, want_lengths) and not torch.equal(got_lengths, lengths)
+    used = 4 + 4 * compact + 4 * int(schedule[0])
+    assert torch.equal(schedule[:2], want_schedule[:2]) and torch.equal(schedule[4:used], want_schedule[4:used])
+
+
+@torch.inference_mode()
+def test_sampler_that_records_its_draw_equals_sample_then_record(ops):
+    torch.manual_seed(25)
+    rows, vocab, cap, eos = 9, 10000, 5, 7
+    logits = (torch.randn(rows, vocab, device=DEV) * 2).bfloat16()
+    logits[2, eos] = 50.0                                   # row 2 draws the end-of-sequence token
+    stop_table = torch.zeros(2 * vocab, dtype=torch.int32, device=DEV)
+    stop_table[vocab + logits[4].float().argmax()] = 65536  # row 4 (greedy, second automaton) hits a stop token
+
+    class Table:
+        pass
+
+    def fresh():
+        t = Table()
+        t.seeds = torch.arange(100, 100 + rows, device=DEV)
+        t.rng_positions = torch.arange(rows, device=DEV) * 3
+        t.temperatures = torch.tensor([1.0, 0.0, 1.0, 0.7, 0.0, 1.0, 1.3, 0.0, 1.0], device=DEV)
+        t.tokens = torch.zeros((rows, cap), dtype=torch.long, device=DEV)
+        t.logprobs = torch.zeros((rows, cap), device=DEV)
+        t.lengths = torch.tensor([0, 1, 2, 3, 0, 4, 1, 0, 2], dtype=torch.int32, device=DEV)
+        t.limits = torch.full((rows,), cap, dtype=torch.int32, device=DEV)
+        t.reasons = torch.zeros(rows, dtype=torch.int8, device=DEV)
+        t.alive = torch.tensor([1, 1, 1, 1, 1, 1, 0, 1, 1], dtype=torch.bool, device=DEV)
+        t.pending = torch.zeros(rows, dtype=torch.bool, device=DEV)
+        t.stop_states = torch.zeros(rows, dtype=torch.long, device=DEV)
+        t.stop_offsets = torch.tensor([0, 0, 0, 0, vocab, 0, 0, 0, 0], device=DEV)
+        t.ignore_eos = torch.zeros(rows, dtype=torch.bool, device=DEV)
+        t.input = torch.full((rows,), -1, dtype=torch.long, device=DEV)
+        return t
+
+    two, one = fresh(), fresh()
+    sampler_a, sampler_b = ops.RowSampler(logits), ops.RowSampler(logits)
+    sampled, logp = sampler_a.sample(logits, two.seeds, two.rng_positions, two.temperatures)
+    ops.record_sample(sampled, logp, two.tokens, two.logprobs, two.lengths, two.limits, two.reasons, two.alive, two.pending,
+                      two.input, two.stop_states, two.stop_offsets, stop_table, two.ignore_eos, two.rng_positions, eos, vocab, cap)
+    got_sampled, got_logp = ops.sample_and_record(sampler_b, logits, one, one.input, stop_table, eos, cap)
+    assert torch.equal(got_sampled, sampled) and torch.equal(got_logp.view(torch.int32), logp.view(torch.int32))
+    for name in ("tokens", "logprobs", "lengths", "reasons", "alive", "pending", "stop_states", "rng_positions", "input"):
+        assert torch.equal(getattr(one, name), getattr(two, name)), name
+    assert one.reasons.cpu().tolist()[2] == 1 and one.reasons.cpu().tolist()[4] == 2 and one.reasons.cpu().tolist()[5] == 3
+    assert one.input.cpu().tolist()[6] == -1     # a row that is not alive records nothing
