@@ -357,17 +357,25 @@ def time_decode_attention(engine, session, samples):
     for args in call_args:
         run(args)   # warm
     # consecutive calls walk the layers' caches as the decode step does, so every call streams its history from HBM
-    # (six layers' histories do not fit the memory-side cache); one pair of events per call: the marker between two
-    # calls also keeps the next call's first waves from starting under the tail of this one, which a kernel trace
-    # would count twice
-    marks = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(samples * layers)]
-    for index, (begin, end) in enumerate(marks):
-        begin.record(stream)
-        run(call_args[index % layers])
-        end.record(stream)
-    marks[-1][1].synchronize()
-    total_ms = sum(begin.elapsed_time(end) for begin, end in marks)
-    launches = len(marks)
+    # (six layers' histories do not fit the memory-side cache).  One pair of events around the whole run of calls,
+    # replayed as a graph like the decode step: kernels of one stream do not overlap, so elapsed / calls is the kernels'
+    # durations plus the dispatch gaps between them (an event pair per call would add about 5 us of idle stream to each)
+    launches = samples * layers
+    side = torch.cuda.Stream()   # captured and replayed as one graph: the host's launch cost stays out of the figure
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side), torch.cuda.graph(graph, stream=side):
+        for index in range(launches):
+            run(call_args[index % layers])
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    begin.record(stream)
+    graph.replay()
+    end.record(stream)
+    end.synchronize()
+    total_ms = begin.elapsed_time(end)
+    del graph
     tokens = int((positions.long() + 1).sum())
     kv_token = cfg.num_key_value_heads * cfg.head_dim * 2 * (1 if cache.fp8 else 2) + (cfg.num_key_value_heads * 2 * 4 if cache.fp8 else 0)
     bytes_per_call = tokens * kv_token + 2 * rows * cfg.num_attention_heads * cfg.head_dim * 2
