@@ -46,6 +46,31 @@ def test_fp8_projection_at_benchmark_shapes_matches_dequantised_product_on_sampl
         assert rel < 4e-3, f"M={m}: beyond bf16 output rounding: {rel:.3e}"
 
 
+@pytest.mark.parametrize("k,n,row_counts", [(2048, 11264, (129, 200, 255, 257, 300, 512, 513)),
+                                            (2048, 6144, (129, 200, 255, 257, 300, 512, 513)),
+                                            (2048, 65536, (192, 193, 256, 300, 512, 513))])
+@torch.inference_mode()
+def test_fp8_projection_at_row_counts_where_the_tile_plan_changes(ops, k, n, row_counts):
+    """Ragged row counts on either side of every rule of the default plan for the wide projections (one tile per CU at
+    129-256 and 257-512 rows, the 256 x 256 tile of the vocabulary projection at 193-512 rows): first, last and sampled
+    rows against the dequantised float64 product, every column of those rows."""
+    g = torch.Generator().manual_seed(k + n)
+    weight = (torch.randn(n, k, generator=g) * 0.02).bfloat16().to(DEV)
+    packed = ops.PackedFP8Weight.from_weight(weight)
+    wq = (packed.values.float() * packed.scales[:, None]).double()
+    for m in row_counts:
+        x = torch.randn(m, k, generator=g).bfloat16().to(DEV)
+        xq, xs = ops.quantize_rows(x)
+        out = packed.linear_quantized(xq, xs)
+        assert out.shape == (m, n)
+        rows = torch.unique(torch.cat((torch.tensor([0, m - 1, m // 2, min(m - 1, 127), min(m - 1, 128), min(m - 1, 255), min(m - 1, 256)]),
+                                       torch.randperm(m, generator=g)[:9]))).to(DEV)
+        want = (xq[rows].float() * xs[rows, None]).double() @ wq.T
+        error = (out[rows].double() - want).abs()
+        bound = 2 ** -8 * want.abs() + 1e-3 * want.abs().max()
+        assert bool((error <= bound).all()), f"M={m}: {int((error > bound).sum())} entries off, worst {float((error - bound).max()):.3e}"
+
+
 # ------------------------------------------------------------------------------------------------ config 3
 @pytest.mark.parametrize("fp8", [True, False])
 @torch.inference_mode()
