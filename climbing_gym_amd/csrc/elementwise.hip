@@ -325,7 +325,6 @@ extern "C" int lfm2_rms_norm_split(void* out, void* summed, const float* partial
 }
 
 // ------------------------------------------------------------------------------------ SwiGLU
-__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
 
 template <typename T>
 __global__ void __launch_bounds__(kThreads) swiglu_kernel(T* out, const T* x, int64_t I) {

@@ -94,6 +94,14 @@ struct QkvEpilogue {
   float eps;
 };
 
+// The fused gate+up projection (EPI = 2) walks the packed weight [gate rows; up rows] in an interleaved order: output
+// column n of the product is gate row 8*(n/16) + n%8 when n%16 < 8 and the up row of the same index otherwise, so that
+// every 16-column MFMA tile holds eight gate columns and the eight up columns that pair with them.  Only the addresses
+// of the weight rows and of their scales change; the weight keeps the layout the unfused path reads.
+__device__ __forceinline__ int swiglu_weight_row(int n, int N) {
+  return ((n >> 4) << 3) + (n & 7) + ((n & 8) ? (N >> 1) : 0);
+}
+
 // The kernel body; the two entry points below differ in their arguments only (the fused QKV projection carries its
 // epilogue's arguments, the plain products do not pay for them in every launch's argument block).
 template <int EB, int BM, int BN, int WM, int WN, int SW, int KS, bool KTAIL, int ST, int EPI>
@@ -216,6 +224,7 @@ gemm_nt_body(void* __restrict__ out, float* __restrict__ partial, const uint8_t*
     }
   };
 
+  static_assert(EPI != 2 || ST > 0, "the fused SwiGLU epilogue is built on the ring tiles");
   if constexpr (ST > 0) {
     static_assert(!KTAIL, "direct-to-LDS loads cannot zero-fill a partial K step");
     static_assert(A_CHUNKS % 64 == 0 && W_CHUNKS % 64 == 0, "a wave fills 64 consecutive slots per instruction");
@@ -244,6 +253,7 @@ gemm_nt_body(void* __restrict__ out, float* __restrict__ partial, const uint8_t*
           const int c = lds_slot<SW, kChunksPerRow>(row, slot % kChunksPerRow) - row * kChunksPerRow;
           int gr = n_base + row;
           gr = gr < N ? gr : N - 1;
+          if (EPI == 2) gr = swiglu_weight_row(gr, N);
           __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(W + (int64_t)gr * Kb + kb + c * 16),
                                            (__attribute__((address_space(3))) void*)(&lds[buf][A_CHUNKS + i * NT + wave * 64]), 16, 0, 0);
         }
@@ -416,6 +426,62 @@ gemm_nt_body(void* __restrict__ out, float* __restrict__ partial, const uint8_t*
     return;
   }
 
+  if constexpr (EPI == 2) {
+    // SwiGLU of lfm25_cuda_kernels.py:58-72 on the product's own tile: gate and up values are rounded to the model dtype
+    // as the plain product stores them, then act = round(silu(gate)), out = round(act * up).  In a 16-column tile lane
+    // groups 0, 1 hold gate columns 0-7 and groups 2, 3 the up columns that pair with them; one half-wave swap per value
+    // of two neighbouring tiles leaves lanes 0-31 with gate and up of the first tile and lanes 32-63 with those of the
+    // second, so every lane finishes four outputs.  out is [M, N / 2].
+    auto finish_rows = [&](auto tag) {
+      typedef decltype(tag) T;
+      const int half = lane >> 5, I = N >> 1;
+#pragma unroll
+      for (int i = 0; i < MI; ++i) {
+        const int m = m_base + wm * TM + i * 16 + lrow;
+        const float sa = a_scales ? a_scales[m < M ? m : M - 1] : 1.0f;
+#pragma unroll
+        for (int j = 0; j < NI; j += 2) {
+          const int j1 = j + 1 < NI ? j + 1 : j;
+          float first[4], second[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int n0 = n_base + wn * TN + j * 16 + 4 * lgrp + r, n1 = n_base + wn * TN + j1 * 16 + 4 * lgrp + r;
+            float y0 = acc[i][j][r], y1 = acc[i][j1][r];
+            if (a_scales) {
+              y0 = (y0 * sa) * w_scales[swiglu_weight_row(n0 < N ? n0 : N - 1, N)];
+              y1 = (y1 * sa) * w_scales[swiglu_weight_row(n1 < N ? n1 : N - 1, N)];
+            }
+            const unsigned a = __builtin_bit_cast(unsigned, round_to<T>(y0)), b = __builtin_bit_cast(unsigned, round_to<T>(y1));
+            const auto swapped = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+            first[r] = __builtin_bit_cast(float, (unsigned)swapped[0]);    // gate: tile j in lanes 0-31, tile j1 in lanes 32-63
+            second[r] = __builtin_bit_cast(float, (unsigned)swapped[1]);   // up, same split
+          }
+          const int jj = half ? j1 : j;
+          if (half && j1 == j) continue;          // an odd last tile is finished by the lower half alone
+          const int tile_n = n_base + wn * TN + jj * 16;
+          if (m >= M || tile_n >= N) continue;
+          const int64_t at = (int64_t)m * I + (tile_n >> 1) + 4 * (lgrp & 1);
+          float h[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) h[r] = round_to<T>(round_to<T>(silu_f(first[r])) * second[r]);
+          T* dst = (T*)out + at;
+          if constexpr (sizeof(T) == 2) {
+            typedef T vec4 __attribute__((ext_vector_type(4)));
+            vec4 o = {Elem<T>::store(h[0]), Elem<T>::store(h[1]), Elem<T>::store(h[2]), Elem<T>::store(h[3])};
+            *reinterpret_cast<vec4*>(dst) = o;
+          } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) dst[r] = Elem<T>::store(h[r]);
+          }
+        }
+      }
+    };
+    if (out_dtype == LFM2_DTYPE_BF16) finish_rows(__bf16{});
+    else if (out_dtype == LFM2_DTYPE_F16) finish_rows(_Float16{});
+    else finish_rows(float{});
+    return;
+  }
+
   // Epilogue: lane holds out[m = .. + lrow][n = .. + 4*lgrp + r], r = 0..3.
   const bool split = partial != nullptr;
   auto finish = [&](f32x4 v, int m_out, int n, float sa) {  // scale (row then column) and store up to 4 columns
@@ -466,6 +532,17 @@ gemm_qkv_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ W, co
                 const float* __restrict__ w_scales, int M, int N, int64_t Kb, QkvEpilogue epi) {
   gemm_nt_body<1, 64, 64, 2, 2, 1, 128, false, ST, 1>(nullptr, nullptr, A, W, a_scales, w_scales, M, N, Kb, (int)(Kb / 128),
                                                       LFM2_DTYPE_BF16, RowMap{nullptr, nullptr, 0x7fffffff}, epi);
+}
+
+// The gate+up projection with SwiGLU as its epilogue, on the 8-wave 128 x 128 ring tile of the large-M plan.
+template <int EB>
+__global__ void __launch_bounds__(512)
+gemm_swiglu_kernel(void* __restrict__ out, const uint8_t* __restrict__ A, const uint8_t* __restrict__ W,
+                   const float* __restrict__ a_scales, const float* __restrict__ w_scales, int M, int N, int64_t Kb,
+                   int out_dtype) {
+  gemm_nt_body<EB, 128, 128, 2, 4, EB == 1 ? 1 : 0, 128, false, 2, 2>(out, nullptr, A, W, a_scales, w_scales, M, N, Kb,
+                                                                        (int)(Kb / 128), out_dtype,
+                                                                        RowMap{nullptr, nullptr, 0x7fffffff}, QkvEpilogue{});
 }
 
 // Sum split-K partials in split order, then scale (row scale, then column scale).  A separate launch on purpose:
@@ -714,6 +791,41 @@ extern "C" int lfm2_fp8_gemm(void* out, const uint8_t* a_q, const float* a_scale
   LFM2_REQUIRE(a_scales && w_scales, "fp8_gemm: scales are required");
   LFM2_REQUIRE(split_k <= 16, "fp8_gemm: split_k above 16");
   return gemm_entry<1>("fp8_gemm", out, a_q, a_scales, w_q, w_scales, workspace, M, N, K, out_dtype, tile, split_k, stream);
+}
+
+namespace {
+// The fused form exists for the tile the default plan takes at large M; other shapes use the two launches.
+bool swiglu_fits(int64_t M, int64_t N, int64_t Kb) {
+  if (M <= 0 || N <= 0 || Kb <= 0 || N % 16 != 0 || Kb % kStepBytes != 0 || M >= (1 << 30) || N >= (1 << 30)) return false;
+  const Plan plan = default_plan(M, N, Kb);
+  return plan.tile == 14 && plan.splits == 1;
+}
+template <int EB>
+int swiglu_entry(const char* name, void* out, const void* a, const float* as, const void* w, const float* ws, int64_t M,
+                 int64_t N, int64_t K, int out_dtype, void* stream) {
+  LFM2_REQUIRE(out && a && w, "%s: a required pointer is null", name);
+  LFM2_REQUIRE(out_dtype >= LFM2_DTYPE_BF16 && out_dtype <= LFM2_DTYPE_F32, "%s: bad output dtype", name);
+  LFM2_REQUIRE(((uintptr_t)a | (uintptr_t)w | (uintptr_t)out) % 16 == 0, "%s: pointers must be aligned to 16 bytes", name);
+  if (!swiglu_fits(M, N, K * EB)) LFM2_FAIL(LFM2_ERR_UNSUPPORTED, "%s: no fused form for M %ld, N %ld, K %ld", name, (long)M, (long)N, (long)K);
+  const int tiles = (int)(((M + 127) / 128) * ((N + 127) / 128));
+  hipLaunchKernelGGL(gemm_swiglu_kernel<EB>, dim3((tiles + 7) / 8 * 8), dim3(512), 0, (hipStream_t)stream, out,
+                     (const uint8_t*)a, (const uint8_t*)w, as, ws, (int)M, (int)N, K * EB, out_dtype);
+  LFM2_LAUNCH_CHECK();
+}
+}  // namespace
+
+extern "C" int lfm2_gemm_swiglu_fits(int64_t M, int64_t N, int64_t K, int element_bytes) {
+  return (element_bytes == 1 || element_bytes == 2) && swiglu_fits(M, N, K * element_bytes) ? 1 : 0;
+}
+
+extern "C" int lfm2_fp8_gemm_swiglu(void* out, const uint8_t* a_q, const float* a_scales, const uint8_t* w_q,
+                                    const float* w_scales, int64_t M, int64_t N, int64_t K, int out_dtype, void* stream) {
+  LFM2_REQUIRE(a_scales && w_scales, "fp8_gemm_swiglu: scales are required");
+  return swiglu_entry<1>("fp8_gemm_swiglu", out, a_q, a_scales, w_q, w_scales, M, N, K, out_dtype, stream);
+}
+
+extern "C" int lfm2_bf16_gemm_swiglu(void* out, const void* x, const void* w, int64_t M, int64_t N, int64_t K, void* stream) {
+  return swiglu_entry<2>("bf16_gemm_swiglu", out, x, nullptr, w, nullptr, M, N, K, LFM2_DTYPE_BF16, stream);
 }
 
 extern "C" int lfm2_fp8_gemm_qkv_store(void* q, const uint8_t* a_q, const float* a_scales, const uint8_t* w_q,

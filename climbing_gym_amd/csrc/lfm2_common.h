@@ -52,6 +52,10 @@ template <> struct Elem<float> {
 // Round an fp32 value to the model dtype and return it as fp32 again.
 template <typename T> __device__ __forceinline__ float round_to(float v) { return Elem<T>::load(Elem<T>::store(v)); }
 
+// SiLU as the SwiGLU kernels compute it (one definition, so that a fused epilogue and the stand-alone kernels give the
+// same bits).
+__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
+
 // ---- wave / block reductions (64-lane wavefronts) ----------------------------------
 // All-reduce butterflies that stay in the vector ALU: two quad permutes, the two row mirrors (lane i <-> 7-i, then
 // i <-> 15-i: by then each half already holds one value, so a mirror pairs the halves), and gfx950's row and

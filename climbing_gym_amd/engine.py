@@ -308,13 +308,22 @@ class LFM25Engine:
             else:
                 op = layer.conv
                 mixed = self._linear(conv_op(op, self._project(normed, op.in_weight, fp8)), op.out_weight, fp8)
-            gate_up, residual = self._norm_linear(mixed, layer.ffn_norm_weight, residual, layer.w13_weight, fp8)
-            down = fp8.get(id(layer.w2_weight))
-            if down is not None:
-                q, scales = ops.swiglu_fp8(gate_up)
+            # gate+up projection and SwiGLU: one launch where the product's shape has the fused form (packed prefill
+            # chunks), the projection and the SwiGLU launch otherwise (decode); the same bits either way
+            normed, residual = self._normed(mixed, layer.ffn_norm_weight, residual, layer.w13_weight, fp8)
+            gate_up, down = fp8.get(id(layer.w13_weight)), fp8.get(id(layer.w2_weight))
+            if gate_up is not None and down is not None:
+                q, scales = gate_up.linear_swiglu_quantized(normed[0], normed[1], dtype=self.dtype)
                 hidden = down.linear_quantized(q, scales, dtype=self.dtype, defer_reduce=defer_reduce)
-            else:
-                hidden = ops.linear(ops.swiglu(gate_up), layer.w2_weight, defer_reduce=defer_reduce)
+            elif gate_up is None and down is None:
+                hidden = ops.linear(ops.linear_swiglu(normed, layer.w13_weight), layer.w2_weight, defer_reduce=defer_reduce)
+            else:   # only one of the two MLP projections has an e4m3 copy
+                product = self._project(normed, layer.w13_weight, fp8)
+                if down is not None:
+                    q, scales = ops.swiglu_fp8(product)
+                    hidden = down.linear_quantized(q, scales, dtype=self.dtype, defer_reduce=defer_reduce)
+                else:
+                    hidden = ops.linear(ops.swiglu(product), layer.w2_weight, defer_reduce=defer_reduce)
         return hidden, residual
 
     def _head(self, hidden, residual, fp8, place=None):

@@ -309,6 +309,22 @@ def linear(x: torch.Tensor, weight: torch.Tensor, *, tile: int = -1, split_k: in
     return out
 
 
+def linear_swiglu(x: torch.Tensor, weight: torch.Tensor):
+    """`swiglu(linear(x, weight))` for the packed gate+up weight [2I, K] (lfm25_cuda_kernels.py:19-29 then :58-72),
+    the same bits, in one launch where the product's shape has the fused form and in the two launches otherwise."""
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise ValueError("linear runs in bfloat16 only: this package has no GEMM for other dtypes")
+    _check(x, weight)
+    m, k, n = _rows(x), x.size(-1), weight.size(0)
+    if weight.size(1) != k or n % 2:
+        raise ValueError("activation and weight widths differ, or the packed gate+up weight has an odd row count")
+    if x.ndim != 2 or not query("lfm2_gemm_swiglu_fits", m, n, k, 2):
+        return swiglu(linear(x, weight))
+    out = torch.empty((m, n // 2), device=x.device, dtype=x.dtype)
+    call("lfm2_bf16_gemm_swiglu", out, x, weight, m, n, k)
+    return out
+
+
 @dataclass
 class PackedFP8Weight:
     """lfm25_fp8.py:120-168: per-output-channel e4m3 copy of a weight.  `refresh()` re-quantises into the
@@ -354,6 +370,20 @@ class PackedFP8Weight:
         ws = torch.empty(need, device=x.device, dtype=torch.float32) if need and split_k != 1 else None
         call("lfm2_fp8_gemm", out, x, scales, self.values, self.scales, ws, batch, rows, width, _code(dtype), tile, split_k)
         return out
+
+    def linear_swiglu_quantized(self, x, scales, *, dtype=torch.bfloat16):
+        """For the packed gate+up weight: `swiglu_fp8(self.linear_quantized(x, scales))` (lfm25_fp8.py:141-168 then
+        :67-73) as (e4m3 rows, row scales), the same bits; where the product's shape has the fused form the SwiGLU runs
+        in the projection's epilogue and only [M, I] is written and quantised, otherwise the two launches run."""
+        batch, width = x.shape
+        rows = self.values.size(0)
+        if width != self.values.size(1) or rows % 2:
+            raise ValueError("FP8 activation and weight widths differ, or the packed gate+up weight has an odd row count")
+        if not query("lfm2_gemm_swiglu_fits", batch, rows, width, 1):
+            return swiglu_fp8(self.linear_quantized(x, scales, dtype=dtype))
+        hidden = torch.empty((batch, rows // 2), device=x.device, dtype=dtype)
+        call("lfm2_fp8_gemm_swiglu", hidden, x, scales, self.values, self.scales, batch, rows, width, _code(dtype))
+        return quantize_rows(hidden)
 
 
 # ----------------------------------------------------------------------------------- KV cache + attention

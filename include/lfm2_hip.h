@@ -152,6 +152,17 @@ int lfm2_bf16_gemm_partials(float* partials, const void* x, const void* w, int64
                             int split_k, void* stream);
 int64_t lfm2_bf16_gemm_default_splits(int64_t M, int64_t N, int64_t K);
 
+/* The gate+up projection with SwiGLU as its epilogue: w[N, K] is the packed weight [gate rows; up rows] (N = 2 I) in
+ * the layout lfm2_fp8_gemm / lfm2_bf16_gemm read; out[M, I] = round(round(silu(gate)) * up) with gate and up the
+ * product's columns rounded to the output type first, i.e. bit for bit lfm2_fp8_gemm (lfm25_fp8.py:141-168) or
+ * lfm2_bf16_gemm followed by lfm2_swiglu (lfm25_cuda_kernels.py:58-72), without the [M, 2 I] intermediate.  Built on
+ * one tile shape: lfm2_gemm_swiglu_fits(M, N, K, element bytes of the operands: 1 or 2) says whether a shape has the
+ * fused form (1) or needs the two launches (0); the fused entry points return LFM2_ERR_UNSUPPORTED for the latter. */
+int lfm2_gemm_swiglu_fits(int64_t M, int64_t N, int64_t K, int element_bytes);
+int lfm2_fp8_gemm_swiglu(void* out, const uint8_t* a_q, const float* a_scales, const uint8_t* w_q, const float* w_scales,
+                         int64_t M, int64_t N, int64_t K, int out_dtype, void* stream);
+int lfm2_bf16_gemm_swiglu(void* out, const void* x, const void* w, int64_t M, int64_t N, int64_t K, void* stream);
+
 /* The two products with placed output rows: row m of the product is written to out row out_rows[m] (m itself when
  * out_rows is NULL) unless that index is negative or >= out_capacity, or row_active[m] is 0 (row_active may be
  * NULL); other rows of out keep their contents.  This is the head projection followed by _scatter_logits of

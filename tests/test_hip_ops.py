@@ -1029,3 +1029,28 @@ def test_sampler_that_records_its_draw_equals_sample_then_record(ops):
         assert torch.equal(getattr(one, name), getattr(two, name)), name
     assert one.reasons.cpu().tolist()[2] == 1 and one.reasons.cpu().tolist()[4] == 2 and one.reasons.cpu().tolist()[5] == 3
     assert one.input.cpu().tolist()[6] == -1     # a row that is not alive records nothing
+
+
+@pytest.mark.parametrize("fp8", (True, False))
+@pytest.mark.parametrize("m,k,inner", [(4096, 256, 512), (2689, 2048, 5632), (1000, 384, 5632), (300, 2048, 5632), (64, 2048, 5632)])
+@torch.inference_mode()
+def test_gate_up_projection_with_swiglu_epilogue_equals_the_two_launches(ops, fp8, m, k, inner):
+    """The fused gate+up projection (SwiGLU in the product's epilogue, [M, I] written) against the projection followed
+    by the SwiGLU launch, bit for bit: both quantised outputs for W8A8, the bf16 rows otherwise.  The last shape has no
+    fused form and must take the two launches by itself; a ragged row count ends inside a tile."""
+    torch.manual_seed(m + inner)
+    weight = (torch.randn(2 * inner, k, device=DEV) * 0.05).bfloat16()
+    x = torch.randn(m, k, device=DEV).bfloat16()
+    fused_exists = bool(ops.query("lfm2_gemm_swiglu_fits", m, 2 * inner, k, 1 if fp8 else 2))
+    assert fused_exists == (m > 64)
+    if fp8:
+        packed = ops.PackedFP8Weight.from_weight(weight)
+        xq, xs = ops.quantize_rows(x)
+        want_q, want_s = ops.swiglu_fp8(packed.linear_quantized(xq, xs))
+        got_q, got_s = packed.linear_swiglu_quantized(xq, xs)
+        assert torch.equal(got_s, want_s)
+        assert torch.equal(got_q.view(torch.uint8), want_q.view(torch.uint8))
+    else:
+        want = ops.swiglu(ops.linear(x, weight))
+        got = ops.linear_swiglu(x, weight)
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16))
