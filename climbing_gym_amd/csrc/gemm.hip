@@ -534,15 +534,16 @@ gemm_qkv_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ W, co
                                                       LFM2_DTYPE_BF16, RowMap{nullptr, nullptr, 0x7fffffff}, epi);
 }
 
-// The gate+up projection with SwiGLU as its epilogue, on the 8-wave 128 x 128 ring tile of the large-M plan.
-template <int EB>
-__global__ void __launch_bounds__(512)
+// The gate+up projection with SwiGLU as its epilogue, on the tiles the default plan gives that projection: the 8-wave
+// 128 x 128 ring tile at large M and the 16-wave 128 x 96 tile of the decode batch.
+template <int EB, int BM, int BN, int WM, int WN, int ST>
+__global__ void __launch_bounds__(WM * WN * 64)
 gemm_swiglu_kernel(void* __restrict__ out, const uint8_t* __restrict__ A, const uint8_t* __restrict__ W,
                    const float* __restrict__ a_scales, const float* __restrict__ w_scales, int M, int N, int64_t Kb,
                    int out_dtype) {
-  gemm_nt_body<EB, 128, 128, 2, 4, EB == 1 ? 1 : 0, 128, false, 2, 2>(out, nullptr, A, W, a_scales, w_scales, M, N, Kb,
-                                                                        (int)(Kb / 128), out_dtype,
-                                                                        RowMap{nullptr, nullptr, 0x7fffffff}, QkvEpilogue{});
+  gemm_nt_body<EB, BM, BN, WM, WN, EB == 1 ? 1 : 0, 128, false, ST, 2>(out, nullptr, A, W, a_scales, w_scales, M, N, Kb,
+                                                                         (int)(Kb / 128), out_dtype,
+                                                                         RowMap{nullptr, nullptr, 0x7fffffff}, QkvEpilogue{});
 }
 
 // Sum split-K partials in split order, then scale (row scale, then column scale).  A separate launch on purpose:
@@ -798,7 +799,7 @@ namespace {
 bool swiglu_fits(int64_t M, int64_t N, int64_t Kb) {
   if (M <= 0 || N <= 0 || Kb <= 0 || N % 16 != 0 || Kb % kStepBytes != 0 || M >= (1 << 30) || N >= (1 << 30)) return false;
   const Plan plan = default_plan(M, N, Kb);
-  return plan.tile == 14 && plan.splits == 1;
+  return (plan.tile == 14 || plan.tile == 36) && plan.splits == 1;
 }
 template <int EB>
 int swiglu_entry(const char* name, void* out, const void* a, const float* as, const void* w, const float* ws, int64_t M,
@@ -807,9 +808,15 @@ int swiglu_entry(const char* name, void* out, const void* a, const float* as, co
   LFM2_REQUIRE(out_dtype >= LFM2_DTYPE_BF16 && out_dtype <= LFM2_DTYPE_F32, "%s: bad output dtype", name);
   LFM2_REQUIRE(((uintptr_t)a | (uintptr_t)w | (uintptr_t)out) % 16 == 0, "%s: pointers must be aligned to 16 bytes", name);
   if (!swiglu_fits(M, N, K * EB)) LFM2_FAIL(LFM2_ERR_UNSUPPORTED, "%s: no fused form for M %ld, N %ld, K %ld", name, (long)M, (long)N, (long)K);
-  const int tiles = (int)(((M + 127) / 128) * ((N + 127) / 128));
-  hipLaunchKernelGGL(gemm_swiglu_kernel<EB>, dim3((tiles + 7) / 8 * 8), dim3(512), 0, (hipStream_t)stream, out,
-                     (const uint8_t*)a, (const uint8_t*)w, as, ws, (int)M, (int)N, K * EB, out_dtype);
+  const int tile = default_plan(M, N, K * EB).tile;
+  const int tiles = (int)(((M + kTiles[tile].bm - 1) / kTiles[tile].bm) * ((N + kTiles[tile].bn - 1) / kTiles[tile].bn));
+  const dim3 grid((tiles + 7) / 8 * 8);
+  if (tile == 14)
+    hipLaunchKernelGGL((gemm_swiglu_kernel<EB, 128, 128, 2, 4, 2>), grid, dim3(512), 0, (hipStream_t)stream, out,
+                       (const uint8_t*)a, (const uint8_t*)w, as, ws, (int)M, (int)N, K * EB, out_dtype);
+  else
+    hipLaunchKernelGGL((gemm_swiglu_kernel<EB, 128, 96, 8, 2, 3>), grid, dim3(1024), 0, (hipStream_t)stream, out,
+                       (const uint8_t*)a, (const uint8_t*)w, as, ws, (int)M, (int)N, K * EB, out_dtype);
   LFM2_LAUNCH_CHECK();
 }
 }  // namespace

@@ -1032,12 +1032,13 @@ def test_sampler_that_records_its_draw_equals_sample_then_record(ops):
 
 
 @pytest.mark.parametrize("fp8", (True, False))
-@pytest.mark.parametrize("m,k,inner", [(4096, 256, 512), (2689, 2048, 5632), (1000, 384, 5632), (300, 2048, 5632), (64, 2048, 5632)])
+@pytest.mark.parametrize("m,k,inner", [(4096, 256, 512), (2689, 2048, 5632), (1000, 384, 5632), (300, 2048, 5632), (256, 2048, 5632), (200, 2048, 5632), (64, 2048, 5632)])
 @torch.inference_mode()
 def test_gate_up_projection_with_swiglu_epilogue_equals_the_two_launches(ops, fp8, m, k, inner):
     """The fused gate+up projection (SwiGLU in the product's epilogue, [M, I] written) against the projection followed
     by the SwiGLU launch, bit for bit: both quantised outputs for W8A8, the bf16 rows otherwise.  The last shape has no
-    fused form and must take the two launches by itself; a ragged row count ends inside a tile."""
+    fused form and must take the two launches by itself; ragged row counts end inside a tile; 256 and 200 rows run
+    the decode batch's 128 x 96 tile (three MFMA tiles per wave: the odd one is finished by half of the lanes)."""
     torch.manual_seed(m + inner)
     weight = (torch.randn(2 * inner, k, device=DEV) * 0.05).bfloat16()
     x = torch.randn(m, k, device=DEV).bfloat16()
