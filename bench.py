@@ -105,6 +105,34 @@ def gemm_workload(args):
             table[f"{name} n{n} k{k} m{m}"] = {"us": round(sec * 1e6, 2), "GBps": round(moved / sec / 1e9, 1),
                                                "TFLOPs": round(2 * m * n * k / sec / 1e12, 1)}
             del graph
+            if name == "w13" and m in (256, 4096):
+                # the MLP's first half as the engine runs it: projection, SwiGLU and per-token e4m3 rows for the down
+                # projection; with the SwiGLU in the product's epilogue, and as projection + SwiGLU launch
+                def timed(step):
+                    def body():
+                        for _ in range(repeats):
+                            for p in packs:
+                                step(p)
+                    body()
+                    torch.cuda.synchronize()
+                    side, graph = torch.cuda.Stream(), torch.cuda.CUDAGraph()
+                    with torch.cuda.stream(side), torch.cuda.graph(graph, stream=side):
+                        body()
+                    torch.cuda.synchronize()
+                    graph.replay()
+                    begin.record(stream)
+                    for _ in range(args.steps):
+                        graph.replay()
+                    end.record(stream)
+                    end.synchronize()
+                    return begin.elapsed_time(end) * 1000 / (args.steps * repeats * copies)
+                fused = timed(lambda p: p.linear_swiglu_quantized(xq, xs))
+                apart = timed(lambda p: ops.swiglu_fp8(p.linear_quantized(xq, xs)))
+                a, b = packs[0].linear_swiglu_quantized(xq, xs), ops.swiglu_fp8(packs[0].linear_quantized(xq, xs))
+                if not (torch.equal(a[0].view(torch.uint8), b[0].view(torch.uint8)) and torch.equal(a[1], b[1])):
+                    raise SystemExit(f"fused gate+up projection differs from the two launches at {m} rows")
+                table[f"w13 + swiglu + quantise m{m}"] = {"fused_us": round(fused, 2), "two_launches_us": round(apart, 2),
+                                                          "fused_TFLOPs": round(2 * m * n * k / fused / 1e6, 1)}
         del packs
         torch.cuda.empty_cache()
     big, small = table["w13 n11264 k2048 m4096"], table["w13 n11264 k2048 m256"]
