@@ -647,11 +647,18 @@ schedule_rows(int32_t* schedule, const int32_t* positions, const uint8_t* active
 #pragma unroll
     for (int k = 0; k < kSchedClasses; ++k) mine[k] += n[k];
   }
+  // a row has at most one partial chunk, so with one row per thread (B <= 1024, every decode batch) the partial
+  // classes are counted with ballots instead of shuffle trees; only the full-chunk counts need a sum
+  const bool one_sweep = B <= 1024;
 #pragma unroll
   for (int k = 0; k < kSchedClasses; ++k) {
     int v = mine[k];
+    if (k > 0 && one_sweep) {
+      v = __popcll(__ballot(v != 0));
+    } else {
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+      for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    }
     if (lane == 0) wave_total[k][wave] = v;
   }
   __syncthreads();
@@ -672,16 +679,23 @@ schedule_rows(int32_t* schedule, const int32_t* positions, const uint8_t* active
     const int len = row_length(b);
     int n[kSchedClasses], before[kSchedClasses];
     classify(len, n);
+    const unsigned long long below = (1ull << lane) - 1;
 #pragma unroll
-    for (int k = 0; k < kSchedClasses; ++k) {   // inclusive scan over the wave
-      int v = n[k];
+    for (int k = 0; k < kSchedClasses; ++k) {   // exclusive scan over the wave, and the wave's total
+      if (k > 0) {                              // 0 or 1 per row: positions of the set lanes
+        const unsigned long long set = __ballot(n[k] != 0);
+        before[k] = __popcll(set & below);
+        if (lane == 63) wave_total[k][wave] = __popcll(set);
+      } else {
+        int v = n[k];
 #pragma unroll
-      for (int o = 1; o < 64; o <<= 1) {
-        const int up = __shfl_up(v, o, 64);
-        if (lane >= o) v += up;
+        for (int o = 1; o < 64; o <<= 1) {
+          const int up = __shfl_up(v, o, 64);
+          if (lane >= o) v += up;
+        }
+        before[k] = v - n[k];
+        if (lane == 63) wave_total[k][wave] = v;
       }
-      before[k] = v - n[k];
-      if (lane == 63) wave_total[k][wave] = v;
     }
     __syncthreads();
     int first[kSchedClasses];
