@@ -21,6 +21,7 @@ from .config import LFM25SamplingConfig
 from .inference_config import InferenceEngineConfig, SamplingConfig
 from .text_stops import build_stop_table, trim_after_stop
 from .types import BehaviorTopK, GenerationOutput, GenerationResult, PromptInput
+from ._checks import reject
 
 _MASK63 = 0x7FFFFFFFFFFFFFFF
 _CHAIN_STRIDE = 0x517CC1B727220A95   # odd 64-bit constants: chain and phase index spread over the whole key
@@ -43,10 +44,8 @@ def chain_seed(base: int, chain: int, phase: int) -> int:
 def to_native_sampling(sampling: SamplingConfig, *, seed: int, tokenizer=None) -> LFM25SamplingConfig:
     """Request-level sampling -> engine sampling (lfm25_async_engine.py:688-709).  String stops become the token
     sequences of the stop text after the usual joiners; `top_k == -1` means no top-k."""
-    if int(sampling.n) != 1:
-        raise ValueError("LFM25AsyncInferenceEngine requires sampling.n == 1")
-    if sampling.stop and tokenizer is None:
-        raise ValueError("A tokenizer is required for string stop sequences")
+    reject(int(sampling.n) != 1, "LFM25AsyncInferenceEngine requires sampling.n == 1")
+    reject(sampling.stop and tokenizer is None, "A tokenizer is required for string stop sequences")
     extra = dict(sampling.extra_params)
     sequences = []
     for text in sampling.stop:
@@ -62,8 +61,8 @@ def to_native_sampling(sampling: SamplingConfig, *, seed: int, tokenizer=None) -
 
 
 def _batch_limit(config: InferenceEngineConfig, requested) -> int:
-    if requested is not None and (type(requested) is not int or requested <= 0):
-        raise ValueError("max_batch_size must be a positive integer")
+    reject(requested is not None and (type(requested) is not int or requested <= 0),
+           "max_batch_size must be a positive integer")
     limit = requested if requested is not None else (config.max_num_seqs or 64)
     return limit if config.max_num_seqs is None else min(limit, config.max_num_seqs)
 
@@ -91,8 +90,8 @@ class _PromptRenderer:
         if not self.config.apply_chat_template:
             return str(prompt)
         template = getattr(self.tokenizer, "apply_chat_template", None)
-        if not callable(template):
-            raise TypeError("apply_chat_template=true requires a tokenizer with apply_chat_template(...)")
+        reject(not callable(template),
+               "apply_chat_template=true requires a tokenizer with apply_chat_template(...)", TypeError)
         thinking = self.config.chat_template_enable_thinking if enable_thinking is None else enable_thinking
         messages = [{"role": "user", "content": str(prompt)}]
         options = {"tokenize": False, "add_generation_prompt": True}
@@ -142,8 +141,7 @@ class LFM25AsyncInferenceEngine:
         del compile_decode, bf16_weight_packing  # no tracing compiler and no separate bf16 packing on this path
         for flag, name in ((fp8_mlp, "FP8 MLP"), (fp8_kv, "FP8 KV cache"), (adaptive_batching, "adaptive batching"),
                            (fp8_lm_head, "FP8 vocabulary head"), (fp8_operators, "FP8 operators")):
-            if flag and not cuda_graphs:
-                raise ValueError(f"Native {name} requires cuda_graphs=True")
+            reject(flag and not cuda_graphs, f"Native {name} requires cuda_graphs=True")
         from transformers import AutoTokenizer
         from .engine import LFM25Engine
         tokenizer = AutoTokenizer.from_pretrained(config.model_path, local_files_only=True)
@@ -188,8 +186,7 @@ class LFM25AsyncInferenceEngine:
     # ------------------------------------------------------------------ small public surface
     @property
     def raw_engine(self):
-        if self._engine is None:
-            raise RuntimeError("LFM25AsyncInferenceEngine is closed")
+        reject(self._engine is None, "LFM25AsyncInferenceEngine is closed", RuntimeError)
         return self._engine
 
     def supports_token_prompt_bridge(self) -> bool:
@@ -210,14 +207,12 @@ class LFM25AsyncInferenceEngine:
                                                   enable_thinking=chat_template_enable_thinking)[2]
 
     def _check_open(self):
-        if self._closed:
-            raise RuntimeError("LFM25AsyncInferenceEngine is closed")
+        reject(self._closed, "LFM25AsyncInferenceEngine is closed", RuntimeError)
 
     def sync_from_model(self, model, *, drain_timeout: int | float = 300):
         """Wait for running generation to drain, then update the packed weights in place."""
         timeout = float(drain_timeout)
-        if not math.isfinite(timeout) or timeout < 0.0:
-            raise ValueError("drain_timeout must be finite and >= 0")
+        reject(not math.isfinite(timeout) or timeout < 0.0, "drain_timeout must be finite and >= 0")
         self._check_open()
         if not self._engine_lock.acquire(timeout=timeout):
             raise TimeoutError(f"Timed out after {timeout:g}s waiting for native LFM2.5 generation to drain")
@@ -265,8 +260,8 @@ class LFM25AsyncInferenceEngine:
             return self.config.default_sampling
         if isinstance(sampling, SamplingConfig):
             return sampling
-        if isinstance(sampling, Mapping):
-            raise TypeError("sampling must be a SamplingConfig or a sampling-attribute object, not a mapping")
+        reject(isinstance(sampling, Mapping),
+               "sampling must be a SamplingConfig or a sampling-attribute object, not a mapping", TypeError)
         read = lambda name, default: getattr(sampling, name, default)
         return SamplingConfig(temperature=float(read("temperature", 0.0)), top_k=int(read("top_k", -1)),
                               top_p=float(read("top_p", 1.0)),
@@ -483,8 +478,8 @@ class LFM25AsyncInferenceEngine:
                                       slots=[slot for slot, _ in restarted])
                         running.update(restarted)
                 self.last_session_stats = dict(session.stats)
-            if self._closed and not cancelled.is_set():
-                raise RuntimeError("LFM25AsyncInferenceEngine closed during generation")
+            reject(self._closed and not cancelled.is_set(),
+                   "LFM25AsyncInferenceEngine closed during generation", RuntimeError)
             return results
 
 

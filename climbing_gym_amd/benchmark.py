@@ -24,6 +24,7 @@ import torch
 
 from .config import LFM2Config, LFM25SamplingConfig
 from .engine import LFM25Engine, flatten_token_batches
+from ._checks import reject
 
 SCHEDULER_NOTE = "synchronous fixed batches; no hidden request concurrency cap"
 SHAPES = ("tiny", "lfm2-1.2b")
@@ -157,13 +158,13 @@ def measure_batch(engine, rows, sampling, *, batch, output_tokens, warmups, repe
         tokens, logprobs, lengths = output.token_ids.cpu(), output.logprobs.cpu(), output.lengths.cpu()
         if output.topk_token_ids is not None:
             output.topk_token_ids.cpu()
-            if not bool(torch.isfinite(output.topk_logprobs.cpu()).all()):
-                raise RuntimeError("Native rollout returned non-finite sparse behavior logprobs")
+            reject(not bool(torch.isfinite(output.topk_logprobs.cpu()).all()),
+                   "Native rollout returned non-finite sparse behavior logprobs", RuntimeError)
         sync()
         seconds = time.perf_counter() - started
         count = int(lengths.sum())
-        if count != batch * output_tokens or not bool(torch.isfinite(logprobs).all()):
-            raise RuntimeError("Native rollout returned an incomplete budget or non-finite logprobs")
+        reject(count != batch * output_tokens or not bool(torch.isfinite(logprobs).all()),
+               "Native rollout returned an incomplete budget or non-finite logprobs", RuntimeError)
         runs.append({"seconds": seconds, "output_tokens": count, "tokens_per_second": count / seconds})
     entry = {"batch_size": batch, "max_num_seqs": batch, "max_inflight_requests": batch, "runs": runs,
              "median_tokens_per_second": statistics.median(run["tokens_per_second"] for run in runs),
@@ -190,8 +191,7 @@ def check_report(report, batch_size: int) -> dict:
     """What the report's reader requires of the entry for `batch_size` (`preflight.py:60-79`): positive median rate,
     positive peak memory on a GPU, at least one run, every run complete.  Returns the entry."""
     def positive(value, name):
-        if not isinstance(value, (int, float)) or not value > 0:
-            raise ValueError(f"Native preflight report has no positive {name}")
+        reject(not isinstance(value, (int, float)) or not value > 0, f"Native preflight report has no positive {name}")
     for entry in report.get("batches", []):
         if int(entry.get("batch_size", 0)) != batch_size:
             continue
@@ -199,13 +199,12 @@ def check_report(report, batch_size: int) -> dict:
         if str(report["config"].get("device", "cuda")).startswith("cuda"):
             positive(entry.get("peak_allocated_bytes", 0), "peak_allocated_bytes")
             positive(entry.get("peak_reserved_bytes", 0), "peak_reserved_bytes")
-        if not entry.get("runs"):
-            raise ValueError("Native preflight report contains no measured rollouts")
+        reject(not entry.get("runs"), "Native preflight report contains no measured rollouts")
         for run in entry["runs"]:
             positive(run.get("seconds", 0), "rollout seconds")
             positive(run.get("tokens_per_second", 0), "rollout tokens_per_second")
-            if int(run.get("output_tokens", 0)) != batch_size * int(report["config"]["output_tokens"]):
-                raise ValueError("Native preflight report did not complete the intended token budget")
+            reject(int(run.get("output_tokens", 0)) != batch_size * int(report["config"]["output_tokens"]),
+                   "Native preflight report did not complete the intended token budget")
         return entry
     raise ValueError(f"Native preflight report must benchmark resolved batch size {batch_size}")
 

@@ -59,47 +59,45 @@ class LFM25HybridCache:
 
     def store_prefill(self, layer: int, k: torch.Tensor, v: torch.Tensor, *, start: int = 0) -> None:
         """Write [batch, tokens, KV heads, D] (or one [tokens, KV heads, D]) at positions 0.. of slots start.."""
-        if k.ndim == 3:
-            k, v = k.unsqueeze(0), v.unsqueeze(0)
-        end, length = start + k.size(0), k.size(1)
-        kc, vc = self.k_cache[layer, start:end, :length], self.v_cache[layer, start:end, :length]
-        if self.k_scales is None:
-            kc.copy_(k)
-            vc.copy_(v)
+        keys, values = (k[None], v[None]) if k.ndim == 3 else (k, v)
+        rows, span = slice(start, start + keys.size(0)), slice(0, keys.size(1))
+        targets = self.k_cache[layer, rows, span], self.v_cache[layer, rows, span]
+        if self.fp8:
+            ops.store_kv(keys, values, *targets, self.k_scales[layer, rows, span], self.v_scales[layer, rows, span])
         else:
-            ops.store_kv(k, v, kc, vc, self.k_scales[layer, start:end, :length], self.v_scales[layer, start:end, :length])
+            for target, source in zip(targets, (keys, values)):
+                target.copy_(source)
 
     def copy_prefix_from(self, source: "LFM25HybridCache", slots: torch.Tensor, length: int) -> None:
         """self[i] <- source[slots[i]] for the first `length` positions, conv state and lengths
-        (lfm25_engine.py:400-423).  Byte-identical when both caches use the same storage; an e4m3 source is
-        dequantised into a model-dtype destination."""
-        same = self.k_cache.dtype == source.k_cache.dtype and self.fp8 == source.fp8
-        slots = slots.to(self.seq_lens.device, torch.long)
-        for layer in range(self.k_cache.size(0)):
-            def pick(t):
-                part = t[layer, :, :length]
-                if part.element_size() == 1:
-                    return part.view(torch.uint8).index_select(0, slots).view(part.dtype)
-                return part.index_select(0, slots)
-            k, v = pick(source.k_cache), pick(source.v_cache)
-            if same:
-                if k.element_size() == 1:
-                    self.k_cache[layer, :, :length].view(torch.uint8).copy_(k.view(torch.uint8))
-                    self.v_cache[layer, :, :length].view(torch.uint8).copy_(v.view(torch.uint8))
-                else:
-                    self.k_cache[layer, :, :length].copy_(k)
-                    self.v_cache[layer, :, :length].copy_(v)
+        (lfm25_engine.py:400-423).  Byte-identical when both caches use the same storage (all layers in one gather per
+        tensor); an e4m3 source is dequantised into a model-dtype destination."""
+        order = slots.to(self.seq_lens.device, torch.long)
+        head = lambda t: _bytes(t[:, :, :length])                     # [layers, slots, positions, ...] as raw bytes
+        taken = lambda t: head(t).index_select(1, order)
+        mine = [self.k_cache, self.v_cache, self.k_scales, self.v_scales]
+        theirs = [source.k_cache, source.v_cache, source.k_scales, source.v_scales]
+        if self.fp8 == source.fp8 and self.k_cache.dtype == source.k_cache.dtype:
+            for target, origin in zip(mine, theirs):
+                if target is not None:
+                    head(target).copy_(taken(origin))
+        else:
+            for layer in range(self.k_cache.size(0)):
+                pick = lambda t: t[layer, :, :length].index_select(0, order) if t.element_size() > 1 else \
+                    t[layer, :, :length].view(torch.uint8).index_select(0, order).view(t.dtype)
+                keys, values = pick(source.k_cache), pick(source.v_cache)
                 if source.fp8:
-                    self.k_scales[layer, :, :length].copy_(pick(source.k_scales))
-                    self.v_scales[layer, :, :length].copy_(pick(source.v_scales))
-                continue
-            if source.fp8:
-                k = (k.float() * pick(source.k_scales)[..., None]).to(self.conv_state.dtype)
-                v = (v.float() * pick(source.v_scales)[..., None]).to(self.conv_state.dtype)
-            self.store_prefill(layer, k.contiguous(), v.contiguous())
-        self.conv_state.copy_(source.conv_state.index_select(1, slots))
-        self.seq_lens.copy_(source.seq_lens.index_select(0, slots))
+                    keys = (keys.float() * pick(source.k_scales)[..., None]).to(self.conv_state.dtype)
+                    values = (values.float() * pick(source.v_scales)[..., None]).to(self.conv_state.dtype)
+                self.store_prefill(layer, keys.contiguous(), values.contiguous())
+        self.conv_state.copy_(source.conv_state.index_select(1, order))
+        self.seq_lens.copy_(source.seq_lens.index_select(0, order))
 
     def nbytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in
                    (self.k_cache, self.v_cache, self.conv_state, self.seq_lens, self.k_scales, self.v_scales) if t is not None)
+
+
+def _bytes(tensor: torch.Tensor) -> torch.Tensor:
+    """One-byte element types as uint8, so that gathers and copies move e4m3 codes as they are."""
+    return tensor.view(torch.uint8) if tensor.element_size() == 1 else tensor

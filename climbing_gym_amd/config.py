@@ -10,6 +10,7 @@ import json
 from dataclasses import dataclass, fields
 from pathlib import Path
 from typing import Any, Mapping
+from ._checks import reject
 
 DEFAULT_LAYER_TYPES = tuple("full_attention" if i in (2, 5, 8, 10, 12, 14) else "conv" for i in range(16))
 
@@ -38,16 +39,13 @@ class LFM2Config:
         return self.hidden_size // self.num_attention_heads
 
     def validate(self) -> None:
-        if len(self.layer_types) != self.num_hidden_layers:
-            raise ValueError("len(layer_types) must match num_hidden_layers")
-        if self.hidden_size % self.num_attention_heads:
-            raise ValueError("hidden_size must be divisible by num_attention_heads")
-        if self.num_attention_heads % self.num_key_value_heads:
-            raise ValueError("num_attention_heads must be divisible by num_key_value_heads")
-        if self.mlp_hidden_size <= 0 or self.conv_kernel_size <= 0:
-            raise ValueError("mlp_hidden_size and conv_kernel_size must be > 0")
-        if any(kind not in ("conv", "full_attention") for kind in self.layer_types):
-            raise ValueError("layer_types entries must be either 'conv' or 'full_attention'")
+        reject(len(self.layer_types) != self.num_hidden_layers, "len(layer_types) must match num_hidden_layers")
+        reject(self.hidden_size % self.num_attention_heads, "hidden_size must be divisible by num_attention_heads")
+        reject(self.num_attention_heads % self.num_key_value_heads,
+               "num_attention_heads must be divisible by num_key_value_heads")
+        reject(self.mlp_hidden_size <= 0 or self.conv_kernel_size <= 0, "mlp_hidden_size and conv_kernel_size must be > 0")
+        reject(any(kind not in ("conv", "full_attention") for kind in self.layer_types),
+               "layer_types entries must be either 'conv' or 'full_attention'")
 
     @classmethod
     def from_dict(cls, payload: Mapping[str, Any]) -> "LFM2Config":
@@ -55,13 +53,10 @@ class LFM2Config:
         data = dict(payload)
         rope = data.get("rope_parameters") or data.get("rope_scaling")
         if rope is not None:
-            if not isinstance(rope, Mapping):
-                raise ValueError("LFM2 rope_parameters must be an object")
-            if any(isinstance(v, Mapping) for v in rope.values()):
-                raise ValueError("Unsupported LFM2 per-layer rope_parameters")
+            reject(not isinstance(rope, Mapping), "LFM2 rope_parameters must be an object")
+            reject(any(isinstance(v, Mapping) for v in rope.values()), "Unsupported LFM2 per-layer rope_parameters")
             kind = rope.get("rope_type", rope.get("type", "default"))
-            if kind != "default":
-                raise ValueError(f"Unsupported LFM2 rope_type: {kind!r}; expected 'default'")
+            reject(kind != "default", f"Unsupported LFM2 rope_type: {kind!r}; expected 'default'")
             if rope.get("rope_theta") is not None:
                 data["rope_theta"] = float(rope["rope_theta"])
         if data.get("tie_embedding") is None and data.get("tie_word_embeddings") is not None:
@@ -101,8 +96,7 @@ def _mlp_width(payload: Mapping[str, Any]) -> int:
     if not bool(payload.get("block_auto_adjust_ff_dim", True)):
         return size
     multiple = int(payload.get("block_multiple_of", 256))
-    if multiple <= 0:
-        raise ValueError("block_multiple_of must be > 0")
+    reject(multiple <= 0, "block_multiple_of must be > 0")
     adjusted = int(float(payload.get("block_ffn_dim_multiplier", 1.0)) * int(2 * size / 3))
     return multiple * ((adjusted + multiple - 1) // multiple)
 
@@ -110,14 +104,11 @@ def _mlp_width(payload: Mapping[str, Any]) -> int:
 def coerce_config(config: Any) -> LFM2Config:
     if isinstance(config, LFM2Config):
         return config
-    if config is None:
-        raise TypeError("LFM25 weight synchronization requires a model with an LFM2 config")
+    reject(config is None, "LFM25 weight synchronization requires a model with an LFM2 config", TypeError)
     to_dict = getattr(config, "to_dict", None)
-    if not callable(to_dict):
-        raise TypeError("LFM25 weight synchronization requires an LFM2 config exposing to_dict()")
+    reject(not callable(to_dict), "LFM25 weight synchronization requires an LFM2 config exposing to_dict()", TypeError)
     payload = to_dict()
-    if not isinstance(payload, Mapping):
-        raise TypeError("LFM2 config.to_dict() must return a mapping")
+    reject(not isinstance(payload, Mapping), "LFM2 config.to_dict() must return a mapping", TypeError)
     return LFM2Config.from_dict(dict(payload))
 
 
@@ -137,23 +128,18 @@ class LFM25SamplingConfig:
     behavior_topk: int = 0
 
     def __post_init__(self) -> None:
-        if self.temperature < 0:
-            raise ValueError("temperature must be >= 0")
-        if self.top_k < 0:
-            raise ValueError("top_k must be 0 or positive")
+        reject(self.temperature < 0, "temperature must be >= 0")
+        reject(self.top_k < 0, "top_k must be 0 or positive")
         if not 0.0 < self.top_p <= 1.0:
             raise ValueError("top_p must be in (0, 1]")
-        if self.repetition_penalty <= 0.0:
-            raise ValueError("repetition_penalty must be > 0")
-        if self.max_new_tokens <= 0:
-            raise ValueError("max_new_tokens must be > 0")
-        if type(self.behavior_topk) is not int or not 0 <= self.behavior_topk <= 128:
-            raise ValueError("behavior_topk must be an integer between 0 and 128")
+        reject(self.repetition_penalty <= 0.0, "repetition_penalty must be > 0")
+        reject(self.max_new_tokens <= 0, "max_new_tokens must be > 0")
+        reject(type(self.behavior_topk) is not int or not 0 <= self.behavior_topk <= 128,
+               "behavior_topk must be an integer between 0 and 128")
         if self.behavior_topk and (not self.return_logprobs or self.temperature != 1.0 or self.top_k
                                    or self.top_p != 1.0 or self.repetition_penalty != 1.0):
             raise ValueError("behavior_topk requires actual full-support temperature-1 logprobs")
-        if any(not sequence for sequence in self.stop_token_sequences):
-            raise ValueError("Stop token sequences must be nonempty")
+        reject(any(not sequence for sequence in self.stop_token_sequences), "Stop token sequences must be nonempty")
 
     @property
     def filtered(self) -> bool:

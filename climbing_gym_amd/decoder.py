@@ -18,6 +18,7 @@ from . import ops
 from .cache import LFM25HybridCache
 from .config import LFM25SamplingConfig
 from .engine import LFM25GenerationOutput
+from ._checks import reject
 
 
 class _EagerStep:
@@ -67,12 +68,10 @@ class LFM25HIPDecoder:
                  skip_finished_attention: bool = True, fp8_mlp: bool = False, fp8_kv: bool = False,
                  adaptive_batching: bool = False, fp8_lm_head: bool = False, fp8_operators: bool = False,
                  capture: bool = True):
-        if max_graphs <= 0:
-            raise ValueError("max_graphs must be > 0")
-        if max_prefill_tokens <= 0:
-            raise ValueError("max_prefill_tokens must be positive")
-        if type(finish_check_interval) is not int or finish_check_interval <= 0:
-            raise ValueError("finish_check_interval must be a positive integer")
+        reject(max_graphs <= 0, "max_graphs must be > 0")
+        reject(max_prefill_tokens <= 0, "max_prefill_tokens must be positive")
+        reject(type(finish_check_interval) is not int or finish_check_interval <= 0,
+               "finish_check_interval must be a positive integer")
         self.engine = engine
         self.max_graphs = max_graphs
         self.max_prefill_tokens = max_prefill_tokens
@@ -222,21 +221,19 @@ class LFM25HIPDecoder:
     # ------------------------------------------------------------------ generate
     @torch.inference_mode()
     def generate(self, input_ids, cu_seqlens, max_seqlen: int, repeats: int, sampling: LFM25SamplingConfig):
-        if self._active_session is not None:
-            raise RuntimeError("Close the native generation session before calling generate")
-        if repeats <= 0:
-            raise ValueError("repeats must be > 0")
+        reject(self._active_session is not None,
+               "Close the native generation session before calling generate", RuntimeError)
+        reject(repeats <= 0, "repeats must be > 0")
         engine = self.engine
         device, vocab = engine.device, engine.config.vocab_size
         new_tokens = sampling.max_new_tokens
         cache_len = int(max_seqlen) + new_tokens
-        if cache_len > engine.max_model_len:
-            raise ValueError(f"max_seq_len={cache_len} exceeds engine max_model_len={engine.max_model_len}")
+        reject(cache_len > engine.max_model_len,
+               f"max_seq_len={cache_len} exceeds engine max_model_len={engine.max_model_len}")
         prompts = cu_seqlens.numel() - 1
         batch = prompts * repeats
         k = sampling.behavior_topk
-        if k > vocab:
-            raise ValueError('Behavior head exceeds the vocabulary')
+        reject(k > vocab, 'Behavior head exceeds the vocabulary')
         entry = self._get_graph(batch, cache_len, masked=self.adaptive_batching) if new_tokens > 1 else None
         direct = entry is not None and repeats == 1
         prefix = engine.prefill(input_ids, cu_seqlens, max_seqlen, max_cache_len=max_seqlen,
@@ -313,8 +310,8 @@ class LFM25HIPDecoder:
             return empty, 0
         table = (torch.zeros((1, vocab), dtype=torch.int32, device=device) if sampling.stop_table is None
                  else sampling.stop_table.to(device).clone())
-        if table.ndim != 2 or table.size(1) != vocab or table.dtype != torch.int32:
-            raise ValueError("stop_table must be an int32 state-by-vocabulary table")
+        reject(table.ndim != 2 or table.size(1) != vocab or table.dtype != torch.int32,
+               "stop_table must be an int32 state-by-vocabulary table")
         if sampling.stop_token_ids:
             table[:, list(sampling.stop_token_ids)] = 65536
         return torch.cat((empty, table.reshape(-1))), vocab

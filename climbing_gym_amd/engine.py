@@ -23,6 +23,7 @@ from . import ops
 from .cache import LFM25HybridCache
 from .config import LFM2Config, LFM25SamplingConfig
 from .weights import LFM25PackedWeights
+from ._checks import reject
 
 MAX_PACKED_TOKENS = 32768  # grid limit of the packed prefill kernels per launch
 
@@ -106,11 +107,9 @@ def plan_packed_chunks(lengths: Sequence[int], budget: int):
 
 def flatten_token_batches(input_ids: Sequence[Sequence[int]], *, device=None):
     """Python prompts -> (flat ids int64, cu_seqlens int32, longest) (lfm25_engine.py:1799-1811)."""
-    if not input_ids:
-        raise ValueError("input_ids must contain at least one prompt")
+    reject(not input_ids, "input_ids must contain at least one prompt")
     lengths = [len(p) for p in input_ids]
-    if any(n <= 0 for n in lengths):
-        raise ValueError("empty prompts are not supported")
+    reject(any(n <= 0 for n in lengths), "empty prompts are not supported")
     device = torch.device(device or "cpu")
     # one pass in C over the concatenated prompts (a Python list comprehension over a few hundred thousand ids is a
     # visible share of an admission)
@@ -123,22 +122,17 @@ def flatten_token_batches(input_ids: Sequence[Sequence[int]], *, device=None):
 
 class LFM25Engine:
     def __init__(self, weights: LFM25PackedWeights, *, max_model_len: int | None = None) -> None:
-        if weights.device.type != "cuda":
-            raise ValueError("this engine runs on the GPU only; weights must live on a HIP device")
-        if weights.dtype != torch.bfloat16:
-            raise ValueError("this engine computes in bfloat16")
+        reject(weights.device.type != "cuda", "this engine runs on the GPU only; weights must live on a HIP device")
+        reject(weights.dtype != torch.bfloat16, "this engine computes in bfloat16")
         cfg = weights.config
-        if cfg.conv_kernel_size != 3 or cfg.conv_bias:
-            raise ValueError("the short-conv kernels need bias-free convolutions of width 3")
-        if cfg.head_dim not in (32, 64, 128):
-            raise ValueError("head_dim must be one of {32, 64, 128}")
+        reject(cfg.conv_kernel_size != 3 or cfg.conv_bias, "the short-conv kernels need bias-free convolutions of width 3")
+        reject(cfg.head_dim not in (32, 64, 128), "head_dim must be one of {32, 64, 128}")
         self.weights, self.config = weights, cfg
         self.device, self.dtype = weights.device, weights.dtype
         self.max_model_len = int(max_model_len or min(int(cfg.max_position_embeddings), 32768))
-        if self.max_model_len <= 0:
-            raise ValueError("max_model_len must be > 0")
-        if self.max_model_len > int(cfg.max_position_embeddings):
-            raise ValueError("max_model_len cannot exceed config.max_position_embeddings")
+        reject(self.max_model_len <= 0, "max_model_len must be > 0")
+        reject(self.max_model_len > int(cfg.max_position_embeddings),
+               "max_model_len cannot exceed config.max_position_embeddings")
         self._scaling = cfg.head_dim ** -0.5
         self._cuda_decoder = None
         self.policy_version = 0
@@ -174,10 +168,8 @@ class LFM25Engine:
     def sync_from_model(self, model: Any, *, drain_timeout: int | float = 300) -> "LFM25Engine":
         """In-place policy sync; captured graphs keep working and see the new weights (lfm25_engine.py:556-578)."""
         timeout = float(drain_timeout)
-        if not math.isfinite(timeout) or timeout < 0.0:
-            raise ValueError("drain_timeout must be finite and >= 0")
-        if self._decoder_busy:
-            raise RuntimeError("Close the native generation session before synchronizing weights")
+        reject(not math.isfinite(timeout) or timeout < 0.0, "drain_timeout must be finite and >= 0")
+        reject(self._decoder_busy, "Close the native generation session before synchronizing weights", RuntimeError)
         self.weights.copy_from_model_(model)
         if self._cuda_decoder is not None:
             self._cuda_decoder.refresh_weights()
@@ -190,8 +182,7 @@ class LFM25Engine:
         """Same switch as the reference (lfm25_engine.py:980-997); graphs are HIP graphs.  `fp8_operators` extends
         W8A8 to the QKV/out and conv in/out projections; `bf16_weight_packing` is accepted and ignored."""
         from .decoder import LFM25HIPDecoder
-        if self._decoder_busy:
-            raise RuntimeError("Close the native generation session before reconfiguring CUDA graphs")
+        reject(self._decoder_busy, "Close the native generation session before reconfiguring CUDA graphs", RuntimeError)
         if self._cuda_decoder is not None:
             self._cuda_decoder.clear()
         self._cuda_decoder = LFM25HIPDecoder(self, max_graphs=max_graphs, max_prefill_tokens=max_prefill_tokens,
@@ -216,8 +207,8 @@ class LFM25Engine:
         decoder = self._cuda_decoder
         if decoder is None:
             return
-        if decoder._active_session is not None:
-            raise RuntimeError("Close the native generation session before releasing inference buffers")
+        reject(decoder._active_session is not None,
+               "Close the native generation session before releasing inference buffers", RuntimeError)
         if not (decoder.graphs or decoder.fp8_weights):
             return
         torch.cuda.synchronize(self.device)
@@ -226,20 +217,17 @@ class LFM25Engine:
 
     def generation_session(self, *, max_batch_size: int, max_new_tokens: int, cache_len: int | None = None,
                            behavior_topk: int = 0, profile_timings: bool = False):
-        if self._cuda_decoder is None:
-            raise RuntimeError("generation_session requires enable_cuda_graphs()")
+        reject(self._cuda_decoder is None, "generation_session requires enable_cuda_graphs()", RuntimeError)
         from .session import LFM25GenerationSession
         return LFM25GenerationSession(self._cuda_decoder, max_batch_size=max_batch_size, max_new_tokens=max_new_tokens,
                                       cache_len=cache_len, behavior_topk=behavior_topk, profile_timings=profile_timings)
 
     # ------------------------------------------------------------------ cache
     def _empty_cache(self, *, max_slots: int, max_seq_len: int, fp8_kv: bool = False) -> LFM25HybridCache:
-        if max_slots <= 0:
-            raise ValueError("max_slots must be > 0")
-        if max_seq_len <= 0:
-            raise ValueError("max_seq_len must be > 0")
-        if max_seq_len > self.max_model_len:
-            raise ValueError(f"max_seq_len={max_seq_len} exceeds engine max_model_len={self.max_model_len}")
+        reject(max_slots <= 0, "max_slots must be > 0")
+        reject(max_seq_len <= 0, "max_seq_len must be > 0")
+        reject(max_seq_len > self.max_model_len,
+               f"max_seq_len={max_seq_len} exceeds engine max_model_len={self.max_model_len}")
         cfg = self.config
         return LFM25HybridCache.allocate(
             attn_layers=self.weights.num_attention_layers, conv_layers=self.weights.num_conv_layers, slots=max_slots,
@@ -411,10 +399,8 @@ class LFM25Engine:
         for the stream and stops the host from running ahead of the GPU."""
         cfg = self.config
         count, total, longest = len(lengths), int(sum(lengths)), int(max(lengths))
-        if longest > cache.max_seq_len:
-            raise RuntimeError("cache capacity exceeded")
-        if longest > self.max_model_len:
-            raise RuntimeError("position exceeds engine max_model_len")
+        reject(longest > cache.max_seq_len, "cache capacity exceeded", RuntimeError)
+        reject(longest > self.max_model_len, "position exceeds engine max_model_len", RuntimeError)
         cu = torch.zeros(count + 1, device=self.device, dtype=torch.int32)
         cu[1:] = lengths_device.cumsum(0)
         seq_of_token, positions = ops.build_token_map(cu, total)
@@ -448,25 +434,18 @@ class LFM25Engine:
         logits to the same rows of `logits_buffer` ([cache slots, vocab]); the other slots are not touched."""
         input_ids = input_ids.to(device=self.device, dtype=torch.long).reshape(-1)
         bounds = cu_seqlens.to(device="cpu", dtype=torch.long).reshape(-1)
-        if bounds.numel() < 2:
-            raise ValueError("cu_seqlens must contain at least [0, total_tokens]")
-        if int(bounds[0]) != 0:
-            raise ValueError("cu_seqlens must start at 0")
-        if int(bounds[-1]) != int(input_ids.numel()):
-            raise ValueError("cu_seqlens[-1] must equal input_ids.numel()")
+        reject(bounds.numel() < 2, "cu_seqlens must contain at least [0, total_tokens]")
+        reject(int(bounds[0]) != 0, "cu_seqlens must start at 0")
+        reject(int(bounds[-1]) != int(input_ids.numel()), "cu_seqlens[-1] must equal input_ids.numel()")
         offsets = bounds.tolist()
         lengths = [b - a for a, b in zip(offsets[:-1], offsets[1:])]
-        if min(lengths) <= 0:
-            raise ValueError("empty prompts are not supported")
-        if max(lengths) > int(max_seqlen):
-            raise ValueError("max_seqlen is smaller than at least one prompt")
-        if max_prefill_tokens is not None and max_prefill_tokens <= 0:
-            raise ValueError("max_prefill_tokens must be positive")
+        reject(min(lengths) <= 0, "empty prompts are not supported")
+        reject(max(lengths) > int(max_seqlen), "max_seqlen is smaller than at least one prompt")
+        reject(max_prefill_tokens is not None and max_prefill_tokens <= 0, "max_prefill_tokens must be positive")
         count = len(lengths)
         cache_len = int(max_cache_len or max_seqlen)
         if cache is None:
-            if slots is not None:
-                raise ValueError("slots address an existing cache")
+            reject(slots is not None, "slots address an existing cache")
             cache = self._empty_cache(max_slots=count, max_seq_len=cache_len)
         elif cache.max_seq_len < cache_len or (slots is None and cache.max_slots != count):
             raise ValueError("destination cache does not fit the prompt batch")
@@ -474,14 +453,14 @@ class LFM25Engine:
             slot_list = list(range(count))
         else:
             slot_list = [int(slot) for slot in slots]
-            if len(slot_list) != count or len(set(slot_list)) != count or min(slot_list) < 0 or max(slot_list) >= cache.max_slots:
-                raise ValueError("slots must be distinct cache slots, one per prompt")
+            reject(len(slot_list) != count or len(set(slot_list)) != count or min(slot_list) < 0 or max(slot_list) >= cache.max_slots,
+                   "slots must be distinct cache slots, one per prompt")
         shape = (cache.max_slots, self.config.vocab_size)
         if logits_buffer is None:
             logits_out = torch.empty(shape, device=self.device, dtype=self.dtype)
         else:
-            if logits_buffer.shape != shape or logits_buffer.dtype != self.dtype or logits_buffer.device != self.weights.embed_tokens.device:
-                raise ValueError("logits buffer must match the prompt batch, vocabulary, device, and model dtype")
+            reject(logits_buffer.shape != shape or logits_buffer.dtype != self.dtype or logits_buffer.device != self.weights.embed_tokens.device,
+                   "logits buffer must match the prompt batch, vocabulary, device, and model dtype")
             logits_out = logits_buffer
         budget = MAX_PACKED_TOKENS if max_prefill_tokens is None else min(int(max_prefill_tokens), MAX_PACKED_TOKENS)
         fp8 = self._fp8()
@@ -505,13 +484,11 @@ class LFM25Engine:
     # ------------------------------------------------------------------ fork / decode_step
     @torch.inference_mode()
     def fork(self, prefix: LFM25PrefixBatch, repeats: int, *, max_cache_len: int | None = None) -> LFM25DecodeBatch:
-        if repeats <= 0:
-            raise ValueError("repeats must be > 0")
+        reject(repeats <= 0, "repeats must be > 0")
         prompts = prefix.batch_size
         total = prompts * int(repeats)
         cache_len = int(max_cache_len or prefix.cache.max_seq_len)
-        if cache_len < prefix.cache.max_seq_len:
-            raise ValueError("max_cache_len cannot be smaller than the prefix cache")
+        reject(cache_len < prefix.cache.max_seq_len, "max_cache_len cannot be smaller than the prefix cache")
         cache = self._empty_cache(max_slots=total, max_seq_len=cache_len)
         arange = lambda n: torch.arange(n, device=self.device, dtype=torch.long)
         cache.copy_prefix_from(prefix.cache, arange(prompts).repeat_interleave(repeats), prefix.cache.max_seq_len)
@@ -524,15 +501,12 @@ class LFM25Engine:
         (lfm25_engine.py:1232-1243)."""
         slot_ids = slot_ids.to(device=self.device, dtype=torch.long).reshape(-1)
         input_tokens = input_tokens.to(device=self.device, dtype=torch.long).reshape(-1)
-        if slot_ids.numel() != input_tokens.numel():
-            raise ValueError("slot_ids and input_tokens must have matching lengths")
-        if torch.any(slot_ids < 0) or torch.any(slot_ids >= cache.max_slots):
-            raise ValueError("slot_ids contain an out-of-range cache slot")
+        reject(slot_ids.numel() != input_tokens.numel(), "slot_ids and input_tokens must have matching lengths")
+        reject(torch.any(slot_ids < 0) or torch.any(slot_ids >= cache.max_slots),
+               "slot_ids contain an out-of-range cache slot")
         positions = cache.seq_lens.index_select(0, slot_ids)
-        if torch.any(positions >= cache.max_seq_len):
-            raise RuntimeError("cache capacity exceeded")
-        if torch.any(positions >= self.max_model_len):
-            raise RuntimeError("position exceeds engine max_model_len")
+        reject(torch.any(positions >= cache.max_seq_len), "cache capacity exceeded", RuntimeError)
+        reject(torch.any(positions >= self.max_model_len), "position exceeds engine max_model_len", RuntimeError)
         active = torch.ones(slot_ids.numel(), device=self.device, dtype=torch.bool)
         return self._decode_forward(cache, input_tokens, active, slot_ids=slot_ids.to(torch.int32), positions=positions.contiguous())
 
@@ -540,8 +514,7 @@ class LFM25Engine:
     def decode_step(self, state: LFM25DecodeBatch, input_tokens, sampling: LFM25SamplingConfig | None = None) -> LFM25StepOutput:
         sampling = sampling or LFM25SamplingConfig()
         input_tokens = input_tokens.to(device=self.device, dtype=torch.long).reshape(-1)
-        if input_tokens.numel() != state.active_slot_ids.numel():
-            raise ValueError("input_tokens must have one token per active slot")
+        reject(input_tokens.numel() != state.active_slot_ids.numel(), "input_tokens must have one token per active slot")
         logits = self._append_decode_tokens(state.cache, state.active_slot_ids, input_tokens)
         tokens, raw = self._sample(logits, sampling, step=0)
         reasons = self._finish_reasons(tokens, sampling)
@@ -591,15 +564,12 @@ class LFM25Engine:
     @torch.inference_mode()
     def score_completions(self, prompts, completions, *, max_prefill_tokens: int = 4096, head_chunk_size: int = 256):
         """Raw log-probabilities of given completions through the packed prefill kernels (lfm25_engine.py:1108-1163)."""
-        if len(prompts) != len(completions):
-            raise ValueError('prompts and completions must have equal lengths')
-        if max_prefill_tokens <= 0 or head_chunk_size <= 0:
-            raise ValueError('scoring chunk sizes must be positive')
-        if any(not p or not c for p, c in zip(prompts, completions)):
-            raise ValueError('scoring requires nonempty prompts and completions')
+        reject(len(prompts) != len(completions), 'prompts and completions must have equal lengths')
+        reject(max_prefill_tokens <= 0 or head_chunk_size <= 0, 'scoring chunk sizes must be positive')
+        reject(any(not p or not c for p, c in zip(prompts, completions)),
+               'scoring requires nonempty prompts and completions')
         sequences = [list(p) + list(c) for p, c in zip(prompts, completions)]
-        if any(len(s) > self.max_model_len for s in sequences):
-            raise ValueError('scored sequence exceeds max_model_len')
+        reject(any(len(s) > self.max_model_len for s in sequences), 'scored sequence exceeds max_model_len')
         cfg, fp8 = self.config, self._fp8()
         result = [()] * len(sequences)
         order = sorted(range(len(sequences)), key=lambda i: len(sequences[i]))

@@ -8,6 +8,7 @@ from dataclasses import dataclass, field
 from numbers import Real
 from pathlib import Path
 from typing import Any
+from ._checks import reject
 
 DEFAULT_STAGED_CHECKPOINT_ROOT = Path.home() / ".cache" / "climbing-gym" / "checkpoints"
 _EXTRA_KEYS = {"repetition_penalty", "ignore_eos", "behavior_topk"}
@@ -43,20 +44,15 @@ class SamplingConfig:
             (isinstance(self.extra_params, Mapping), "extra_params must be a mapping"),
         )
         for ok, message in checks:
-            if not ok:
-                raise ValueError(message)
+            reject(not ok, message)
         object.__setattr__(self, "stop", tuple(self.stop))
         unknown = sorted(str(k) for k in set(self.extra_params) - _EXTRA_KEYS)
-        if unknown:
-            raise ValueError(f"Unsupported native sampling extra_params: {unknown}")
+        reject(unknown, f"Unsupported native sampling extra_params: {unknown}")
         penalty = self.extra_params.get("repetition_penalty", 1.0)
-        if not _is_number(penalty) or penalty <= 0:
-            raise ValueError("repetition_penalty must be finite and > 0")
-        if type(self.extra_params.get("ignore_eos", False)) is not bool:
-            raise ValueError("ignore_eos must be a boolean")
+        reject(not _is_number(penalty) or penalty <= 0, "repetition_penalty must be finite and > 0")
+        reject(type(self.extra_params.get("ignore_eos", False)) is not bool, "ignore_eos must be a boolean")
         head = self.extra_params.get("behavior_topk", 0)
-        if type(head) is not int or not 0 <= head <= 128:
-            raise ValueError("behavior_topk must be an integer between 0 and 128")
+        reject(type(head) is not int or not 0 <= head <= 128, "behavior_topk must be an integer between 0 and 128")
 
     def batching_key(self) -> tuple:
         """Requests with equal keys may share one engine.generate call (lfm25_async_engine.py:675-685)."""
@@ -82,9 +78,6 @@ class InferenceEngineConfig:
     staged_checkpoint_root: Path = field(default_factory=lambda: DEFAULT_STAGED_CHECKPOINT_ROOT)
 
     def __post_init__(self) -> None:
-        if not 0.0 < self.gpu_memory_utilization <= 1.0:
-            raise ValueError("gpu_memory_utilization must be between 0 and 1")
-        if self.max_model_len is not None and self.max_model_len <= 0:
-            raise ValueError("max_model_len must be > 0 when provided")
-        if self.max_num_seqs is not None and self.max_num_seqs <= 0:
-            raise ValueError("max_num_seqs must be > 0 when provided")
+        reject(not 0.0 < self.gpu_memory_utilization <= 1.0, "gpu_memory_utilization must be between 0 and 1")
+        reject(self.max_model_len is not None and self.max_model_len <= 0, "max_model_len must be > 0 when provided")
+        reject(self.max_num_seqs is not None and self.max_num_seqs <= 0, "max_num_seqs must be > 0 when provided")

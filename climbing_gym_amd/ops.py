@@ -15,6 +15,7 @@ import torch
 
 from . import _lib
 from ._lib import DTYPE_CODE, call, query
+from ._checks import reject
 
 FP8 = torch.float8_e4m3fn
 
@@ -34,10 +35,8 @@ def _check(*tensors):
     for t in tensors:
         if t is None:
             continue
-        if not t.is_cuda:
-            raise ValueError("HIP kernels require GPU tensors")
-        if not t.is_contiguous():
-            raise ValueError("HIP kernels require contiguous tensors")
+        reject(not t.is_cuda, "HIP kernels require GPU tensors")
+        reject(not t.is_contiguous(), "HIP kernels require contiguous tensors")
 
 
 # ----------------------------------------------------------------------------------- embedding / norms
@@ -74,8 +73,7 @@ def rms_norm(x, weight: torch.Tensor, eps: float, residual: torch.Tensor | None 
     `x` may be a `SplitProduct` (then a residual is required and the projection's reduce pass runs inside the norm)."""
     if isinstance(x, SplitProduct):
         _check(weight, residual)
-        if residual is None:
-            raise ValueError("a deferred projection can only feed a norm that adds a residual")
+        reject(residual is None, "a deferred projection can only feed a norm that adds a residual")
         rows, width = x.shape
         out = torch.empty((rows, width), device=weight.device, dtype=x.dtype)
         summed = torch.empty_like(out)
@@ -121,8 +119,7 @@ def rms_norm_fp8(x, weight, eps, residual=None):
         rows, width = x.shape
         q = torch.empty((rows, width), device=weight.device, dtype=FP8)
         scales = torch.empty(rows, device=weight.device, dtype=torch.float32)
-        if residual is None:
-            raise ValueError("a deferred projection can only feed a norm that adds a residual")
+        reject(residual is None, "a deferred projection can only feed a norm that adds a residual")
         summed = torch.empty((rows, width), device=weight.device, dtype=x.dtype)
         call("lfm2_rms_norm_fp8_split", q, scales, summed, x.partials, x.partials.size(0), x.a_scales, x.w_scales, weight,
              residual, rows, width, float(eps), _code(x.dtype))
@@ -157,10 +154,9 @@ def swiglu_fp8(x: torch.Tensor):
 
 def quantize_rows(x: torch.Tensor, *, out: tuple[torch.Tensor, torch.Tensor] | None = None):
     """lfm25_fp8.py:108-117, including its argument errors."""
-    if x.ndim != 2 or not x.is_cuda or not x.is_contiguous() or x.dtype not in (torch.bfloat16, torch.float16):
-        raise ValueError("FP8 quantization requires a contiguous 2D CUDA BF16/FP16 tensor")
-    if min(x.shape) <= 0 or x.size(1) > 32768:
-        raise ValueError("FP8 row width must be in [1, 32768]")
+    reject(x.ndim != 2 or not x.is_cuda or not x.is_contiguous() or x.dtype not in (torch.bfloat16, torch.float16),
+           "FP8 quantization requires a contiguous 2D CUDA BF16/FP16 tensor")
+    reject(min(x.shape) <= 0 or x.size(1) > 32768, "FP8 row width must be in [1, 32768]")
     if out is None:
         out = (torch.empty(x.shape, device=x.device, dtype=FP8),
                torch.empty(x.size(0), device=x.device, dtype=torch.float32))
@@ -196,8 +192,7 @@ def prepare_qkv_store(x, q_weight, k_weight, cos, sin, positions, q_heads: int, 
     lfm25_fp8_kv.py:58-69 when scale tensors are given, `append_bf16_kv` of lfm25_batching.py:66-69 otherwise):
     returns q [M,1,QH,D]; keys and values go straight into the cache views at `positions`."""
     _check(x, q_weight, k_weight, cos, sin, positions, active, slot_ids)
-    if positions.dtype != torch.int32:
-        raise ValueError("positions must be int32")
+    reject(positions.dtype != torch.int32, "positions must be int32")
     m = x.size(0)
     q = torch.empty((m, 1, q_heads, head_dim), device=x.device, dtype=x.dtype)
     c0, c1, c2 = _cache_strides(k_cache)
@@ -220,11 +215,10 @@ def qkv_project_store(xq, x_scales, packed, q_weight, k_weight, cos, sin, positi
     its epilogue: quantised rows in, q [M,1,QH,D] out, keys and values appended to the cache.  Same bytes as the two
     calls."""
     _check(xq, x_scales, q_weight, k_weight, cos, sin, positions, active, slot_ids)
-    if positions.dtype != torch.int32:
-        raise ValueError("positions must be int32")
+    reject(positions.dtype != torch.int32, "positions must be int32")
     m, width = xq.shape
-    if packed.values.shape != ((q_heads + 2 * kv_heads) * head_dim, width):
-        raise ValueError("QKV weight does not match the activation width and head counts")
+    reject(packed.values.shape != ((q_heads + 2 * kv_heads) * head_dim, width),
+           "QKV weight does not match the activation width and head counts")
     q = torch.empty((m, 1, q_heads, head_dim), device=xq.device, dtype=q_weight.dtype)
     c0, c1, c2 = _cache_strides(k_cache)
     call("lfm2_fp8_gemm_qkv_store", q, xq, x_scales, packed.values, packed.scales, q_weight, k_weight, cos, sin, positions,
@@ -236,8 +230,7 @@ def qkv_project_store(xq, x_scales, packed, q_weight, k_weight, cos, sin, positi
 def prepare_qkv(x, q_weight, k_weight, cos, sin, positions, q_heads: int, kv_heads: int, head_dim: int, eps: float):
     """lfm25_cuda_kernels.py:143-151: QK RMSNorm + rotate-half RoPE + split; q/k/v come back as [M,1,heads,D]."""
     _check(x, q_weight, k_weight, cos, sin, positions)
-    if positions.dtype != torch.int32:
-        raise ValueError("positions must be int32")
+    reject(positions.dtype != torch.int32, "positions must be int32")
     m = x.size(0)
     q = torch.empty((m, 1, q_heads, head_dim), device=x.device, dtype=x.dtype)
     k = torch.empty((m, 1, kv_heads, head_dim), device=x.device, dtype=x.dtype)
@@ -270,14 +263,13 @@ class RowPlacement:
 
     def check(self, rows: int, columns: int, dtype) -> None:
         out = self.out
-        if out.ndim != 2 or out.size(1) != columns or out.dtype != dtype or not out.is_contiguous():
-            raise ValueError("placed rows need a contiguous [slots, columns] destination of the product's dtype")
-        if self.slots is None and rows > out.size(0):
-            raise ValueError("more product rows than destination rows")
-        if self.slots is not None and (self.slots.dtype != torch.int32 or self.slots.numel() != rows):
-            raise ValueError("slots must be int32, one per product row")
-        if self.active is not None and (self.active.dtype not in (torch.bool, torch.uint8) or self.active.numel() != rows):
-            raise ValueError("active must be a bool mask, one per product row")
+        reject(out.ndim != 2 or out.size(1) != columns or out.dtype != dtype or not out.is_contiguous(),
+               "placed rows need a contiguous [slots, columns] destination of the product's dtype")
+        reject(self.slots is None and rows > out.size(0), "more product rows than destination rows")
+        reject(self.slots is not None and (self.slots.dtype != torch.int32 or self.slots.numel() != rows),
+               "slots must be int32, one per product row")
+        reject(self.active is not None and (self.active.dtype not in (torch.bool, torch.uint8) or self.active.numel() != rows),
+               "active must be a bool mask, one per product row")
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, *, tile: int = -1, split_k: int = 0,
@@ -285,13 +277,12 @@ def linear(x: torch.Tensor, weight: torch.Tensor, *, tile: int = -1, split_k: in
     """lfm25_cuda_kernels.py:19-29: y = x W^T on the bf16 MFMA kernel of this package; any other dtype is refused
     (there is no vendor-library path).  With `place`, rows land in `place.out`.  With `defer_reduce`, a product the
     plan splits along K comes back as a `SplitProduct` for `rms_norm` to reduce."""
-    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
-        raise ValueError("linear runs in bfloat16 only: this package has no GEMM for other dtypes")
+    reject(x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16,
+           "linear runs in bfloat16 only: this package has no GEMM for other dtypes")
     _check(x, weight)
     m, k = _rows(x), x.size(-1)
     n = weight.size(0)
-    if weight.size(1) != k:
-        raise ValueError("activation and weight widths differ")
+    reject(weight.size(1) != k, "activation and weight widths differ")
     if place is not None:
         place.check(m, n, x.dtype)
         call("lfm2_bf16_gemm_rows", place.out, x, weight, place.slots, place.active, place.out.size(0), m, n, k, tile)
@@ -312,12 +303,12 @@ def linear(x: torch.Tensor, weight: torch.Tensor, *, tile: int = -1, split_k: in
 def linear_swiglu(x: torch.Tensor, weight: torch.Tensor):
     """`swiglu(linear(x, weight))` for the packed gate+up weight [2I, K] (lfm25_cuda_kernels.py:19-29 then :58-72),
     the same bits, in one launch where the product's shape has the fused form and in the two launches otherwise."""
-    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
-        raise ValueError("linear runs in bfloat16 only: this package has no GEMM for other dtypes")
+    reject(x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16,
+           "linear runs in bfloat16 only: this package has no GEMM for other dtypes")
     _check(x, weight)
     m, k, n = _rows(x), x.size(-1), weight.size(0)
-    if weight.size(1) != k or n % 2:
-        raise ValueError("activation and weight widths differ, or the packed gate+up weight has an odd row count")
+    reject(weight.size(1) != k or n % 2,
+           "activation and weight widths differ, or the packed gate+up weight has an odd row count")
     if x.ndim != 2 or not query("lfm2_gemm_swiglu_fits", m, n, k, 2):
         return swiglu(linear(x, weight))
     out = torch.empty((m, n // 2), device=x.device, dtype=x.dtype)
@@ -351,8 +342,7 @@ class PackedFP8Weight:
         With `place` (a `RowPlacement`) the rows land in `place.out`."""
         batch, width = x.shape
         rows = self.values.size(0)
-        if width != self.values.size(1):
-            raise ValueError("FP8 activation and weight widths differ")
+        reject(width != self.values.size(1), "FP8 activation and weight widths differ")
         tile, split_k = (-1, 0) if config is None else (int(config[0]), int(config[1]) if len(config) > 1 else 0)
         if place is not None:
             place.check(batch, rows, dtype)
@@ -377,8 +367,8 @@ class PackedFP8Weight:
         in the projection's epilogue and only [M, I] is written and quantised, otherwise the two launches run."""
         batch, width = x.shape
         rows = self.values.size(0)
-        if width != self.values.size(1) or rows % 2:
-            raise ValueError("FP8 activation and weight widths differ, or the packed gate+up weight has an odd row count")
+        reject(width != self.values.size(1) or rows % 2,
+               "FP8 activation and weight widths differ, or the packed gate+up weight has an odd row count")
         if not query("lfm2_gemm_swiglu_fits", batch, rows, width, 1):
             return swiglu_fp8(self.linear_quantized(x, scales, dtype=dtype))
         hidden = torch.empty((batch, rows // 2), device=x.device, dtype=dtype)
@@ -388,8 +378,8 @@ class PackedFP8Weight:
 
 # ----------------------------------------------------------------------------------- KV cache + attention
 def _cache_strides(cache: torch.Tensor):
-    if cache.ndim != 4 or cache.stride(3) != 1:
-        raise ValueError("cache views must be [slots, positions, heads, dim] with a contiguous last dimension")
+    reject(cache.ndim != 4 or cache.stride(3) != 1,
+           "cache views must be [slots, positions, heads, dim] with a contiguous last dimension")
     return cache.stride(0), cache.stride(1), cache.stride(2)
 
 
@@ -397,8 +387,7 @@ def store_kv(k, v, k_cache, v_cache, k_scales, v_scales, *, positions=None, acti
     """lfm25_fp8_kv.py:58-69: write [batch, tokens, KV heads, dim] as e4m3 rows with fp32 scales into (possibly
     strided) cache views; append mode when `positions` is given."""
     batch, tokens, heads, dim = k.shape
-    if k.stride(3) != 1 or v.stride(3) != 1:
-        raise ValueError("k and v need a contiguous head dimension")
+    reject(k.stride(3) != 1 or v.stride(3) != 1, "k and v need a contiguous head dimension")
     c0, c1, c2 = _cache_strides(k_cache)
     call("lfm2_store_kv_fp8", k, v, k_cache, v_cache, k_scales, v_scales, positions, active, slot_ids, batch, tokens,
          heads, dim, *k.stride()[:3], *v.stride()[:3], c0, c1, c2, _code(k.dtype))
@@ -454,8 +443,7 @@ def attend(q, k_cache, v_cache, k_scales, v_scales, positions, *, active=None, s
     """lfm25_fp8_kv.py:138-167 (e4m3 history + scales) and flash_attn_with_kvcache of lfm25_cuda.py:156-165
     (`k_scales is None`: history in the model dtype).  Attends over positions [0, positions[b]]; inactive rows
     return zeros.  With `block_table` the caches are page pools [pages, page, KV heads, dim]."""
-    if window:
-        raise ValueError("sliding windows belong to LFM3 and are not part of this path")
+    reject(window, "sliding windows belong to LFM3 and are not part of this path")
     batch, _, query_heads, dim = q.shape
     _check(q, positions)
     heads = k_cache.size(2)
@@ -528,12 +516,11 @@ def sample_logits(logits: torch.Tensor, *, temperature: float, seed: int, step: 
     full support (one uniform number per row through the inverse cumulative distribution: the same law as the
     reference's Gumbel-max); log-probabilities are the raw log-softmax of the chosen token.  Deterministic in
     (seed, step)."""
-    if logits.ndim != 2 or not logits.is_cuda or logits.dtype not in (torch.bfloat16, torch.float16, torch.float32):
-        raise ValueError("sampling requires a 2D CUDA BF16/FP16/FP32 logits tensor")
+    reject(logits.ndim != 2 or not logits.is_cuda or logits.dtype not in (torch.bfloat16, torch.float16, torch.float32),
+           "sampling requires a 2D CUDA BF16/FP16/FP32 logits tensor")
     logits = logits.contiguous()
     batch, vocab = logits.shape
-    if batch == 0 or vocab == 0 or temperature < 0:
-        raise ValueError("sampling requires nonempty logits and nonnegative temperature")
+    reject(batch == 0 or vocab == 0 or temperature < 0, "sampling requires nonempty logits and nonnegative temperature")
     tokens = torch.empty(batch, device=logits.device, dtype=torch.long)
     logprobs = torch.empty(batch, device=logits.device, dtype=torch.float32) if return_logprobs else None
     call("lfm2_sample", tokens, logprobs, logits, _sample_scratch(batch, vocab, logits.device), None, None, None,
@@ -546,8 +533,8 @@ def sample_logits_static(logits: torch.Tensor, tokens: torch.Tensor, logprobs: t
     """`sample_logits` into caller-provided outputs with no device allocation at all: the sampler's tile statistics
     live in a fixed 256 KiB array inside the library (at most 16384 row-tiles of 4096 logits per call; calls that
     overlap on one GPU race on it).  For callers that must not allocate; no counterpart in the reference."""
-    if logits.ndim != 2 or not logits.is_cuda or not logits.is_contiguous():
-        raise ValueError("sampling requires a contiguous 2D GPU logits tensor")
+    reject(logits.ndim != 2 or not logits.is_cuda or not logits.is_contiguous(),
+           "sampling requires a contiguous 2D GPU logits tensor")
     batch, vocab = logits.shape
     call("lfm2_sample_static", tokens, logprobs, logits, None, None, None, int(seed) & 0x7FFFFFFFFFFFFFFF, int(step),
          float(temperature), batch, vocab, _code(logits.dtype))
@@ -586,8 +573,7 @@ def sample_filtered(logits, *, temperature: float = 1.0, top_k: int = 0, top_p: 
     returns (tokens, raw log-probabilities[, survivors per row]).  With per-row `temperatures`, `top_ks` (int32) and
     `top_ps` every row has its own parameters, and rows that ask for no filter or for greedy decoding are left as `out`
     holds them."""
-    if logits.ndim != 2 or not logits.is_cuda:
-        raise ValueError("sampling requires a 2D GPU logits tensor")
+    reject(logits.ndim != 2 or not logits.is_cuda, "sampling requires a 2D GPU logits tensor")
     logits = logits.contiguous()
     batch, vocab = logits.shape
     tokens, logprobs = out if out is not None else (
@@ -602,8 +588,7 @@ def sample_filtered(logits, *, temperature: float = 1.0, top_k: int = 0, top_p: 
 
 def behavior_topk(logits, selected, logprobs, k):
     """lfm25_sampling.py:137-149: top-k ids with log-probabilities that reuse the sampler's normaliser."""
-    if not 0 < k <= min(logits.size(1), 128):
-        raise ValueError('Behavior head exceeds the vocabulary or supported size')
+    reject(not 0 < k <= min(logits.size(1), 128), 'Behavior head exceeds the vocabulary or supported size')
     values, ids = torch.topk(logits, k, dim=-1, sorted=True)
     probs = torch.empty(values.shape, dtype=torch.float32, device=logits.device)
     call("lfm2_head_logprobs", probs, logits, selected, logprobs, values.contiguous(), logits.size(0), logits.size(1),

@@ -23,6 +23,7 @@ from statistics import pstdev
 from typing import Any, Mapping, Optional, Protocol, runtime_checkable
 
 from .types import BehaviorTopK
+from ._checks import reject
 
 log = logging.getLogger(__name__)
 
@@ -36,10 +37,9 @@ class RolloutConfig:
     max_total_requests: Optional[int] = None
 
     def __post_init__(self):
-        if self.num_rollouts <= 0:
-            raise ValueError("num_rollouts must be > 0")
-        if self.max_total_requests is not None and self.max_total_requests <= 0:
-            raise ValueError("max_total_requests must be > 0 when provided")
+        reject(self.num_rollouts <= 0, "num_rollouts must be > 0")
+        reject(self.max_total_requests is not None and self.max_total_requests <= 0,
+               "max_total_requests must be > 0 when provided")
 
 
 @dataclass(frozen=True)
@@ -53,13 +53,11 @@ class RolloutRunnerConfig:
     progress_log_interval_seconds: float = 15.0
 
     def __post_init__(self):
-        if self.effective_batch_size <= 0:
-            raise ValueError("effective_batch_size must be > 0")
-        if self.max_inflight_requests is not None and self.max_inflight_requests <= 0:
-            raise ValueError("max_inflight_requests must be > 0 when provided")
+        reject(self.effective_batch_size <= 0, "effective_batch_size must be > 0")
+        reject(self.max_inflight_requests is not None and self.max_inflight_requests <= 0,
+               "max_inflight_requests must be > 0 when provided")
         for name in ("reward_std_epsilon", "stall_timeout_seconds", "progress_log_interval_seconds"):
-            if getattr(self, name) < 0:
-                raise ValueError(f"{name} must be >= 0")
+            reject(getattr(self, name) < 0, f"{name} must be >= 0")
 
 
 # ------------------------------------------------------------------------------------------------ records
@@ -163,8 +161,7 @@ def require_single_output(sampling) -> None:
         count = None if count is None else int(count)
     except (TypeError, ValueError):
         count = None
-    if count not in (None, 1):
-        raise ValueError("RolloutRunner requires sampling.n == 1 for each engine request.")
+    reject(count not in (None, 1), "RolloutRunner requires sampling.n == 1 for each engine request.")
 
 
 @dataclass
@@ -345,8 +342,7 @@ class _Collection:
         limit = cfg.progress_log_interval_seconds if cfg.progress_log_interval_seconds > 0.0 else None
         if cfg.stall_timeout_seconds > 0.0:
             left = cfg.stall_timeout_seconds - (self.loop.time() - self.progress_at)
-            if left <= 0.0:
-                raise RuntimeError(f"Rollout runner stalled before wait: {self.summary()}")
+            reject(left <= 0.0, f"Rollout runner stalled before wait: {self.summary()}", RuntimeError)
             limit = left if limit is None else min(limit, left)
         return limit
 
@@ -356,8 +352,8 @@ class _Collection:
         if cfg.progress_log_interval_seconds > 0.0 and now - self.logged_at >= cfg.progress_log_interval_seconds:
             log.info("Rollout runner heartbeat: %s", self.summary())
             self.logged_at = now
-        if cfg.stall_timeout_seconds > 0.0 and now - self.progress_at >= cfg.stall_timeout_seconds:
-            raise RuntimeError(f"Rollout runner stalled waiting for completions: {self.summary()}")
+        reject(cfg.stall_timeout_seconds > 0.0 and now - self.progress_at >= cfg.stall_timeout_seconds,
+               f"Rollout runner stalled waiting for completions: {self.summary()}", RuntimeError)
 
     def absorb(self, done) -> None:
         for task in done:
@@ -511,8 +507,7 @@ class RolloutCoordinator:
         stats = self.last_stats
         nothing_to_do = (not found and waiting <= 0 and loaded <= 0 and stats.get("sampled_group_count", 0.0) <= 0.0
                          and stats.get("carried_in_unfinished_group_count", 0.0) <= 0.0)
-        if nothing_to_do:
-            raise RuntimeError("RolloutCoordinator could not build a prompt batch from the provided rows.")
+        reject(nothing_to_do, "RolloutCoordinator could not build a prompt batch from the provided rows.", RuntimeError)
         indices = []
         for item in found:   # dataset rows behind the batch, each once, in order of appearance
             row = getattr(item.example, "dataset_index", None)

@@ -31,12 +31,37 @@ from .cache import LFM25HybridCache
 from .config import LFM25SamplingConfig
 from .engine import flatten_token_batches
 from .types import BehaviorTopK
+from ._checks import reject
 
+_no_grad = torch.inference_mode   # every public method runs without autograd state
 STAT_KEYS = ("prefilled_tokens", "resumed_prefix_tokens", "appended_tokens", "admitted_requests", "resumed_requests",
              "decode_steps", "slot_refills", "peak_live_slots", "decode_row_steps", "reserved_row_steps",
              "adaptive_graph_captures", "forked_requests", "copied_prefix_tokens", "snapshot_prefilled_tokens",
              "snapshot_count", "peak_snapshots", "peak_snapshot_bytes")
 _SEED_MASK = (1 << 63) - 1
+# the reference's error texts (callers and tests match on them), by the condition that raises them
+_REFUSALS = {
+    "already_open": (RuntimeError, "A native generation session is already open"),
+    "head_width": (ValueError, "behavior_topk must be an integer between 0 and min(vocab, 128)"),
+    "closed": (RuntimeError, "Native generation session is closed"),
+    "session_policy": (ValueError, "Session cache belongs to another policy version"),
+    "sampling_per_prompt": (ValueError, "One sampling configuration is required per prompt"),
+    "snapshot_policy": (ValueError, "Snapshot belongs to another policy version"),
+    "snapshot_gone": (ValueError, "Snapshot is released or belongs to another session"),
+    "position_mismatch": (ValueError, "Cached position does not match the pending-token prefix"),
+    "foreign_handle": (ValueError, "Continuation handle belongs to another session"),
+    "stale_handle": (ValueError, "Continuation handle is stale or already consumed"),
+    "per_handle": (ValueError, "One prompt and sampling configuration is required per handle"),
+    "twice": (ValueError, "Cannot resume a handle twice"),
+    "prefix_differs": (ValueError, "Continuation requires the exact cached token prefix"),
+    "pause_rules": (ValueError, "Internal pauses must preserve the exact context, seed and stop rules"),
+    "steps": (ValueError, "steps must be a positive integer"),
+}
+
+
+def _refuse(condition: str):
+    kind, text = _REFUSALS[condition]
+    raise kind(text)
 
 
 # ---------------------------------------------------------------------------------------------- what callers hold
@@ -195,18 +220,17 @@ class _PhaseSpan:
 
 # ---------------------------------------------------------------------------------------------- the session
 class LFM25GenerationSession:
-    @torch.inference_mode()
+    @_no_grad()
     def __init__(self, decoder, *, max_batch_size: int, max_new_tokens: int, cache_len: int | None = None,
                  behavior_topk: int = 0, profile_timings: bool = False):
         if decoder._active_session is not None:
-            raise RuntimeError("A native generation session is already open")
+            _refuse("already_open")
         for name, value in (("max_batch_size", max_batch_size), ("max_new_tokens", max_new_tokens)):
-            if type(value) is not int or value <= 0:
-                raise ValueError(f"{name} must be a positive integer")
+            reject(type(value) is not int or value <= 0, f"{name} must be a positive integer")
         engine = decoder.engine
         vocab = engine.config.vocab_size
         if type(behavior_topk) is not int or not 0 <= behavior_topk <= min(128, vocab):
-            raise ValueError('behavior_topk must be an integer between 0 and min(vocab, 128)')
+            _refuse("head_width")
         self.decoder, self.engine = decoder, engine
         self.batch_size, self.max_new_tokens, self.behavior_topk = max_batch_size, max_new_tokens, behavior_topk
         self.policy_version = engine.policy_version
@@ -229,9 +253,9 @@ class LFM25GenerationSession:
     def _require_open(self) -> None:
         mine = self.decoder._active_session is self and self.engine._cuda_decoder is self.decoder
         if self.closed or not mine:
-            raise RuntimeError("Native generation session is closed")
+            _refuse("closed")
         if self.engine.policy_version != self.policy_version:
-            raise ValueError('Session cache belongs to another policy version')
+            _refuse("session_policy")
 
     def timing_stats(self) -> dict:
         """GPU seconds per phase (`prefill`, `cache_copy`, `append`), resolved once, outside the hot loop."""
@@ -257,8 +281,7 @@ class LFM25GenerationSession:
 
     def _validate(self, prompt, sampling: LFM25SamplingConfig) -> None:
         for broken, message in self._violations(prompt, sampling):
-            if broken:
-                raise ValueError(message)
+            reject(broken, message)
 
     def _claim(self, wanted, count: int, purpose: str) -> list:
         """`count` free slots: the lowest ones, or exactly the requested ones."""
@@ -268,8 +291,7 @@ class LFM25GenerationSession:
             chosen = [int(i) for i in wanted]
         ok = (len(chosen) == count and len(set(chosen)) == count
               and all(0 <= i < self.batch_size and not self.slots[i].busy for i in chosen))
-        if not ok:
-            raise ValueError(f"{purpose} requires distinct free session slots")
+        reject(not ok, f"{purpose} requires distinct free session slots")
         return chosen
 
     def _start(self, work, *, carried=None) -> None:
@@ -293,12 +315,12 @@ class LFM25GenerationSession:
         return graph, width
 
     # ------------------------------------------------------------------ admission
-    @torch.inference_mode()
+    @_no_grad()
     def admit(self, prompts: Sequence[Sequence[int]], samplings: Sequence[LFM25SamplingConfig], *,
               slots: Sequence[int] | None = None) -> list:
         self._require_open()
         if len(prompts) != len(samplings):
-            raise ValueError("One sampling configuration is required per prompt")
+            _refuse("sampling_per_prompt")
         chosen = self._claim(slots, len(prompts), "Admission")
         for prompt, sampling in zip(prompts, samplings):
             self._validate(prompt, sampling)
@@ -331,13 +353,13 @@ class LFM25GenerationSession:
     def _lookup(self, snapshot: LFM25PrefixSnapshot) -> _StoredPrefix:
         self._require_open()
         if snapshot.policy_version != self.engine.policy_version:
-            raise ValueError('Snapshot belongs to another policy version')
+            _refuse("snapshot_policy")
         stored = self._stored.get(snapshot.identity) if snapshot.session is self else None
         if stored is None or stored.lease is not snapshot:
-            raise ValueError('Snapshot is released or belongs to another session')
+            _refuse("snapshot_gone")
         return stored
 
-    @torch.inference_mode()
+    @_no_grad()
     def prefill_snapshot(self, prompt: Sequence[int]) -> LFM25PrefixSnapshot:
         """Prefill one exact prefix once under the current weights, outside the session's slots."""
         self._require_open()
@@ -351,14 +373,14 @@ class LFM25GenerationSession:
         self.stats["snapshot_prefilled_tokens"] += len(prompt)
         return self._store(_StoredPrefix(self._new_lease(prompt), cache, done.next_token_logits))
 
-    @torch.inference_mode()
+    @_no_grad()
     def snapshot(self, handle: LFM25ContinuationHandle) -> LFM25PrefixSnapshot:
         """Copy a delivered row: the valid part of its KV bytes and scales, its conv state, its logits and the token it
         still owes the model."""
         slot = self._leased(handle)
         cached = len(handle.prefix_token_ids) - 1
         if int(self.entry.cache.seq_lens[handle.slot]) != cached:
-            raise ValueError('Cached position does not match the pending-token prefix')
+            _refuse("position_mismatch")
         with self.clock("cache_copy"):
             row = self.entry.cache.rows(handle.slot, handle.slot + 1)
             history = [None if t is None else t[:, :, :cached].clone() for t in (row.k_cache, row.v_cache, row.k_scales, row.v_scales)]
@@ -371,7 +393,7 @@ class LFM25GenerationSession:
     def release_snapshot(self, snapshot: LFM25PrefixSnapshot) -> None:
         del self._stored[self._lookup(snapshot).lease.identity]
 
-    @torch.inference_mode()
+    @_no_grad()
     def fork(self, snapshot: LFM25PrefixSnapshot, samplings: Sequence[LFM25SamplingConfig], *,
              slots: Sequence[int] | None = None) -> list:
         """Start independent children of a stored prefix in free slots without any prefill."""
@@ -406,10 +428,10 @@ class LFM25GenerationSession:
     def _leased(self, handle: LFM25ContinuationHandle) -> _Slot:
         self._require_open()
         if handle.session is not self or not 0 <= handle.slot < self.batch_size:
-            raise ValueError("Continuation handle belongs to another session")
+            _refuse("foreign_handle")
         slot = self.slots[handle.slot]
         if slot.lease is not handle or slot.generation != handle.version:
-            raise ValueError("Continuation handle is stale or already consumed")
+            _refuse("stale_handle")
         return slot
 
     def _feed(self, queues: dict) -> None:
@@ -430,28 +452,28 @@ class LFM25GenerationSession:
         self.entry.input_tokens.copy_(owed_tokens)
         self.rows.pending.copy_(owed_flags)
 
-    @torch.inference_mode()
+    @_no_grad()
     def resume(self, handles: Sequence[LFM25ContinuationHandle], prompts: Sequence[Sequence[int]],
                samplings: Sequence[LFM25SamplingConfig], *, preserve_rng: bool = False) -> None:
         """Continue delivered rows from an exact extension of what they hold: the owed token and the new suffix are
         appended under per-row masks, then the rows run again.  `preserve_rng` keeps the random stream's position and
         the stop automaton's state (an internal pause of the same request)."""
         if not len(handles) == len(prompts) == len(samplings):
-            raise ValueError("One prompt and sampling configuration is required per handle")
+            _refuse("per_handle")
         if len({handle.slot for handle in handles}) != len(handles):
-            raise ValueError("Cannot resume a handle twice")
+            _refuse("twice")
         queues, carried = {}, {}
         for handle, prompt, sampling in zip(handles, prompts, samplings):
             slot = self._leased(handle)
             self._validate(prompt, sampling)
             held = handle.prefix_token_ids
             if tuple(prompt[:len(held)]) != held:
-                raise ValueError("Continuation requires the exact cached token prefix")
+                _refuse("prefix_differs")
             if preserve_rng:
                 before = slot.sampling
                 if (len(prompt) != len(held) or sampling.seed != before.seed or sampling.stop_table is not before.stop_table
                         or sampling.stop_token_ids != before.stop_token_ids):
-                    raise ValueError('Internal pauses must preserve the exact context, seed and stop rules')
+                    _refuse("pause_rules")
             queues[handle.slot] = [held[-1], *prompt[len(held):]]
         if not queues:
             return
@@ -476,13 +498,13 @@ class LFM25GenerationSession:
                                 top_ks=state.top_ks, top_ps=state.top_ps, out=(tokens, logprobs))
         return tokens, logprobs
 
-    @torch.inference_mode()
+    @_no_grad()
     def poll(self, *, steps: int | None = None) -> list:
         """Run `steps` decode steps (default: the decoder's finish-check interval) and hand out what finished."""
         self._require_open()
         steps = self.decoder.finish_check_interval if steps is None else steps
         if type(steps) is not int or steps <= 0:
-            raise ValueError("steps must be a positive integer")
+            _refuse("steps")
         running = [index for index, slot in enumerate(self.slots) if slot.running]
         if not running:
             return []
@@ -538,7 +560,7 @@ class LFM25GenerationSession:
                                               codes[index], head))
         return results
 
-    @torch.inference_mode()
+    @_no_grad()
     def release(self, handle: LFM25ContinuationHandle) -> None:
         """Give a delivered row's slot back."""
         slot = self._leased(handle)

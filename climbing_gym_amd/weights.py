@@ -14,6 +14,7 @@ from typing import Any, Mapping
 import torch
 
 from .config import LFM2Config, coerce_config
+from ._checks import reject
 
 SYNC_FIELDS = ("vocab_size", "hidden_size", "mlp_hidden_size", "num_hidden_layers", "num_attention_heads",
                "num_key_value_heads", "max_position_embeddings", "rope_theta", "norm_eps", "conv_kernel_size",
@@ -137,8 +138,8 @@ class LFM25PackedWeights:
             for attr, rows, key in _layer_sources(config, index, kind):
                 tensor = put(key)
                 if rows == "squeeze":
-                    if tensor.ndim != 3 or tensor.size(1) != 1:
-                        raise ValueError(f"Expected depthwise conv weight [H,1,K], got {tuple(tensor.shape)}")
+                    reject(tensor.ndim != 3 or tensor.size(1) != 1,
+                           f"Expected depthwise conv weight [H,1,K], got {tuple(tensor.shape)}")
                     tensor = tensor[:, 0, :].contiguous()
                 parts.setdefault(attr, []).append(tensor)
             packed = {a: (v[0] if len(v) == 1 else torch.cat(v, 0).contiguous()) for a, v in parts.items()}
@@ -172,16 +173,14 @@ class LFM25PackedWeights:
         source_cfg.validate()
         bad = [f"{f}: engine={getattr(self.config, f)!r}, model={getattr(source_cfg, f)!r}"
                for f in SYNC_FIELDS if getattr(self.config, f) != getattr(source_cfg, f)]
-        if bad:
-            raise ValueError("Cannot synchronize an incompatible LFM2 config (" + "; ".join(bad) + ")")
+        reject(bad, "Cannot synchronize an incompatible LFM2 config (" + "; ".join(bad) + ")")
         state = model.state_dict()
-        if not isinstance(state, Mapping):
-            raise TypeError("model.state_dict() must return a mapping of tensor names to tensors")
+        reject(not isinstance(state, Mapping),
+               "model.state_dict() must return a mapping of tensor names to tensors", TypeError)
         plan = []
 
         def add(name, destination, source):
-            if not torch.is_tensor(source):
-                raise TypeError(f"LFM25 sync source {name!r} is not a tensor")
+            reject(not torch.is_tensor(source), f"LFM25 sync source {name!r} is not a tensor", TypeError)
             if tuple(source.shape) != tuple(destination.shape):
                 raise ValueError(f"LFM25 sync shape mismatch for {name!r}: expected {tuple(destination.shape)}, "
                                  f"got {tuple(source.shape)}")
@@ -192,8 +191,8 @@ class LFM25PackedWeights:
         head_key = "model.lm_head.weight" if has(state, "model.lm_head.weight") else "model.embed_tokens.weight"
         add("model.lm_head.weight", self.lm_head_weight, lookup(state, head_key))
         for index, (kind, layer) in enumerate(zip(source_cfg.layer_types, self.layers, strict=True)):
-            if (kind == "full_attention") != (layer.attention is not None):
-                raise ValueError(f"LFM25 packed layer {index} does not match {kind} config")
+            reject((kind == "full_attention") != (layer.attention is not None),
+                   f"LFM25 packed layer {index} does not match {kind} config")
             for attr, rows, key in _layer_sources(source_cfg, index, kind):
                 target = layer
                 for part in attr.split("."):
@@ -201,10 +200,9 @@ class LFM25PackedWeights:
                 source = lookup(state, key)
                 if rows == "squeeze":
                     expected = (target.size(0), 1, target.size(1))
-                    if not torch.is_tensor(source):
-                        raise TypeError(f"LFM25 sync source {key!r} is not a tensor")
-                    if tuple(source.shape) != expected:
-                        raise ValueError(f"LFM25 sync shape mismatch for {key!r}: expected {expected}, got {tuple(source.shape)}")
+                    reject(not torch.is_tensor(source), f"LFM25 sync source {key!r} is not a tensor", TypeError)
+                    reject(tuple(source.shape) != expected,
+                           f"LFM25 sync shape mismatch for {key!r}: expected {expected}, got {tuple(source.shape)}")
                     plan.append((target, source[:, 0, :]))
                 else:
                     add(key, target if rows is None else target[rows[0]:rows[1]], source)
