@@ -40,6 +40,8 @@ _SIGNATURES = {
     "lfm2_fp8_gemm_rows": "ppppppp" "lllliip",
     "lfm2_fp8_gemm_swiglu": "ppppp" "llli" "p",
     "lfm2_bf16_gemm_swiglu": "ppp" "lll" "p",
+    "lfm2_fp8_gemm_conv_update": "ppppppppp" "lllli" "p",
+    "lfm2_bf16_gemm_conv_update": "ppppppp" "llll" "p",
     "lfm2_bf16_gemm_rows": "ppppp" "llllip",
     "lfm2_store_kv_fp8": "ppppppppp" "lliilllllllllip",
     "lfm2_append_kv": "ppppppp" "liilllip",
@@ -64,6 +66,7 @@ _SIGNATURES = {
 _INT64_RESULT = {
     "lfm2_fp8_gemm_workspace": "lll",
     "lfm2_gemm_swiglu_fits": "llli",
+    "lfm2_gemm_conv_fits": "llli",
     "lfm2_fp8_gemm_default_splits": "lll",
     "lfm2_bf16_gemm_default_splits": "lll",
     "lfm2_bf16_gemm_workspace": "lll",

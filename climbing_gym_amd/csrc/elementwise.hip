@@ -429,18 +429,6 @@ extern "C" int lfm2_quantize_rows(uint8_t* q, float* scales, const void* x, int6
 }
 
 // ------------------------------------------------------------------------------------ short-conv update
-// One channel of the gated short conv: taps (state[1], state[2], b*x) with weights w[0..2]; returns c * conv and the
-// new state entry b*x, every product and the tap sum rounded to T as the reference's kernel rounds them.
-template <typename T>
-__device__ __forceinline__ float conv_channel(float b, float c, float x, float s0, float s1, float w0, float w1, float w2,
-                                              float* bx_out) {
-  const float bx = round_to<T>(b * x);
-  const float p0 = round_to<T>(s0 * w0), p1 = round_to<T>(s1 * w1), p2 = round_to<T>(bx * w2);
-  const float conv = round_to<T>((p0 + p1) + p2);
-  *bx_out = bx;
-  return round_to<T>(c * conv);
-}
-
 // Eight consecutive channels of one row with 16-byte accesses (16-bit T): 3 loads of the (B, C, x) thirds, 3 of the
 // weights [8][3], 3 loads and 3 stores of the state [8][3].
 template <typename T>

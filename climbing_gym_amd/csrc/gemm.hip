@@ -102,13 +102,29 @@ __device__ __forceinline__ int swiglu_weight_row(int n, int N) {
   return ((n >> 4) << 3) + (n & 7) + ((n & 8) ? (N >> 1) : 0);
 }
 
+// The conv in-projection with the gated short-conv update as its epilogue (EPI = 3): the packed weight [B rows; C rows;
+// x rows] (N = 3 H) is walked so that output columns 48g .. 48g+47 are the B, C and x rows of channels 16g .. 16g+15,
+// 16 columns each: the three MFMA tiles of a wave (tile columns 96, two waves across) then hold B, C and x of the same
+// channels in the same lanes.
+__device__ __forceinline__ int conv_weight_row(int n, int N) {
+  const int group = n / 48, within = n % 48;
+  return (within >> 4) * (N / 3) + 16 * group + (within & 15);
+}
+struct ConvEpilogue {
+  const void* weight;        // [H, 3] model dtype
+  void* state;               // [slots, H, 3] model dtype, updated in place for rows that take part
+  const uint8_t* active;     // per row, or NULL
+  const int32_t* slot_ids;   // row -> state slot (negative: padding), or NULL for row = slot
+};
+
 // The kernel body; the two entry points below differ in their arguments only (the fused QKV projection carries its
 // epilogue's arguments, the plain products do not pay for them in every launch's argument block).
 template <int EB, int BM, int BN, int WM, int WN, int SW, int KS, bool KTAIL, int ST, int EPI>
 __device__ __forceinline__ void
 gemm_nt_body(void* __restrict__ out, float* __restrict__ partial, const uint8_t* __restrict__ A,
              const uint8_t* __restrict__ W, const float* __restrict__ a_scales, const float* __restrict__ w_scales,
-             int M, int N, int64_t Kb, int steps_per_split, int out_dtype, const RowMap& rows, const QkvEpilogue& epi) {
+             int M, int N, int64_t Kb, int steps_per_split, int out_dtype, const RowMap& rows, const QkvEpilogue& epi,
+             const ConvEpilogue& conv = ConvEpilogue{}) {
   constexpr int NT = WM * WN * 64;
   constexpr int TM = BM / WM, TN = BN / WN, MI = TM / 16, NI = TN / 16;
   constexpr int kChunksPerRow = KS / 16;  // KS = K bytes staged per step and row: 128, or 256 (two MFMA sub-steps per barrier)
@@ -224,7 +240,7 @@ gemm_nt_body(void* __restrict__ out, float* __restrict__ partial, const uint8_t*
     }
   };
 
-  static_assert(EPI != 2 || ST > 0, "the fused SwiGLU epilogue is built on the ring tiles");
+  static_assert((EPI != 2 && EPI != 3) || ST > 0, "the fused SwiGLU and conv epilogues are built on the ring tiles");
   if constexpr (ST > 0) {
     static_assert(!KTAIL, "direct-to-LDS loads cannot zero-fill a partial K step");
     static_assert(A_CHUNKS % 64 == 0 && W_CHUNKS % 64 == 0, "a wave fills 64 consecutive slots per instruction");
@@ -254,6 +270,7 @@ gemm_nt_body(void* __restrict__ out, float* __restrict__ partial, const uint8_t*
           int gr = n_base + row;
           gr = gr < N ? gr : N - 1;
           if (EPI == 2) gr = swiglu_weight_row(gr, N);
+          if (EPI == 3) gr = conv_weight_row(gr, N);
           __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(W + (int64_t)gr * Kb + kb + c * 16),
                                            (__attribute__((address_space(3))) void*)(&lds[buf][A_CHUNKS + i * NT + wave * 64]), 16, 0, 0);
         }
@@ -482,6 +499,65 @@ gemm_nt_body(void* __restrict__ out, float* __restrict__ partial, const uint8_t*
     return;
   }
 
+  if constexpr (EPI == 3) {
+    // conv_update of lfm25_cuda_kernels.py:75-110 on the product's own tile: B, C and x are rounded to the model dtype as
+    // the plain product stores them; a lane owns four channels of one row: their taps (12 values, contiguous in the
+    // state), their weights, their outputs.  out is [M, N / 3].
+    static_assert(NI == 3, "a wave's three MFMA tiles are B, C and x of the same channels");
+    auto finish_rows = [&](auto tag) {
+      typedef decltype(tag) T;
+      const int H = N / 3;
+      const int channel = ((n_base + wn * TN) / 48) * 16 + 4 * lgrp;
+      if (n_base + wn * TN >= N) return;
+      float wt[12];
+      {
+        const T* w = (const T*)conv.weight + (int64_t)channel * 3;
+#pragma unroll
+        for (int e = 0; e < 12; ++e) wt[e] = Elem<T>::load(w[e]);
+      }
+#pragma unroll
+      for (int i = 0; i < MI; ++i) {
+        const int m = m_base + wm * TM + i * 16 + lrow;
+        if (m >= M) continue;
+        const float sa = a_scales ? a_scales[m] : 1.0f;
+        float v[3][4];
+#pragma unroll
+        for (int t = 0; t < 3; ++t)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            float y = acc[i][t][r];
+            if (a_scales) y = (y * sa) * w_scales[t * H + channel + r];
+            v[t][r] = round_to<T>(y);
+          }
+        int64_t slot = m;
+        if (conv.slot_ids) { const int32_t sid = conv.slot_ids[m]; slot = sid < 0 ? 0 : sid; }
+        const bool on = conv.active ? conv.active[m] != 0 : true;
+        T* st = (T*)conv.state + (slot * H + channel) * 3;
+        float taps[12], fresh[12], y[4];
+#pragma unroll
+        for (int e = 0; e < 12; ++e) taps[e] = Elem<T>::load(st[e]);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float bx;
+          y[r] = conv_channel<T>(v[0][r], v[1][r], v[2][r], taps[3 * r + 1], taps[3 * r + 2], wt[3 * r], wt[3 * r + 1],
+                                 wt[3 * r + 2], &bx);
+          fresh[3 * r] = taps[3 * r + 1]; fresh[3 * r + 1] = taps[3 * r + 2]; fresh[3 * r + 2] = bx;
+        }
+        if (on) {
+#pragma unroll
+          for (int e = 0; e < 12; ++e) st[e] = Elem<T>::store(fresh[e]);
+        }
+        T* dst = (T*)out + (int64_t)m * H + channel;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) dst[r] = Elem<T>::store(y[r]);
+      }
+    };
+    if (out_dtype == LFM2_DTYPE_BF16) finish_rows(__bf16{});
+    else if (out_dtype == LFM2_DTYPE_F16) finish_rows(_Float16{});
+    else finish_rows(float{});
+    return;
+  }
+
   // Epilogue: lane holds out[m = .. + lrow][n = .. + 4*lgrp + r], r = 0..3.
   const bool split = partial != nullptr;
   auto finish = [&](f32x4 v, int m_out, int n, float sa) {  // scale (row then column) and store up to 4 columns
@@ -544,6 +620,17 @@ gemm_swiglu_kernel(void* __restrict__ out, const uint8_t* __restrict__ A, const 
   gemm_nt_body<EB, BM, BN, WM, WN, EB == 1 ? 1 : 0, 128, false, ST, 2>(out, nullptr, A, W, a_scales, w_scales, M, N, Kb,
                                                                          (int)(Kb / 128), out_dtype,
                                                                          RowMap{nullptr, nullptr, 0x7fffffff}, QkvEpilogue{});
+}
+
+// The conv in-projection with the short-conv update as its epilogue, on the 64 x 96 tile of the decode batch.
+template <int EB>
+__global__ void __launch_bounds__(512)
+gemm_conv_kernel(void* __restrict__ out, const uint8_t* __restrict__ A, const uint8_t* __restrict__ W,
+                 const float* __restrict__ a_scales, const float* __restrict__ w_scales, int M, int N, int64_t Kb,
+                 int out_dtype, ConvEpilogue conv) {
+  gemm_nt_body<EB, 64, 96, 4, 2, EB == 1 ? 1 : 0, 128, false, 4, 3>(out, nullptr, A, W, a_scales, w_scales, M, N, Kb,
+                                                                     (int)(Kb / 128), out_dtype,
+                                                                     RowMap{nullptr, nullptr, 0x7fffffff}, QkvEpilogue{}, conv);
 }
 
 // Sum split-K partials in split order, then scale (row scale, then column scale).  A separate launch on purpose:
@@ -820,6 +907,49 @@ int swiglu_entry(const char* name, void* out, const void* a, const float* as, co
   LFM2_LAUNCH_CHECK();
 }
 }  // namespace
+
+namespace {
+bool conv_fits(int64_t M, int64_t N, int64_t Kb) {
+  if (M <= 0 || N <= 0 || Kb <= 0 || N % 48 != 0 || Kb % kStepBytes != 0 || M >= (1 << 30) || N >= (1 << 30)) return false;
+  const Plan plan = default_plan(M, N, Kb);
+  return plan.tile == 37 && plan.splits == 1;
+}
+template <int EB>
+int conv_entry(const char* name, void* out, const void* a, const float* as, const void* w, const float* ws,
+               const void* conv_weight, void* state, const uint8_t* active, const int32_t* slot_ids, int64_t M, int64_t N,
+               int64_t K, int64_t slots, int out_dtype, void* stream) {
+  LFM2_REQUIRE(out && a && w && conv_weight && state, "%s: a required pointer is null", name);
+  LFM2_REQUIRE(out_dtype >= LFM2_DTYPE_BF16 && out_dtype <= LFM2_DTYPE_F32, "%s: bad output dtype", name);
+  LFM2_REQUIRE(((uintptr_t)a | (uintptr_t)w) % 16 == 0, "%s: operands must be aligned to 16 bytes", name);
+  LFM2_REQUIRE(slots > 0 && (slot_ids != nullptr || M <= slots), "%s: %ld rows but only %ld state slots", name, (long)M, (long)slots);
+  if (!conv_fits(M, N, K * EB)) LFM2_FAIL(LFM2_ERR_UNSUPPORTED, "%s: no fused form for M %ld, N %ld, K %ld", name, (long)M, (long)N, (long)K);
+  const int tiles = (int)(((M + 63) / 64) * (N / 96));
+  hipLaunchKernelGGL(gemm_conv_kernel<EB>, dim3((tiles + 7) / 8 * 8), dim3(512), 0, (hipStream_t)stream, out,
+                     (const uint8_t*)a, (const uint8_t*)w, as, ws, (int)M, (int)N, K * EB, out_dtype,
+                     ConvEpilogue{conv_weight, state, active, slot_ids});
+  LFM2_LAUNCH_CHECK();
+}
+}  // namespace
+
+extern "C" int lfm2_gemm_conv_fits(int64_t M, int64_t N, int64_t K, int element_bytes) {
+  return (element_bytes == 1 || element_bytes == 2) && conv_fits(M, N, K * element_bytes) ? 1 : 0;
+}
+
+extern "C" int lfm2_fp8_gemm_conv_update(void* out, const uint8_t* a_q, const float* a_scales, const uint8_t* w_q,
+                                         const float* w_scales, const void* conv_weight, void* state, const uint8_t* active,
+                                         const int32_t* slot_ids, int64_t M, int64_t N, int64_t K, int64_t slots,
+                                         int out_dtype, void* stream) {
+  LFM2_REQUIRE(a_scales && w_scales, "fp8_gemm_conv_update: scales are required");
+  return conv_entry<1>("fp8_gemm_conv_update", out, a_q, a_scales, w_q, w_scales, conv_weight, state, active, slot_ids, M, N,
+                       K, slots, out_dtype, stream);
+}
+
+extern "C" int lfm2_bf16_gemm_conv_update(void* out, const void* x, const void* w, const void* conv_weight, void* state,
+                                          const uint8_t* active, const int32_t* slot_ids, int64_t M, int64_t N, int64_t K,
+                                          int64_t slots, void* stream) {
+  return conv_entry<2>("bf16_gemm_conv_update", out, x, nullptr, w, nullptr, conv_weight, state, active, slot_ids, M, N, K,
+                       slots, LFM2_DTYPE_BF16, stream);
+}
 
 extern "C" int lfm2_gemm_swiglu_fits(int64_t M, int64_t N, int64_t K, int element_bytes) {
   return (element_bytes == 1 || element_bytes == 2) && swiglu_fits(M, N, K * element_bytes) ? 1 : 0;

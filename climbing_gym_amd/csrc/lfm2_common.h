@@ -56,6 +56,18 @@ template <typename T> __device__ __forceinline__ float round_to(float v) { retur
 // same bits).
 __device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
 
+// One channel of the gated short conv: taps (state[1], state[2], b*x) with weights w[0..2]; returns c * conv and the
+// new state entry b*x, every product and the tap sum rounded to T as the reference's kernel rounds them.
+template <typename T>
+__device__ __forceinline__ float conv_channel(float b, float c, float x, float s0, float s1, float w0, float w1, float w2,
+                                              float* bx_out) {
+  const float bx = round_to<T>(b * x);
+  const float p0 = round_to<T>(s0 * w0), p1 = round_to<T>(s1 * w1), p2 = round_to<T>(bx * w2);
+  const float conv = round_to<T>((p0 + p1) + p2);
+  *bx_out = bx;
+  return round_to<T>(c * conv);
+}
+
 // ---- wave / block reductions (64-lane wavefronts) ----------------------------------
 // All-reduce butterflies that stay in the vector ALU: two quad permutes, the two row mirrors (lane i <-> 7-i, then
 // i <-> 15-i: by then each half already holds one value, so a mirror pairs the halves), and gfx950's row and

@@ -267,13 +267,15 @@ class LFM25Engine:
             return packed.linear_quantized(x[0], x[1], dtype=self.dtype)
         return packed.linear(x) if packed is not None else ops.linear(x, weight)
 
-    def _backbone(self, tokens, attention_op, conv_op, fp8, *, defer_reduce=False, projecting_attention_op=None):
+    def _backbone(self, tokens, attention_op, conv_op, fp8, *, defer_reduce=False, projecting_attention_op=None,
+                  projecting_conv_op=None):
         """Embedding and all layers with the fused residual chain of lfm25_cuda.py:134-184: every RMSNorm also adds
         the previous block's output into the running residual; the first norm, which has nothing to add, runs in the
         launch that gathers the embedding rows.  Returns (last MLP output, residual).  With `defer_reduce` (decode) a
         split-K down projection hands its partial sums to the next norm.  `projecting_attention_op(op, packed, rows_q,
         row_scales)` (decode), when it takes the layer (returns something), runs the W8A8 QKV projection itself, with the
-        head preparation and the KV append as the product's epilogue."""
+        head preparation and the KV append as the product's epilogue; `projecting_conv_op(op, normed)` likewise runs the conv
+        in-projection with the short-conv update as its epilogue."""
         layers = self.weights.layers
         if not layers:
             return ops.embedding(tokens, self.weights.embed_tokens), None
@@ -295,7 +297,10 @@ class LFM25Engine:
                 mixed = self._linear(attended, op.out_weight, fp8)
             else:
                 op = layer.conv
-                mixed = self._linear(conv_op(op, self._project(normed, op.in_weight, fp8)), op.out_weight, fp8)
+                gated = projecting_conv_op(op, normed) if projecting_conv_op is not None else None
+                if gated is None:   # no fused projection for this shape: the plain one, then the conv launch
+                    gated = conv_op(op, self._project(normed, op.in_weight, fp8))
+                mixed = self._linear(gated, op.out_weight, fp8)
             # gate+up projection and SwiGLU: one launch where the product's shape has the fused form (packed prefill
             # chunks), the projection and the SwiGLU launch otherwise (decode); the same bits either way
             normed, residual = self._normed(mixed, layer.ffn_norm_weight, residual, layer.w13_weight, fp8)
@@ -383,8 +388,20 @@ class LFM25Engine:
                              scale=self._scaling, slot_ids=slot_ids, schedule=schedule, quantized=quantized)
             return out if quantized else out.view(rows, -1)
 
+        def projecting_conv_op(op, normed):
+            # With a W8A8 out projection the conv launch that also quantises its rows is as fast as this form plus a
+            # quantise launch (1.5438 against 1.5454 ms per step), so the fused projection serves the model-dtype path,
+            # where it removes a launch per conv layer (all-bf16 step 2.178 -> 2.150 ms).
+            if id(op.out_weight) in fp8:
+                return None
+            state = cache.conv_state[op.cache_index]
+            packed = fp8.get(id(op.in_weight))
+            if packed is not None:
+                return packed.linear_conv_update(normed[0], normed[1], op.conv_weight, state, active, slot_ids, dtype=self.dtype)
+            return ops.linear_conv_update(normed, op.in_weight, op.conv_weight, state, active, slot_ids)
+
         hidden, residual = self._backbone(tokens, attention_op, conv_op, fp8, defer_reduce=True,
-                                          projecting_attention_op=projecting_attention_op)
+                                          projecting_attention_op=projecting_attention_op, projecting_conv_op=projecting_conv_op)
         place = None if logits_out is None else ops.RowPlacement(logits_out, slot_ids, active)
         logits = self._head(hidden, residual, fp8, place)
         if advance_after:

@@ -316,6 +316,27 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor):
     return out
 
 
+def _conv_rows(rows: int, state, active, slot_ids):
+    reject(state.ndim != 3 or state.size(2) != 3 or not state.is_contiguous(), "conv state must be a contiguous [slots, H, 3] tensor")
+    reject(slot_ids is None and rows > state.size(0), "more rows than conv state slots")
+
+
+def linear_conv_update(x: torch.Tensor, weight: torch.Tensor, conv_weight, state, active=None, slot_ids=None):
+    """`conv_update(linear(x, weight), conv_weight, state, active, slot_ids)` for the packed in-projection weight [3H, K]
+    (lfm25_cuda_kernels.py:19-29 then :103-110) in one launch, the same bits, where the product's shape has the fused
+    form; None otherwise (the caller runs the two launches)."""
+    reject(x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16, "linear runs in bfloat16 only: this package has no GEMM for other dtypes")
+    _check(x, weight, conv_weight)
+    m, k, n = _rows(x), x.size(-1), weight.size(0)
+    reject(weight.size(1) != k or n % 3 or conv_weight.shape != (n // 3, 3), "in-projection, conv weight and activation shapes differ")
+    if x.ndim != 2 or not query("lfm2_gemm_conv_fits", m, n, k, 2):
+        return None
+    _conv_rows(m, state, active, slot_ids)
+    out = torch.empty((m, n // 3), device=x.device, dtype=x.dtype)
+    call("lfm2_bf16_gemm_conv_update", out, x, weight, conv_weight, state, active, slot_ids, m, n, k, state.size(0))
+    return out
+
+
 @dataclass
 class PackedFP8Weight:
     """lfm25_fp8.py:120-168: per-output-channel e4m3 copy of a weight.  `refresh()` re-quantises into the
@@ -359,6 +380,22 @@ class PackedFP8Weight:
         need = query("lfm2_fp8_gemm_workspace", batch, rows, width) if split_k == 0 else max(split_k, 1) * batch * rows
         ws = torch.empty(need, device=x.device, dtype=torch.float32) if need and split_k != 1 else None
         call("lfm2_fp8_gemm", out, x, scales, self.values, self.scales, ws, batch, rows, width, _code(dtype), tile, split_k)
+        return out
+
+    def linear_conv_update(self, x, scales, conv_weight, state, active=None, slot_ids=None, *, dtype=torch.bfloat16):
+        """For the packed conv in-projection weight: `conv_update(self.linear_quantized(x, scales), conv_weight, state,
+        active, slot_ids)` (lfm25_fp8.py:141-168 then lfm25_cuda_kernels.py:103-110) in one launch, the same bits,
+        where the product's shape has the fused form; None otherwise."""
+        batch, width = x.shape
+        rows = self.values.size(0)
+        reject(width != self.values.size(1) or rows % 3 or conv_weight.shape != (rows // 3, 3),
+               "in-projection, conv weight and activation shapes differ")
+        if not query("lfm2_gemm_conv_fits", batch, rows, width, 1):
+            return None
+        _conv_rows(batch, state, active, slot_ids)
+        out = torch.empty((batch, rows // 3), device=x.device, dtype=dtype)
+        call("lfm2_fp8_gemm_conv_update", out, x, scales, self.values, self.scales, conv_weight, state, active, slot_ids,
+             batch, rows, width, state.size(0), _code(dtype))
         return out
 
     def linear_swiglu_quantized(self, x, scales, *, dtype=torch.bfloat16):

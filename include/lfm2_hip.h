@@ -163,6 +163,19 @@ int lfm2_fp8_gemm_swiglu(void* out, const uint8_t* a_q, const float* a_scales, c
                          int64_t M, int64_t N, int64_t K, int out_dtype, void* stream);
 int lfm2_bf16_gemm_swiglu(void* out, const void* x, const void* w, int64_t M, int64_t N, int64_t K, void* stream);
 
+/* The conv in-projection with the gated short-conv update as its epilogue (decode): w[N, K] is the packed in-projection
+ * weight [B rows; C rows; x rows] (N = 3 H); out[M, H] and the in-place update of state[slots, H, 3] are bit for bit
+ * lfm2_fp8_gemm / lfm2_bf16_gemm followed by lfm2_conv_update (lfm25_cuda_kernels.py:75-110) with the same active and
+ * slot_ids arguments, without the [M, 3 H] intermediate.  Built on one tile shape: lfm2_gemm_conv_fits(M, N, K, element
+ * bytes of the operands) says whether a shape has the fused form; LFM2_ERR_UNSUPPORTED otherwise. */
+int lfm2_gemm_conv_fits(int64_t M, int64_t N, int64_t K, int element_bytes);
+int lfm2_fp8_gemm_conv_update(void* out, const uint8_t* a_q, const float* a_scales, const uint8_t* w_q, const float* w_scales,
+                              const void* conv_weight, void* state, const uint8_t* active, const int32_t* slot_ids,
+                              int64_t M, int64_t N, int64_t K, int64_t slots, int out_dtype, void* stream);
+int lfm2_bf16_gemm_conv_update(void* out, const void* x, const void* w, const void* conv_weight, void* state,
+                               const uint8_t* active, const int32_t* slot_ids, int64_t M, int64_t N, int64_t K,
+                               int64_t slots, void* stream);
+
 /* The two products with placed output rows: row m of the product is written to out row out_rows[m] (m itself when
  * out_rows is NULL) unless that index is negative or >= out_capacity, or row_active[m] is 0 (row_active may be
  * NULL); other rows of out keep their contents.  This is the head projection followed by _scatter_logits of

@@ -1055,3 +1055,41 @@ def test_gate_up_projection_with_swiglu_epilogue_equals_the_two_launches(ops, fp
         want = ops.swiglu(ops.linear(x, weight))
         got = ops.linear_swiglu(x, weight)
         assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+@pytest.mark.parametrize("fp8", (True, False))
+@pytest.mark.parametrize("rows,mapped", [(256, False), (200, False), (160, True)])
+@torch.inference_mode()
+def test_conv_in_projection_with_conv_update_epilogue_equals_the_two_launches(ops, fp8, rows, mapped):
+    """The fused conv in-projection (gated short-conv update in the product's epilogue, [M, H] written, state updated)
+    against the projection followed by the conv-update launch, bit for bit: outputs and every slot's state, with an
+    activity mask (rows that sit out keep their taps but still get an output) and, for the compact form, rows mapped to
+    slots through slot ids with padding rows."""
+    torch.manual_seed(rows)
+    hidden, k, slots = 2048, 2048, 300
+    weight = (torch.randn(3 * hidden, k, device=DEV) * 0.05).bfloat16()
+    conv_weight = torch.randn(hidden, 3, device=DEV).bfloat16()
+    x = torch.randn(rows, k, device=DEV).bfloat16()
+    state = torch.randn(slots, hidden, 3, device=DEV).bfloat16()
+    active = torch.rand(rows, device=DEV) < 0.8
+    slot_ids = None
+    if mapped:
+        slot_ids = torch.randperm(slots, device=DEV)[:rows].to(torch.int32)
+        slot_ids[-7:] = -1
+        active[-7:] = False
+    assert ops.query("lfm2_gemm_conv_fits", rows, 3 * hidden, k, 1 if fp8 else 2) == 1
+    assert ops.query("lfm2_gemm_conv_fits", 64, 3 * hidden, k, 1 if fp8 else 2) == 0
+    want_state, got_state = state.clone(), state.clone()
+    if fp8:
+        packed = ops.PackedFP8Weight.from_weight(weight)
+        xq, xs = ops.quantize_rows(x)
+        want = ops.conv_update(packed.linear_quantized(xq, xs), conv_weight, want_state, active, slot_ids)
+        got = packed.linear_conv_update(xq, xs, conv_weight, got_state, active, slot_ids)
+        assert packed.linear_conv_update(xq[:64], xs[:64], conv_weight, got_state.clone(), None, None) is None
+    else:
+        want = ops.conv_update(ops.linear(x, weight), conv_weight, want_state, active, slot_ids)
+        got = ops.linear_conv_update(x, weight, conv_weight, got_state, active, slot_ids)
+    live = slice(0, rows - 7) if mapped else slice(0, rows)   # padding rows have no defined output
+    assert torch.equal(got[live].view(torch.int16), want[live].view(torch.int16))
+    assert torch.equal(got_state.view(torch.int16), want_state.view(torch.int16))
+    assert not torch.equal(got_state, state)
