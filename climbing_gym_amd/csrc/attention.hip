@@ -335,8 +335,11 @@ __device__ __forceinline__ int quad_transpose_bytes(int x, int lane) {
 // and nothing is loaded straight into LDS (with such a load in flight the compiler waits for all loads at once).
 struct ItemRecord { int b, chunk, len, slot; };
 
-template <bool PAGED, bool FP8>
+template <bool PAGED, bool FP8, bool ROWHEAD = false>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) decode_attn_mfma_kernel(DecodeArgs a) {
+  // ROWHEAD: a workgroup owns one (row, KV head): its four waves take the history's tiles round robin, merge their
+  // four partial results through LDS and write the row's output themselves; no partial results leave the chip and no
+  // merge launch follows.  Workgroup r * KH + h takes the row of rank r by length (longest first).
   constexpr int D = 64;
   constexpr int TT = FP8 ? 64 : 32;   // tokens per tile: 4 KiB of K rows and 4 KiB of V rows either way
   constexpr int ES = FP8 ? 1 : 2;     // bytes per element of the history
@@ -345,10 +348,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
   __shared__ __bf16 lds_p[4][4][64];   // one P tile per wave; nothing in LDS is shared between waves
   __shared__ __attribute__((aligned(16))) uint8_t lds_v[4][TT][D * ES];   // per wave: the tile's V rows, for the transposing read
   __shared__ __attribute__((aligned(16))) __bf16 lds_q[4][4][D];          // per wave: the item's query rows
+  __shared__ float lds_merge[ROWHEAD ? 4 : 1][4][D + 2];   // per wave and head: O[dim], then the maximum and the sum
   const int32_t* const records = a.schedule + kSchedRows + 4 * a.B;
-  const int items = a.schedule[0] * a.KH;
-  const int first = blockIdx.x * 4 + wave, nwaves = gridDim.x * 4;
+  const int items = ROWHEAD ? 1 : a.schedule[0] * a.KH;
+  const int first = ROWHEAD ? 0 : blockIdx.x * 4 + wave, nwaves = gridDim.x * 4;
   if (first >= items) return;
+  constexpr int kStride = ROWHEAD ? 4 * TT : TT;   // from one tile of a wave to its next
 
   // ---- the pieces of the pipeline
   // An item's record comes through the scalar cache (nothing writes the records while this kernel runs, so they are
@@ -439,17 +444,33 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
   int idx = first, idx_next = first + nwaves;
   int b, chunk, len, h;
   int64_t slot;
-  {
+  i32x4 rec_next;
+  int chunk_tokens, wbeg, wend;
+  if constexpr (ROWHEAD) {
+    const int rank = blockIdx.x / a.KH;
+    h = blockIdx.x % a.KH;
+    b = a.schedule[kSchedRows + 4 * rank + 3];
+    len = a.schedule[kSchedRows + 4 * b + 2];
+    slot = a.slot_ids ? a.slot_ids[b] : b;
+    chunk = 0; chunk_tokens = 0; rec_next = i32x4{0, 0, 0, 0};
+    wbeg = wave * TT;
+    wend = len;
+    if (len <= 0) {   // a row that sits out: zeros, as the merge kernel writes them (the same for the whole workgroup)
+      if (wave < a.G) ((__bf16*)a.out)[((int64_t)b * a.QH + h * a.G + wave) * D + lane] = (__bf16)0.f;
+      return;
+    }
+  } else {
     const i32x4 rec = read_record(idx);
     b = rec[0]; chunk = rec[1]; len = rec[2]; slot = rec[3]; h = idx % a.KH;
+    rec_next = read_record(idx_next);
+    chunk_tokens = a.schedule[1];
+    wbeg = chunk * chunk_tokens;
+    wend = wbeg + chunk_tokens;
+    wend = wend < len ? wend : len;
   }
-  i32x4 rec_next = read_record(idx_next);
-  const int chunk_tokens = a.schedule[1];
-  int wbeg = chunk * chunk_tokens;
-  int wend = wbeg + chunk_tokens;
-  wend = wend < len ? wend : len;
   Tile tile, ahead;
-  fetch(b, slot, h, wbeg, wend, tile);
+  const bool has_tiles = !ROWHEAD || wbeg < wend;   // the same for the whole wave
+  if (has_tiles) fetch(b, slot, h, wbeg, wend, tile);
 
   float m[4], l[4];
   f32x4 acc;   // O[head 0..3][dim lane]
@@ -466,17 +487,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
     }
     // ---- the next tile of the stream: this item's, or the first of the next item (its record was asked for one
     // item ago); without a next item, the current tile again (a cache hit)
-    const bool last = T + TT >= wend;
+    const bool last = T + kStride >= wend;
     int nb = b, nlen = len, nh = h, nwbeg = wbeg, nwend = wend;
     int64_t nslot = slot;
-    const bool have_next = last && idx_next < items;
+    const bool have_next = !ROWHEAD && last && idx_next < items;
     if (have_next) {
       nb = rec_next[0]; nlen = rec_next[2]; nslot = rec_next[3]; nh = idx_next % a.KH;
       nwbeg = rec_next[1] * chunk_tokens;
       nwend = nwbeg + chunk_tokens;
       nwend = nwend < nlen ? nwend : nlen;
     }
-    const int fT = last ? (have_next ? nwbeg : T) : T + TT;
+    const int fT = last ? (have_next ? nwbeg : T) : T + kStride;
     fetch(nb, nslot, nh, fT, nwend, nxt);
 
     const bool valid = T + tl < wend;
@@ -563,12 +584,20 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
       }
     }
     }
-    T += TT;
+    T += kStride;
     if (!last) return true;
 
     // ---- item end.  Wave totals of l; lane L holds O[head 0..3][dim L], so a head's row leaves as 256 contiguous bytes
 #pragma unroll
     for (int i = 0; i < 4; ++i) l[i] = wave_sum(l[i]);
+    if constexpr (ROWHEAD) {   // this wave's share of the (row, KV head) is done: its partial result waits in LDS
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        lds_merge[wave][i][lane] = acc[i];
+        if (lane == 0) { lds_merge[wave][i][D] = m[i]; lds_merge[wave][i][D + 1] = l[i]; }
+      }
+      return false;
+    }
     // The partial results leave through hand-written stores.  Reads and writes share one counter and complete out
     // of order with respect to each other, so with a store it knows of in flight the compiler turns every wait for
     // a load into a wait for everything, which would stop the stream at each item.  Unknown to it, a pending store
@@ -595,7 +624,33 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
     rec_next = read_record(idx_next);
     return true;
   };
-  while (step(tile, ahead) && step(ahead, tile)) {}
+  if (has_tiles) {
+    while (step(tile, ahead) && step(ahead, tile)) {}
+  }
+  if constexpr (ROWHEAD) {
+    if (!has_tiles) {   // a history shorter than this wave's first tile: a neutral partial result
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        lds_merge[wave][i][lane] = 0.f;
+        if (lane == 0) { lds_merge[wave][i][D] = -1.0e30f; lds_merge[wave][i][D + 1] = 0.f; }
+      }
+    }
+    __syncthreads();
+    // wave w merges query head w of the group over the four partial results: lane = dim, one 128-byte row out
+    if (wave < a.G) {
+      float mm = -1.0e30f;
+#pragma unroll
+      for (int p = 0; p < 4; ++p) mm = fmaxf(mm, lds_merge[p][wave][D]);
+      float lt = 0.f, o = 0.f;
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        const float f = __builtin_amdgcn_exp2f(lds_merge[p][wave][D] - mm);
+        lt = fmaf(lds_merge[p][wave][D + 1], f, lt);
+        o = fmaf(lds_merge[p][wave][lane], f, o);
+      }
+      ((__bf16*)a.out)[((int64_t)b * a.QH + h * a.G + wave) * D + lane] = (__bf16)(o * (1.0f / fmaxf(lt, 1.0e-20f)));
+    }
+  }
 }
 
 // One workgroup turns the rows' lengths into the item list of the persistent kernel: row b contributes
@@ -729,6 +784,29 @@ schedule_rows(int32_t* schedule, const int32_t* positions, const uint8_t* active
       class_base[threadIdx.x] += add;
     }
     __syncthreads();
+  }
+  // The rows by decreasing length, for the kernel that gives every (row, KV head) a workgroup of its own: the spare
+  // word of record r names the row of rank r (ties: the lower row first).  A bitonic sort of (length, row) keys in
+  // LDS, one key per thread: batches of up to 1024 rows; larger ones keep the item list.
+  if (B <= 1024) {
+    __shared__ unsigned keys[1024];
+    int width = 64;
+    while (width < B) width <<= 1;
+    const int t = threadIdx.x;
+    if (t < width) keys[t] = t < B ? ((unsigned)row_length(t) << 10) | (unsigned)(1023 - t) : 0u;
+    __syncthreads();
+    for (int k = 2; k <= width; k <<= 1) {
+      for (int j = k >> 1; j > 0; j >>= 1) {
+        const int partner = t ^ j;
+        if (t < width && partner > t) {
+          const unsigned mine = keys[t], theirs = keys[partner];
+          const bool descending = (t & k) == 0;
+          if ((mine < theirs) == descending) { keys[t] = theirs; keys[partner] = mine; }
+        }
+        __syncthreads();
+      }
+    }
+    if (t < B) schedule[kSchedRows + 4 * t + 3] = 1023 - (int)(keys[t] & 1023u);
   }
 }
 
@@ -1221,6 +1299,24 @@ extern "C" int lfm2_decode_attention(void* out, const void* q, const void* k_cac
       schedule = own;
     }
     a.schedule = schedule;
+    // With at least four workgroups per CU to hand out, every (row, KV head) gets a workgroup of its own, longest rows
+    // first: the output is written by the kernel itself (no partial results, no merge launch); rows quantised for a
+    // W8A8 out projection go through the row quantiser.  Smaller batches keep the item list, which balances a handful
+    // of long rows over all the waves.
+    if ((int64_t)B * KH >= 1024 && B <= 1024) {
+      float* scratch = workspace;   // bf16 rows [B, QH * D] when the caller only wants the quantised rows
+      a.out = out ? out : (void*)scratch;
+      const dim3 rgrid((unsigned)(B * KH));
+      if (kv_fp8) {
+        if (block_table) hipLaunchKernelGGL((decode_attn_mfma_kernel<true, true, true>), rgrid, dim3(256), 0, s, a);
+        else hipLaunchKernelGGL((decode_attn_mfma_kernel<false, true, true>), rgrid, dim3(256), 0, s, a);
+      } else {
+        if (block_table) hipLaunchKernelGGL((decode_attn_mfma_kernel<true, false, true>), rgrid, dim3(256), 0, s, a);
+        else hipLaunchKernelGGL((decode_attn_mfma_kernel<false, false, true>), rgrid, dim3(256), 0, s, a);
+      }
+      if (out_q) return lfm2_quantize_rows(out_q, out_scales, a.out, B, (int64_t)QH * D, dtype, stream);
+      LFM2_LAUNCH_CHECK();
+    }
     // 3 workgroups per CU (the register budget of 128 would allow 4, but with a handful of items per wave more
     // waves only make the shares of work more unequal); never more than the worst case
     int64_t blocks = ((int64_t)B * nch * KH + 3) / 4;
