@@ -1223,6 +1223,10 @@ extern "C" int lfm2_store_kv_packed(const void* k, const void* v, void* k_cache,
   LFM2_LAUNCH_CHECK();
 }
 
+// (row, KV head) workgroups from which the row-head kernel is used.  Decode step of the 1.2B shape against the item
+// list, prompts U[256, 2048] / U[6000, 7000]: 1 row 0.800 / 0.888 ms against 0.837 / 0.869, 8 rows 0.840 / 0.922 against
+// 0.863 / 0.929, 16 rows 0.850 / 0.949 against 0.875 / 1.001, 64 rows 0.995 / 1.367 against 1.043 / 1.497.
+constexpr int kRowHeadMinGroups = 64;
 constexpr int kMinChunk = kMfmaChunk < kChunk ? kMfmaChunk : kChunk;
 static int64_t schedule_ints(int64_t B, int64_t capacity) {
   return kSchedRows + 4 * B + 4 * B * ((capacity + kMfmaChunk - 1) / kMfmaChunk);
@@ -1299,11 +1303,11 @@ extern "C" int lfm2_decode_attention(void* out, const void* q, const void* k_cac
       schedule = own;
     }
     a.schedule = schedule;
-    // With at least four workgroups per CU to hand out, every (row, KV head) gets a workgroup of its own, longest rows
-    // first: the output is written by the kernel itself (no partial results, no merge launch); rows quantised for a
-    // W8A8 out projection go through the row quantiser.  Smaller batches keep the item list, which balances a handful
-    // of long rows over all the waves.
-    if ((int64_t)B * KH >= 1024 && B <= 1024) {
+    // From a few dozen (row, KV head) pairs on, each pair gets a workgroup of its own, longest rows first: the output is
+    // written by the kernel itself (no partial results, no merge launch); rows quantised for a W8A8 out projection go
+    // through the row quantiser.  A handful of rows keeps the item list, which spreads one long history over all the
+    // waves; so do batches beyond the 1024 rows the work-list launch sorts.
+    if ((int64_t)B * KH >= kRowHeadMinGroups && B <= 1024) {
       float* scratch = workspace;   // bf16 rows [B, QH * D] when the caller only wants the quantised rows
       a.out = out ? out : (void*)scratch;
       const dim3 rgrid((unsigned)(B * KH));
