@@ -283,7 +283,7 @@ def attention_workload(args):
         "dtype": "fp8_e4m3 history, bf16 queries, fp32 accumulate", "data": "synthetic",
         "config": {"workload": "one decode-attention call: 256 sequences, history U[128,8192] tokens, 32 query / 8 KV heads x 64, "
                                "dense and 16-token pages, e4m3 + scales and bf16", "context_tokens": tokens, "variants": results},
-        "roofline": {"kernel": "decode_attn_mfma_kernel + decode_combine_row_kernel", "bound": "hbm", "achieved": head["GB/s"],
+        "roofline": {"kernel": "decode_attn_mfma_kernel (one workgroup per row and KV head) + quantize_kernel", "bound": "hbm", "achieved": head["GB/s"],
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(head["GB/s"] / HBM_PEAK_GBS, 4), "traffic": None},
         "cpu_baseline": None}))
 
@@ -602,8 +602,8 @@ def main():
                    "gemm": gemms, "step_algorithmic_bytes": step_bytes,
                    "step_hbm_fraction": round(step_bytes / (ms_per_step / 1000) / 1e9 / HBM_PEAK_GBS, 4),
                    "mid_job": mid_job},
-        "roofline": {"kernel": "decode_attn_mfma_kernel + decode_combine_row_kernel (one ragged GQA decode-attention call, e4m3 KV, rows quantised for the W8A8 out projection as in the decode step)"
-                               if fp8 else "decode_attn_mfma_kernel + decode_combine_row_kernel (one ragged GQA decode-attention call, bf16 KV)",
+        "roofline": {"kernel": "decode_attn_mfma_kernel, one workgroup per row and KV head, + quantize_kernel (one ragged GQA decode-attention call, e4m3 KV, rows quantised for the W8A8 out projection as in the decode step)"
+                               if fp8 else "decode_attn_mfma_kernel, one workgroup per row and KV head (one ragged GQA decode-attention call, bf16 KV)",
                      "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(args, attn_bytes),
                      "avg_launch_us": round(attn_s * 1e6, 2), "algorithmic_bytes_per_launch": attn_bytes},
