@@ -339,7 +339,7 @@ template <bool PAGED, bool FP8, bool ROWHEAD = false>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) decode_attn_mfma_kernel(DecodeArgs a) {
   // ROWHEAD: a workgroup owns one (row, KV head): its four waves take the history's tiles round robin, merge their
   // four partial results through LDS and write the row's output themselves; no partial results leave the chip and no
-  // merge launch follows.  Workgroup r * KH + h takes the row of rank r by length (longest first).
+  // merge launch follows.  Rows are taken by rank of length, longest first.
   constexpr int D = 64;
   constexpr int TT = FP8 ? 64 : 32;   // tokens per tile: 4 KiB of K rows and 4 KiB of V rows either way
   constexpr int ES = FP8 ? 1 : 2;     // bytes per element of the history
@@ -447,8 +447,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
   i32x4 rec_next;
   int chunk_tokens, wbeg, wend;
   if constexpr (ROWHEAD) {
-    const int rank = blockIdx.x / a.KH;
-    h = blockIdx.x % a.KH;
+    // workgroup ids are dealt round robin over the 8 XCDs: the KV heads of one row go to one XCD, one after the other,
+    // so that with token-major histories (a token's heads share cache lines) the heads meet in one L2
+    const int stream = blockIdx.x / 8;
+    const int rank = 8 * (stream / a.KH) + (int)(blockIdx.x % 8);
+    h = stream % a.KH;
+    if (rank >= a.B) return;
     b = a.schedule[kSchedRows + 4 * rank + 3];
     len = a.schedule[kSchedRows + 4 * b + 2];
     slot = a.slot_ids ? a.slot_ids[b] : b;
@@ -1310,7 +1314,7 @@ extern "C" int lfm2_decode_attention(void* out, const void* q, const void* k_cac
     if ((int64_t)B * KH >= kRowHeadMinGroups && B <= 1024) {
       float* scratch = workspace;   // bf16 rows [B, QH * D] when the caller only wants the quantised rows
       a.out = out ? out : (void*)scratch;
-      const dim3 rgrid((unsigned)(B * KH));
+      const dim3 rgrid((unsigned)(8 * KH * ((B + 7) / 8)));
       if (kv_fp8) {
         if (block_table) hipLaunchKernelGGL((decode_attn_mfma_kernel<true, true, true>), rgrid, dim3(256), 0, s, a);
         else hipLaunchKernelGGL((decode_attn_mfma_kernel<false, true, true>), rgrid, dim3(256), 0, s, a);
