@@ -446,13 +446,64 @@ def test_decode_over_more_rows_than_one_scan_block(ops, quantized, fp8):
     assert torch.count_nonzero(result[~active]) == 0
 
 
+@pytest.mark.parametrize("groups", [1, 2, 4])
+@pytest.mark.parametrize("quantized", [False, True])
 @pytest.mark.parametrize("fp8", [True, False])
 @torch.inference_mode()
-def test_paged_slot_mapped_history_equals_dense_history(ops, fp8):
+def test_decode_with_a_workgroup_per_row_and_kv_head_matches_the_oracle(ops, groups, quantized, fp8):
+    """37 rows of 8 KV heads: from 64 (row, KV head) pairs on, a workgroup's four waves share one pair's tiles and merge
+    through LDS.  Lengths sit on both sides of the 32- and 64-token tile and of the four-tile round; a row count that is
+    no multiple of 8 leaves empty places in the last round of the XCD mapping; inactive rows and padding slots give
+    zeros; every live row is checked against the oracle."""
+    torch.manual_seed(41)
+    rows, capacity, heads, dim = 37, 700, 8, 64
+    k = torch.randn(rows, capacity, heads, dim).bfloat16()
+    v = torch.randn_like(k)
+    q = torch.randn(rows, 1, heads * groups, dim).bfloat16()
+    lengths = torch.randint(1, capacity + 1, (rows,))
+    fixed = [1, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 511, 512, 513, 700]
+    lengths[:len(fixed)] = torch.tensor(fixed)
+    active = torch.rand(rows) > 0.15
+    slots = torch.randperm(rows).to(torch.int32)
+    padding = [5, 20]
+    slots[padding] = -1
+    if fp8:
+        kc, vc, ks, vs = _cache_tensors(rows, capacity, heads, dim, "HND")
+        ops.store_kv(k.to(DEV), v.to(DEV), kc, vc, ks, vs)
+        hist = (kc.cpu(), vc.cpu(), ks.cpu(), vs.cpu())
+    else:
+        head_major = lambda t: t.to(DEV).permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+        kc, vc, ks, vs = head_major(k), head_major(v), None, None
+        hist = (k, v, [None] * rows, [None] * rows)
+    positions = (lengths[slots.clamp_min(0).long()] - 1).to(torch.int32)     # row i reads slot slots[i]
+    out = ops.attend(q.to(DEV), kc, vc, ks, vs, positions.to(DEV), active=active.to(DEV), slot_ids=slots.to(DEV),
+                     quantized=quantized)
+    if quantized:
+        codes, scales = out
+        result = (codes.float() * scales[:, None]).view(rows, heads * groups, dim).cpu()
+    else:
+        result = out[:, 0].float().cpu()
+    checked = 0
+    for row in range(rows):
+        slot = int(slots[row])
+        if not active[row] or slot < 0:
+            assert torch.count_nonzero(result[row]) == 0
+            continue
+        expected = O.k_attend(q[row, 0], hist[0][slot], hist[1][slot], int(lengths[slot]), dim ** -0.5, hist[2][slot], hist[3][slot])
+        tolerance = dict(atol=0.05, rtol=0.07) if quantized else dict(atol=0.012, rtol=0.025)   # e4m3 rows: 1/16 relative steps
+        torch.testing.assert_close(result[row], expected, **tolerance)
+        checked += 1
+    assert checked >= 24
+
+
+@pytest.mark.parametrize("batch", [6, 11])    # 48 and 88 (row, KV head) pairs: the item list, a workgroup per pair
+@pytest.mark.parametrize("fp8", [True, False])
+@torch.inference_mode()
+def test_paged_slot_mapped_history_equals_dense_history(ops, fp8, batch):
     """Block-16 paged layout: the same tokens reached through a shuffled block table give the same output."""
     torch.manual_seed(4)
-    batch, heads, groups, dim, page = 6, 8, 4, 64, 16
-    lengths = torch.tensor([1, 16, 17, 300, 1000, 777])
+    heads, groups, dim, page = 8, 4, 64, 16
+    lengths = torch.tensor([1, 16, 17, 300, 1000, 777, 64, 65, 1008, 513, 48][:batch])
     cap = 1008
     k = torch.randn(batch, cap, heads, dim).bfloat16()
     v = torch.randn_like(k)
