@@ -700,7 +700,7 @@ struct Plan { int tile, splits; };
 // once it alone fills the 256 CUs (1.3-2.0 PFLOP/s at M = 4096; 42 us for the 65536-row head at M = 256), otherwise
 // smaller tiles with deeper rings the fewer workgroups a CU gets (its K loop is then a serial chain that nothing
 // overlaps).  With K bytes not a multiple of the step these indices run their register-staged twins.
-Plan default_plan(int64_t M, int64_t N, int64_t Kb) {
+Plan default_plan(int64_t M, int64_t N, int64_t Kb, bool deferred = false) {
   auto count = [&](int t) { return ((M + kTiles[t].bm - 1) / kTiles[t].bm) * ((N + kTiles[t].bn - 1) / kTiles[t].bn); };
   const int64_t steps = (Kb + kStepBytes - 1) / kStepBytes;
   // Few output tiles on a K loop of 32 steps or more: split K (2 or 4 ways) while every part keeps 8 steps and the
@@ -724,6 +724,11 @@ Plan default_plan(int64_t M, int64_t N, int64_t Kb) {
     const int splits = (int)(512 / count(13));
     return {13, splits > 4 ? 4 : splits};
   }
+  // A product whose partial sums the next norm adds up (the e4m3 down projection of a decode step: 44 steps on a
+  // 256 x 2048 output): 64x64 tiles on two halves of K, one workgroup per CU.  Alone 9.9 us against 13.1 for the
+  // unsplit 32x64 tiles; the norm then reads two fp32 partials instead of one 16-bit product, which leaves 6 us of
+  // the step's 1.48 ms (four-way splits on 64x128 tiles: 9.5 us alone, nothing left in the step).
+  if (deferred && M > 128 && M <= 256 && steps >= 32 && steps < 64 && count(16) <= 128) return {16, 2};
   // One tile per CU, as square as the output allows, with many waves: the K loop moves about 50 B/ns into a CU
   // whatever the ring depth or step size, so the bytes a CU pulls decide (tile rows + columns, times K).
   // 256 rows: N 11264 on 128x96 tiles of 16 waves 15.4 us against 19.4 on 64x64; N 6144 on 64x96 tiles of 8 waves
@@ -786,7 +791,7 @@ int gemm_entry(const char* name, void* out, const void* a, const float* as, cons
     hipLaunchKernelGGL(gemm_naive_kernel<EB>, dim3(ceil_div(M * N, 256)), dim3(256), 0, s, out, A, W, as, ws, M, N, K, out_dtype, rows);
     LFM2_LAUNCH_CHECK();
   }
-  Plan plan = default_plan(M, N, Kb);
+  Plan plan = default_plan(M, N, Kb, !reduce);
   if (tile >= 0) {
     LFM2_REQUIRE(tile < kNumTiles, "%s: tile index %d out of range", name, tile);
     plan.tile = tile;
@@ -997,7 +1002,7 @@ extern "C" int lfm2_fp8_gemm_partials(float* partials, const uint8_t* a_q, const
                                       int64_t K, int tile, int split_k, void* stream) {
   LFM2_REQUIRE(split_k >= 1 && split_k <= 16, "fp8_gemm_partials: split_k %d not in [1,16]", split_k);
   LFM2_REQUIRE(tile < kNumTiles, "fp8_gemm_partials: tile index %d out of range", tile);
-  const int64_t steps = tile_steps(tile >= 0 ? tile : default_plan(M, N, K).tile, K);
+  const int64_t steps = tile_steps(tile >= 0 ? tile : default_plan(M, N, K, true).tile, K);
   LFM2_REQUIRE(split_k <= steps && (steps + split_k - 1) / split_k * (split_k - 1) < steps,
                "fp8_gemm_partials: %d splits leave one without a K step", split_k);
   return gemm_entry<1>("fp8_gemm_partials", nullptr, a_q, nullptr, w_q, nullptr, partials, M, N, K, LFM2_DTYPE_F32, tile,
@@ -1005,7 +1010,7 @@ extern "C" int lfm2_fp8_gemm_partials(float* partials, const uint8_t* a_q, const
 }
 
 extern "C" int64_t lfm2_fp8_gemm_default_splits(int64_t M, int64_t N, int64_t K) {
-  return K % 16 == 0 ? default_plan(M, N, K).splits : 1;
+  return K % 16 == 0 ? default_plan(M, N, K, true).splits : 1;
 }
 
 extern "C" int64_t lfm2_fp8_gemm_workspace(int64_t M, int64_t N, int64_t K) {

@@ -136,7 +136,8 @@ int lfm2_fp8_gemm_qkv_store(void* q, const uint8_t* a_q, const float* a_scales, 
  * pass (lfm2_rms_norm_fp8_split).  No counterpart in the reference, which always materialises the projection. */
 int lfm2_fp8_gemm_partials(float* partials, const uint8_t* a_q, const uint8_t* w_q, int64_t M, int64_t N, int64_t K,
                            int tile, int split_k, void* stream);
-/* Split count lfm2_fp8_gemm would choose for a shape (1 = no split). */
+/* Split count to give lfm2_fp8_gemm_partials for a shape (the tile it then picks suits that count); 1 = leave the
+ * product whole with lfm2_fp8_gemm. */
 int64_t lfm2_fp8_gemm_default_splits(int64_t M, int64_t N, int64_t K);
 /* Workspace floats lfm2_fp8_gemm needs for a shape under its default choice (0 = none). */
 int64_t lfm2_fp8_gemm_workspace(int64_t M, int64_t N, int64_t K);

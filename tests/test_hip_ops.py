@@ -909,8 +909,18 @@ def test_split_k_partials_reduce_inside_the_following_norm(ops):
     assert torch.equal(got[0].view(torch.uint8), expected[0].view(torch.uint8))
     assert torch.equal(got[1], expected[1])
     assert torch.equal(got[2].view(torch.int16), expected[2].view(torch.int16))
-    unsplit = weight.linear_quantized(xq, xs, defer_reduce=True)
-    assert isinstance(unsplit, torch.Tensor)  # nothing to defer when the plan does not split
+    # the default plan for a deferred reduce at this shape: two halves of K; the same bytes after the norm as the split
+    # product materialised by the GEMM's own reduce launch
+    halves = weight.linear_quantized(xq, xs, defer_reduce=True)
+    assert isinstance(halves, ops.SplitProduct) and halves.partials.size(0) == 2
+    whole = weight.linear_quantized(xq, xs, config=(16, 2))
+    assert torch.equal(halves.materialize().view(torch.int16), whole.view(torch.int16))
+    expected, got = ops.rms_norm_fp8(whole, norm_w, 1e-5, residual), ops.rms_norm_fp8(halves, norm_w, 1e-5, residual)
+    assert all(torch.equal(a.view(torch.uint8), b.view(torch.uint8)) for a, b in zip(got, expected))
+    # nothing to defer when the plan does not split (a K loop of 16 steps)
+    narrow = ops.PackedFP8Weight.from_weight(torch.randn(outputs, 2048, dtype=torch.bfloat16, device=DEV) * 0.02)
+    aq, a_s = ops.quantize_rows(act[:, :2048].contiguous())
+    assert isinstance(narrow.linear_quantized(aq, a_s, defer_reduce=True), torch.Tensor)
 
 
 @torch.inference_mode()
