@@ -670,11 +670,15 @@ schedule_rows(int32_t* schedule, const int32_t* positions, const uint8_t* active
   __shared__ int class_base[kSchedClasses + 1];   // where each class starts; running, during the second sweep
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int pairs_at = kSchedRows + 4 * B;
-  auto row_length = [&](int b) {
+  auto read_length = [&](int b) {
     int len = 0;
     if (b < B && (!active || active[b]) && (!slot_ids || slot_ids[b] >= 0)) len = positions[b] + 1;
     return len > 0 ? len : 0;
   };
+  // every sweep below hands row base + threadIdx.x to this thread: the first 1024 rows (every decode batch) are read
+  // from memory once, not once per sweep (each read is a round trip the next phase would wait for)
+  const int first_length = read_length(threadIdx.x);
+  auto row_length = [&](int b) { return b == (int)threadIdx.x ? first_length : read_length(b); };
   // sweep 0: the chunk size, from the number of items the rows would make at the short one
   int short_items = 0;
   for (int base = 0; base < B; base += 1024) short_items += (row_length(base + threadIdx.x) + kMfmaChunk - 1) / kMfmaChunk;
@@ -770,7 +774,8 @@ schedule_rows(int32_t* schedule, const int32_t* positions, const uint8_t* active
 #pragma unroll
       for (int k = 1; k < kSchedClasses; ++k) if (n[k]) partial = first[k];
       int32_t* row = schedule + kSchedRows + 4 * b;
-      row[0] = first[0]; row[1] = partial; row[2] = len; row[3] = 0;
+      row[0] = first[0]; row[1] = partial; row[2] = len;
+      if (B > 1024) row[3] = 0;   // up to 1024 rows the word names the row of this rank (below)
       const int slot = slot_ids ? slot_ids[b] : b;
       for (int c = 0; c < full; ++c) {   // the record the attention kernel reads: row, chunk, length, slot
         int32_t* rec = schedule + pairs_at + 4 * (first[0] + c);
@@ -790,27 +795,25 @@ schedule_rows(int32_t* schedule, const int32_t* positions, const uint8_t* active
     __syncthreads();
   }
   // The rows by decreasing length, for the kernel that gives every (row, KV head) a workgroup of its own: the spare
-  // word of record r names the row of rank r (ties: the lower row first).  A bitonic sort of (length, row) keys in
-  // LDS, one key per thread: batches of up to 1024 rows; larger ones keep the item list.
+  // word of record r names the row of rank r (ties: the lower row first).  Keys (length, row) are distinct, so a row's
+  // rank is the number of larger keys: every thread counts them over the keys in LDS (four per read, the same
+  // address for all lanes) and writes its row at its rank.  Batches of up to 1024 rows; larger ones keep the item list.
   if (B <= 1024) {
-    __shared__ unsigned keys[1024];
-    int width = 64;
-    while (width < B) width <<= 1;
+    __shared__ __attribute__((aligned(16))) unsigned keys[1024];
     const int t = threadIdx.x;
-    if (t < width) keys[t] = t < B ? ((unsigned)row_length(t) << 10) | (unsigned)(1023 - t) : 0u;
+    const unsigned mine = t < B ? ((unsigned)first_length << 10) | (unsigned)(1023 - t) : 0u;
+    keys[t] = mine;
     __syncthreads();
-    for (int k = 2; k <= width; k <<= 1) {
-      for (int j = k >> 1; j > 0; j >>= 1) {
-        const int partner = t ^ j;
-        if (t < width && partner > t) {
-          const unsigned mine = keys[t], theirs = keys[partner];
-          const bool descending = (t & k) == 0;
-          if ((mine < theirs) == descending) { keys[t] = theirs; keys[partner] = mine; }
-        }
-        __syncthreads();
+    if (t < B) {
+      int rank = 0;
+      typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+      const u32x4* quad = reinterpret_cast<const u32x4*>(keys);
+      for (int i = 0; i < (B + 3) / 4; ++i) {
+        const u32x4 k = quad[i];
+        rank += (k[0] > mine) + (k[1] > mine) + (k[2] > mine) + (k[3] > mine);
       }
+      schedule[kSchedRows + 4 * rank + 3] = t;
     }
-    if (t < B) schedule[kSchedRows + 4 * t + 3] = 1023 - (int)(keys[t] & 1023u);
   }
 }
 
