@@ -584,8 +584,9 @@ class RowSampler:
     def __init__(self, logits):
         self.batch, self.vocab = logits.shape
         self.scratch = _sample_scratch(self.batch, self.vocab, logits.device)
-        self.tokens = torch.empty(self.batch, device=logits.device, dtype=torch.long)
-        self.logprobs = torch.empty(self.batch, device=logits.device, dtype=torch.float32)
+        # zeros, not empty: a caller that draws only some rows into these buffers still hands valid token ids on
+        self.tokens = torch.zeros(self.batch, device=logits.device, dtype=torch.long)
+        self.logprobs = torch.zeros(self.batch, device=logits.device, dtype=torch.float32)
 
     def sample(self, logits, seeds, steps, temperatures):
         call("lfm2_sample", self.tokens, self.logprobs, logits, self.scratch, seeds, steps, temperatures, 0, 0, 1.0,

@@ -490,9 +490,12 @@ class LFM25GenerationSession:
                     carried=carried or None)
 
     # ------------------------------------------------------------------ the hot loop
-    def _draw(self):
+    def _draw(self, every_row_filtered=False):
         state = self.rows
-        tokens, logprobs = self.sampler.sample(self.entry.logits, state.seeds, state.rng_positions, state.temperatures)
+        if every_row_filtered:    # no running row keeps the full-support draw: its two launches are left out
+            tokens, logprobs = self.sampler.tokens, self.sampler.logprobs
+        else:
+            tokens, logprobs = self.sampler.sample(self.entry.logits, state.seeds, state.rng_positions, state.temperatures)
         if self._filtered_rows:   # rows with top-k / top-p are redrawn with their own parameters; the others are skipped
             ops.sample_filtered(self.entry.logits, seeds=state.seeds, steps=state.rng_positions, temperatures=state.temperatures,
                                 top_ks=state.top_ks, top_ps=state.top_ps, out=(tokens, logprobs))
@@ -511,13 +514,14 @@ class LFM25GenerationSession:
         graph, width = self._graph_for(running)
         state, config = self.rows, self.engine.config
         fused_record = not self._filtered_rows and not self.behavior_topk
+        every_row_filtered = self._filtered_rows.issuperset(running)
         for _ in range(steps):
             graph.replay()       # consumes the owed token of every row whose pending flag is set
             if fused_record:     # no redraw and no behaviour head between the draw and its record: one launch less
                 ops.sample_and_record(self.sampler, self.entry.logits, state, self.entry.input_tokens, self.stops.flat,
                                       config.eos_token_id, self.max_new_tokens)
                 continue
-            tokens, logprobs = self._draw()
+            tokens, logprobs = self._draw(every_row_filtered)
             if self.behavior_topk:
                 ids, values = ops.behavior_topk(self.entry.logits, tokens, logprobs, self.behavior_topk)
                 ops.record_head(ids, values, state.head_ids, state.head_logprobs, state.lengths, state.alive,
