@@ -1121,13 +1121,17 @@ prefill_attn_kernel(T* __restrict__ out, const T* __restrict__ q, const T* __res
     rs = add_lane_xor32(add_lane_xor16(rs));
     l = fmaf(l, alpha, rs);
     m = mnew;
-    const bool rescale = __any(alpha != 1.0f);   // the running maximum rarely moves after the first tiles
+    // the running maximum rarely moves after the first tiles: a branch the whole wave takes or skips (the empty asm
+    // keeps it a branch; as selects it costs twice the multiplies it saves)
+    if (__any(alpha != 1.0f)) {
+      asm volatile("" ::: "memory");
 #pragma unroll
-    for (int dd = 0; dd < D / 16; ++dd) {
-      if (rescale) {
+      for (int dd = 0; dd < D / 16; ++dd)
 #pragma unroll
         for (int i = 0; i < 4; ++i) o[dd][i] *= alpha;
-      }
+    }
+#pragma unroll
+    for (int dd = 0; dd < D / 16; ++dd) {
 #pragma unroll
       for (int kk2 = 0; kk2 < 2; ++kk2) {
         // tokens 32 kk2 + 4 grp + 0..3 and the same + 16 of dim 16 dd + r: the order P holds them in
