@@ -446,22 +446,22 @@ def test_decode_over_more_rows_than_one_scan_block(ops, quantized, fp8):
     assert torch.count_nonzero(result[~active]) == 0
 
 
-@pytest.mark.parametrize("groups", [1, 2, 4])
+@pytest.mark.parametrize("groups,rows,capacity", [(1, 37, 700), (2, 37, 700), (4, 37, 700), (4, 1001, 300)])
 @pytest.mark.parametrize("quantized", [False, True])
 @pytest.mark.parametrize("fp8", [True, False])
 @torch.inference_mode()
-def test_decode_with_a_workgroup_per_row_and_kv_head_matches_the_oracle(ops, groups, quantized, fp8):
+def test_decode_with_a_workgroup_per_row_and_kv_head_matches_the_oracle(ops, groups, rows, capacity, quantized, fp8):
     """37 rows of 8 KV heads: from 64 (row, KV head) pairs on, a workgroup's four waves share one pair's tiles and merge
     through LDS.  Lengths sit on both sides of the 32- and 64-token tile and of the four-tile round; a row count that is
     no multiple of 8 leaves empty places in the last round of the XCD mapping; inactive rows and padding slots give
-    zeros; every live row is checked against the oracle."""
+    zeros; every live row is checked against the oracle (of 1001 rows, near the 1024 the rows are ranked for, a sample)."""
     torch.manual_seed(41)
-    rows, capacity, heads, dim = 37, 700, 8, 64
+    heads, dim = 8, 64
     k = torch.randn(rows, capacity, heads, dim).bfloat16()
     v = torch.randn_like(k)
     q = torch.randn(rows, 1, heads * groups, dim).bfloat16()
     lengths = torch.randint(1, capacity + 1, (rows,))
-    fixed = [1, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 511, 512, 513, 700]
+    fixed = [n for n in (1, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 511, 512, 513, 700) if n <= capacity]
     lengths[:len(fixed)] = torch.tensor(fixed)
     active = torch.rand(rows) > 0.15
     slots = torch.randperm(rows).to(torch.int32)
@@ -484,10 +484,11 @@ def test_decode_with_a_workgroup_per_row_and_kv_head_matches_the_oracle(ops, gro
     else:
         result = out[:, 0].float().cpu()
     checked = 0
-    for row in range(rows):
+    dead = ~active | (slots < 0)
+    assert torch.count_nonzero(result[dead]) == 0
+    for row in (range(rows) if rows < 100 else [*range(0, rows, 17), rows - 2, rows - 1]):
         slot = int(slots[row])
-        if not active[row] or slot < 0:
-            assert torch.count_nonzero(result[row]) == 0
+        if dead[row]:
             continue
         expected = O.k_attend(q[row, 0], hist[0][slot], hist[1][slot], int(lengths[slot]), dim ** -0.5, hist[2][slot], hist[3][slot])
         tolerance = dict(atol=0.05, rtol=0.07) if quantized else dict(atol=0.012, rtol=0.025)   # e4m3 rows: 1/16 relative steps
