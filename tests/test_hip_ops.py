@@ -481,6 +481,15 @@ def test_decode_with_a_workgroup_per_row_and_kv_head_matches_the_oracle(ops, gro
     if quantized:
         codes, scales = out
         result = (codes.float() * scales[:, None]).view(rows, heads * groups, dim).cpu()
+        # the bits of the row quantiser on the plain result, also through a schedule shared by two calls
+        plain = ops.attend(q.to(DEV), kc, vc, ks, vs, positions.to(DEV), active=active.to(DEV), slot_ids=slots.to(DEV))
+        want_codes, want_scales = ops.quantize_rows(plain.view(rows, -1))
+        shared = ops.decode_schedule(positions.to(DEV), active.to(DEV), slots.to(DEV), capacity=capacity)
+        again = [ops.attend(q.to(DEV), kc, vc, ks, vs, positions.to(DEV), active=active.to(DEV), slot_ids=slots.to(DEV),
+                            quantized=True, schedule=shared) for _ in range(2)]
+        for got_codes, got_scales in (out, *again):
+            assert torch.equal(got_codes.view(torch.uint8), want_codes.view(torch.uint8))
+            assert torch.equal(got_scales, want_scales)
     else:
         result = out[:, 0].float().cpu()
     checked = 0
