@@ -721,6 +721,9 @@ Plan default_plan(int64_t M, int64_t N, int64_t Kb, bool deferred = false) {
     // a long K loop on few output tiles (the bf16 down projection at decode: 88 steps on 128 tiles): split K so that
     // about 512 workgroups share it.  M 256, N 2048, 11264 K bytes: 16.5 us against 24.3 (bf16), 21.1 against 22.4
     // (e4m3); M 128: 13.0 against 24.5
+    // where 64x128 tiles of 8 waves on four parts of K make one workgroup per CU they pull fewer bytes into it: the
+    // same shape 14.9 us alone against 17.5, the all-bf16 decode step 2.036 against 2.070 ms
+    if (count(29) * 4 > 128 && count(29) * 4 <= 256) return {29, 4};
     const int splits = (int)(512 / count(13));
     return {13, splits > 4 ? 4 : splits};
   }
