@@ -1051,7 +1051,7 @@ extern "C" int lfm2_bf16_gemm_partials(float* partials, const void* x, const voi
                                        int tile, int split_k, void* stream) {
   LFM2_REQUIRE(split_k >= 1 && split_k <= 16, "bf16_gemm_partials: split_k %d not in [1,16]", split_k);
   LFM2_REQUIRE(tile < kNumTiles, "bf16_gemm_partials: tile index %d out of range", tile);
-  const int64_t steps = tile_steps(tile >= 0 ? tile : default_plan(M, N, K * 2).tile, K * 2);
+  const int64_t steps = tile_steps(tile >= 0 ? tile : default_plan(M, N, K * 2, true).tile, K * 2);
   LFM2_REQUIRE(split_k <= steps && (steps + split_k - 1) / split_k * (split_k - 1) < steps,
                "bf16_gemm_partials: %d splits leave one without a K step", split_k);
   return gemm_entry<2>("bf16_gemm_partials", nullptr, x, nullptr, w, nullptr, partials, M, N, K, LFM2_DTYPE_F32, tile, split_k,
@@ -1059,7 +1059,7 @@ extern "C" int lfm2_bf16_gemm_partials(float* partials, const void* x, const voi
 }
 
 extern "C" int64_t lfm2_bf16_gemm_default_splits(int64_t M, int64_t N, int64_t K) {
-  return (K * 2) % 16 == 0 ? default_plan(M, N, K * 2).splits : 1;
+  return (K * 2) % 16 == 0 ? default_plan(M, N, K * 2, true).splits : 1;
 }
 
 extern "C" int64_t lfm2_bf16_gemm_workspace(int64_t M, int64_t N, int64_t K) {

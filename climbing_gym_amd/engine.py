@@ -260,12 +260,13 @@ class LFM25Engine:
         normed, residual = self._normed(x, norm_weight, residual, weight, fp8)
         return self._project(normed, weight, fp8, place), residual
 
-    def _linear(self, x, weight, fp8):
-        """Out projection of an operator; `x` is a tensor or, from a fused producer, (e4m3 rows, scales)."""
+    def _linear(self, x, weight, fp8, defer_reduce=False):
+        """Out projection of an operator; `x` is a tensor or, from a fused producer, (e4m3 rows, scales).  With
+        `defer_reduce` a bf16 product that the plan splits along K is left to the norm that follows."""
         packed = fp8.get(id(weight))
         if isinstance(x, tuple):
             return packed.linear_quantized(x[0], x[1], dtype=self.dtype)
-        return packed.linear(x) if packed is not None else ops.linear(x, weight)
+        return packed.linear(x) if packed is not None else ops.linear(x, weight, defer_reduce=defer_reduce)
 
     def _backbone(self, tokens, attention_op, conv_op, fp8, *, defer_reduce=False, projecting_attention_op=None,
                   projecting_conv_op=None):
@@ -294,13 +295,13 @@ class LFM25Engine:
                     attended = projecting_attention_op(op, packed, normed[0], normed[1])
                 if attended is None:   # no fused projection for this shape: the plain one, then the head preparation
                     attended = attention_op(op, self._project(normed, op.qkv_weight, fp8))
-                mixed = self._linear(attended, op.out_weight, fp8)
+                mixed = self._linear(attended, op.out_weight, fp8, defer_reduce)
             else:
                 op = layer.conv
                 gated = projecting_conv_op(op, normed) if projecting_conv_op is not None else None
                 if gated is None:   # no fused projection for this shape: the plain one, then the conv launch
                     gated = conv_op(op, self._project(normed, op.in_weight, fp8))
-                mixed = self._linear(gated, op.out_weight, fp8)
+                mixed = self._linear(gated, op.out_weight, fp8, defer_reduce)
             # gate+up projection and SwiGLU: one launch where the product's shape has the fused form (packed prefill
             # chunks), the projection and the SwiGLU launch otherwise (decode); the same bits either way
             normed, residual = self._normed(mixed, layer.ffn_norm_weight, residual, layer.w13_weight, fp8)

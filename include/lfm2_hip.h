@@ -148,7 +148,7 @@ int lfm2_bf16_gemm(void* out, const void* x, const void* w, float* workspace, in
                    int tile, int split_k, void* stream);
 int64_t lfm2_bf16_gemm_workspace(int64_t M, int64_t N, int64_t K);
 /* The bf16 product left as split-K partial sums, float[split_k, M, N] (see lfm2_fp8_gemm_partials), and the split
- * count lfm2_bf16_gemm would choose for a shape.  No counterpart in the reference. */
+ * count to give lfm2_bf16_gemm_partials for a shape (1 = leave the product whole).  No counterpart in the reference. */
 int lfm2_bf16_gemm_partials(float* partials, const void* x, const void* w, int64_t M, int64_t N, int64_t K, int tile,
                             int split_k, void* stream);
 int64_t lfm2_bf16_gemm_default_splits(int64_t M, int64_t N, int64_t K);

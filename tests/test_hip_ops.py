@@ -953,7 +953,18 @@ def test_bf16_split_k_partials_reduce_inside_the_following_norm(ops):
     assert torch.equal(got[1].view(torch.int16), expected[1].view(torch.int16))
     expected, got = ops.rms_norm_fp8(whole, norm_w, 1e-5, residual), ops.rms_norm_fp8(deferred, norm_w, 1e-5, residual)
     assert torch.equal(got[0].view(torch.uint8), expected[0].view(torch.uint8)) and torch.equal(got[1], expected[1])
-    assert isinstance(ops.linear(act[:, :2048].contiguous(), weight[:, :2048].contiguous(), defer_reduce=True), torch.Tensor)
+    # the out projection's shape (32 K steps): two halves of K when the reduce is left to the norm, the same bytes
+    # after it as the split product summed by the GEMM's own reduce launch
+    act2, weight2 = act[:, :2048].contiguous(), weight[:, :2048].contiguous()
+    halves = ops.linear(act2, weight2, defer_reduce=True)
+    assert isinstance(halves, ops.SplitProduct) and halves.partials.size(0) == 2
+    whole = ops.linear(act2, weight2, tile=16, split_k=2)
+    assert torch.equal(halves.materialize().view(torch.int16), whole.view(torch.int16))
+    expected, got = ops.rms_norm(whole, norm_w, 1e-5, residual), ops.rms_norm(halves, norm_w, 1e-5, residual)
+    assert torch.equal(got[0].view(torch.int16), expected[0].view(torch.int16))
+    assert torch.equal(got[1].view(torch.int16), expected[1].view(torch.int16))
+    # nothing to defer when the plan does not split (16 K steps)
+    assert isinstance(ops.linear(act[:, :1024].contiguous(), weight[:, :1024].contiguous(), defer_reduce=True), torch.Tensor)
 
 
 # ------------------------------------------------------------------------------------------------ rounding points
