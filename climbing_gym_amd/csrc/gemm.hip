@@ -740,7 +740,11 @@ Plan default_plan(int64_t M, int64_t N, int64_t Kb, bool deferred = false) {
     if (N % 96 == 0 && count(37) <= 256 && count(37) > 128) return {37, 1};
     if (N >= 8192 && count(36) <= 256) return {36, 1};
   }
-  if (M > 256 && M <= 512 && steps <= 32 && N % 96 == 0 && count(31) <= 256 && count(31) > 128) return {31, 1};
+  // 257-512 rows: the same 128x96 tile of 16 waves (N 6144: 13.6 us against 15.0 with 8 waves), and for the widest
+  // outputs 256x128 tiles of 16 waves, which halve the weight bytes a CU pulls (N 11264: 23.2 us against 26.2 on
+  // 128x128 tiles)
+  if (M > 256 && M <= 512 && steps <= 32 && N % 96 == 0 && count(36) <= 256 && count(36) > 128) return {36, 1};
+  if (M > 256 && M <= 512 && steps <= 32 && N >= 8192 && count(56) <= 256) return {56, 1};
   // The vocabulary projection at a decode batch (N 65536): one 256x256 tile per CU instead of four 128x128 tiles
   // halves the activation bytes a CU pulls (M 256: 48.8 us against 60.0; M 512: 79.4 against 103.9; up to 128 rows the
   // 128x128 tile stays ahead, 37.6 against 43.9).
@@ -749,7 +753,7 @@ Plan default_plan(int64_t M, int64_t N, int64_t Kb, bool deferred = false) {
   if (count(2) >= 512) return {13, 1};                // 64x64, ring of 3
   // one round of 64x64 tiles over the 256 CUs beats two rounds of 32x64 (512 rows, N 2048: K 5632 16.8 us against
   // 21.0, K 2048 8.9 against 9.9)
-  if (count(1) > 384 && count(2) <= 256) return {16, 1};
+  if (count(1) > 384 && count(2) <= 256) return {38, 1};   // sixteen waves (512 rows, N 2048: 8.1 us against 8.9 with four)
   if (count(1) > 384) return {15, 1};                 // 32x64, 256-byte steps, ring of 2
   if (count(1) > 256) return {16, 1};                 // 64x64, ring of 4
   return {steps >= 32 ? 17 : 12, splits_for(count(1))};   // 32x64, ring of 5 (long K) or 4
@@ -894,7 +898,7 @@ namespace {
 bool swiglu_fits(int64_t M, int64_t N, int64_t Kb) {
   if (M <= 0 || N <= 0 || Kb <= 0 || N % 16 != 0 || Kb % kStepBytes != 0 || M >= (1 << 30) || N >= (1 << 30)) return false;
   const Plan plan = default_plan(M, N, Kb);
-  return (plan.tile == 14 || plan.tile == 36) && plan.splits == 1;
+  return (plan.tile == 14 || plan.tile == 36 || plan.tile == 56) && plan.splits == 1;
 }
 template <int EB>
 int swiglu_entry(const char* name, void* out, const void* a, const float* as, const void* w, const float* ws, int64_t M,
@@ -908,6 +912,9 @@ int swiglu_entry(const char* name, void* out, const void* a, const float* as, co
   const dim3 grid((tiles + 7) / 8 * 8);
   if (tile == 14)
     hipLaunchKernelGGL((gemm_swiglu_kernel<EB, 128, 128, 2, 4, 2>), grid, dim3(512), 0, (hipStream_t)stream, out,
+                       (const uint8_t*)a, (const uint8_t*)w, as, ws, (int)M, (int)N, K * EB, out_dtype);
+  else if (tile == 56)
+    hipLaunchKernelGGL((gemm_swiglu_kernel<EB, 256, 128, 4, 4, 3>), grid, dim3(1024), 0, (hipStream_t)stream, out,
                        (const uint8_t*)a, (const uint8_t*)w, as, ws, (int)M, (int)N, K * EB, out_dtype);
   else
     hipLaunchKernelGGL((gemm_swiglu_kernel<EB, 128, 96, 8, 2, 3>), grid, dim3(1024), 0, (hipStream_t)stream, out,
