@@ -736,6 +736,10 @@ Plan default_plan(int64_t M, int64_t N, int64_t Kb, bool deferred = false) {
   // whatever the ring depth or step size, so the bytes a CU pulls decide (tile rows + columns, times K).
   // 256 rows: N 11264 on 128x96 tiles of 16 waves 15.4 us against 19.4 on 64x64; N 6144 on 64x96 tiles of 8 waves
   // 10.9 against 13.1; 512 rows, N 6144 on 128x96 tiles of 8 waves 15.2 against 17.7.
+  // 65-128 rows of a wide output: 64x96 tiles of 8 waves, one per CU (N 11264: 11.0 us against 14.7 and more on 32x64 tiles)
+  if (M > 64 && M <= 128 && steps <= 32 && N >= 8192 && count(37) <= 256 && count(37) > 128) return {37, 1};
+  // and of a narrow one: 16x64 tiles with 256-byte steps, one per CU (128 rows, N 2048, K 2048: 4.9 us against 6.0)
+  if (M > 64 && M <= 128 && steps <= 16 && count(18) <= 256 && count(18) > 128) return {18, 1};
   if (M > 128 && M <= 256 && steps <= 32) {
     if (N % 96 == 0 && count(37) <= 256 && count(37) > 128) return {37, 1};
     if (N >= 8192 && count(36) <= 256) return {36, 1};
@@ -755,7 +759,7 @@ Plan default_plan(int64_t M, int64_t N, int64_t Kb, bool deferred = false) {
   // 21.0, K 2048 8.9 against 9.9)
   if (count(1) > 384 && count(2) <= 256) return {38, 1};   // sixteen waves (512 rows, N 2048: 8.1 us against 8.9 with four)
   if (count(1) > 384) return {15, 1};                 // 32x64, 256-byte steps, ring of 2
-  if (count(1) > 256) return {16, 1};                 // 64x64, ring of 4
+  if (count(1) > 256) return {38, 1};                 // 64x64, ring of 4, sixteen waves (128 rows, N 6144: 8.5 us against 9.2 with four)
   return {steps >= 32 ? 17 : 12, splits_for(count(1))};   // 32x64, ring of 5 (long K) or 4
 }
 
