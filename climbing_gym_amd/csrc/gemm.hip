@@ -714,6 +714,12 @@ Plan default_plan(int64_t M, int64_t N, int64_t Kb, bool deferred = false) {
   };
   // up to 64 rows the direct-to-LDS rings win over register staging by 25-40 % once the weights come from HBM
   // (e4m3 N 3072: 6.2 / 7.2 / 7.1 us at 16 / 32 / 64 rows against 9.2 / 10.9 / 12.9)
+  // A short K loop on few tiles whose partial sums the next norm adds up anyway (the out projection of a small decode
+  // batch): four parts of K (16 rows, N 2048, K 2048: 3.3 us against 4.8 whole; the reduce launch would cost more)
+  if (deferred && M <= 64 && steps >= 16 && steps < 32) {
+    const int t = M <= 16 ? 18 : 17;
+    if (count(t) * 4 <= 256) return {t, 4};
+  }
   if (M <= 16) return {18, splits_for(count(18))};            // 16x64, 256-byte steps, ring of 3
   if (M <= 32) return {17, splits_for(count(17))};            // 32x64, ring of 5
   if (M <= 64 && count(1) <= 256) return {17, splits_for(count(17))};

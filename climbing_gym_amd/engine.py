@@ -262,10 +262,10 @@ class LFM25Engine:
 
     def _linear(self, x, weight, fp8, defer_reduce=False):
         """Out projection of an operator; `x` is a tensor or, from a fused producer, (e4m3 rows, scales).  With
-        `defer_reduce` a bf16 product that the plan splits along K is left to the norm that follows."""
+        `defer_reduce` a product that the plan splits along K is left to the norm that follows."""
         packed = fp8.get(id(weight))
         if isinstance(x, tuple):
-            return packed.linear_quantized(x[0], x[1], dtype=self.dtype)
+            return packed.linear_quantized(x[0], x[1], dtype=self.dtype, defer_reduce=defer_reduce)
         return packed.linear(x) if packed is not None else ops.linear(x, weight, defer_reduce=defer_reduce)
 
     def _backbone(self, tokens, attention_op, conv_op, fp8, *, defer_reduce=False, projecting_attention_op=None,
