@@ -766,7 +766,9 @@ Plan default_plan(int64_t M, int64_t N, int64_t Kb, bool deferred = false) {
   if (count(1) > 384 && count(2) <= 256) return {38, 1};   // sixteen waves (512 rows, N 2048: 8.1 us against 8.9 with four)
   if (count(1) > 384) return {15, 1};                 // 32x64, 256-byte steps, ring of 2
   if (count(1) > 256) return {38, 1};                 // 64x64, ring of 4, sixteen waves (128 rows, N 6144: 8.5 us against 9.2 with four)
-  return {steps >= 32 ? 17 : 12, splits_for(count(1))};   // 32x64, ring of 5 (long K) or 4
+  // 32x64, ring of 5 (a long K loop; above 128 rows a short one as well: the out projection of the 256-row decode step
+  // gains 5-11 us per step over the ring of 4, which is level with it alone) or 4
+  return {steps >= 32 || M > 128 ? 17 : 12, splits_for(count(1))};
 }
 
 template <int EB, int BM, int BN, int WM, int WN, int SW, int KS, int ST = 0>
