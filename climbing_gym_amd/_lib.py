@@ -54,9 +54,9 @@ _SIGNATURES = {
     "lfm2_gather_inputs": "ppppppp" "lp",
     "lfm2_scatter_logits": "pppp" "llip",
     "lfm2_advance_positions": "pppp" "lp",
-    "lfm2_sample": "ppppppp" "llfllip",
+    "lfm2_sample": "pppppppp" "llfllip",
     "lfm2_sample_static": "pppppp" "llfllip",
-    "lfm2_sample_filtered": "ppppppppp" "llfifllip",
+    "lfm2_sample_filtered": "pppppppppp" "llfifllip",
     "lfm2_configure_rows": "p" "ll" "ppppppppppppp" "p",
     "lfm2_head_logprobs": "ppppp" "lliip",
     "lfm2_record_sample": "ppppppppppppppp" "llllp",

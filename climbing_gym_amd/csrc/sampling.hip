@@ -159,13 +159,13 @@ __device__ __forceinline__ void record_row(const RecordArgs& r, int64_t row, int
 // the target past the end).  At most 256 tiles (a vocabulary of 2^20).
 template <typename T>
 __global__ void __launch_bounds__(256)
-sample_finish_kernel(const T* logits, const float* scratch, int64_t* tokens, float* logprobs, const int64_t* seeds,
-                     const int64_t* steps, const float* temperatures, int64_t seed, int64_t step, float temperature,
-                     int64_t V, int parts, RecordArgs record) {
+sample_finish_kernel(const T* logits, const float* scratch, int64_t* tokens, float* logprobs, float* sampling_logprobs,
+                     const int64_t* seeds, const int64_t* steps, const float* temperatures, int64_t seed, int64_t step,
+                     float temperature, int64_t V, int parts, RecordArgs record) {
   __shared__ TileStat s_stat[4];
   __shared__ float s_tile_mass[256];
   __shared__ float s_wave[4];
-  __shared__ float s_target;
+  __shared__ float s_target, s_log_mass;
   __shared__ double s_uniform;
   __shared__ int s_tile, s_pick;
   const int64_t row = blockIdx.x;
@@ -214,6 +214,7 @@ sample_finish_kernel(const T* logits, const float* scratch, int64_t* tokens, flo
         before += m;
       }
       inside = (float)(target - before);
+      s_log_mass = (float)log(z);   // log sum exp((x - max) / T): the normaliser of the distribution the draw is from
     } else {
       while (tile < parts - 1 && s_tile_mass[tile] == 0.f) ++tile;   // first tile that holds the maximum
     }
@@ -281,6 +282,9 @@ sample_finish_kernel(const T* logits, const float* scratch, int64_t* tokens, flo
     for (int i = 1; i < 16; ++i) chosen = token - col0 == i ? x[i] : chosen;
     const float logp = chosen - (mx + logf(total));
     if (logprobs) logprobs[row] = logp;
+    // log-probability under softmax(logits / T), the distribution sampled from (lfm25_engine.py:1605-1608); greedy
+    // rows report the raw one (lfm25_engine.py:1591-1596)
+    if (sampling_logprobs) sampling_logprobs[row] = temp > 0.f ? (chosen - mx) * inv_temp - s_log_mass : logp;
     if (record.tokens) record_row(record, row, token, logp);
   }
 }
@@ -299,7 +303,7 @@ constexpr int kFT = 1024;  // threads of the filtered sampler
 // registers; the register form below makes the same decisions.
 template <typename T>
 __global__ void __launch_bounds__(kFT)
-sample_filtered_stream_kernel(const T* logits, int64_t* tokens, float* logprobs, int32_t* kept_count, const int64_t* seeds,
+sample_filtered_stream_kernel(const T* logits, int64_t* tokens, float* logprobs, float* sampling_logprobs, int32_t* kept_count, const int64_t* seeds,
                        const int64_t* steps, const float* temperatures, const int32_t* top_ks, const float* top_ps, int64_t seed,
                        int64_t step, float temperature, int top_k, float top_p, int64_t V) {
   if (temperatures) {   // per-row parameters: rows that ask for no filter (or are greedy) keep what the outputs hold
@@ -310,7 +314,7 @@ sample_filtered_stream_kernel(const T* logits, int64_t* tokens, float* logprobs,
   }
   __shared__ uint32_t h_cnt[256];
   __shared__ unsigned long long h_mass[256];
-  __shared__ float s_f[kFT / 64];
+  __shared__ float s_f[kFT / 64], s_kept[kFT / 64];
   __shared__ int s_i[kFT / 64];
   __shared__ uint32_t s_digit, s_remaining, s_cnt_above;
   __shared__ unsigned long long s_mass_above, s_total;
@@ -467,12 +471,13 @@ sample_filtered_stream_kernel(const T* logits, int64_t* tokens, float* logprobs,
   }
 
   // ---- Gumbel-max over the survivors
-  float best = -INFINITY;
+  float best = -INFINITY, kept_mass = 0.f;
   int best_i = 0x7fffffff;
   for (int64_t i = tid; i < V; i += kFT) {
     const float x = scaled(i);
     const uint32_t k = order_key(x);
     if (!(k > kp || (k == kp && i <= cut))) continue;
+    kept_mass += exp2f((x - xmax) * LFM2_LOG2E);
     uint32_t rnd[4];
     // per-row streams depend on the row's own (seed, step) only; a shared seed also counts the row
     philox((uint32_t)(i >> 2), seeds ? 0u : (uint32_t)row, 0x5eed5eedu, seeds ? 0u : (uint32_t)((uint64_t)row >> 32),
@@ -487,7 +492,8 @@ sample_filtered_stream_kernel(const T* logits, int64_t* tokens, float* logprobs,
     if (oi != 0x7fffffff && (best_i == 0x7fffffff || ob > best || (ob == best && oi < best_i))) { best = ob; best_i = oi; }
   }
   __syncthreads();
-  if (lane == 0) { s_f[wave] = best; s_i[wave] = best_i; }
+  kept_mass = wave_sum(kept_mass);
+  if (lane == 0) { s_f[wave] = best; s_i[wave] = best_i; s_kept[wave] = kept_mass; }
   __syncthreads();
   if (tid == 0) {
     float b = s_f[0];
@@ -497,6 +503,11 @@ sample_filtered_stream_kernel(const T* logits, int64_t* tokens, float* logprobs,
     if (bi == 0x7fffffff) bi = 0;
     tokens[row] = bi;
     if (logprobs) logprobs[row] = Elem<T>::load(src[bi]) - (mx + logf(raw_sum));
+    if (sampling_logprobs) {   // under the tempered, filtered distribution (lfm25_engine.py:1605-1608)
+      float kept = 0.f;
+      for (int w = 0; w < kFT / 64; ++w) kept += s_kept[w];
+      sampling_logprobs[row] = (scaled(bi) - xmax) - logf(kept);
+    }
   }
 }
 
@@ -519,7 +530,7 @@ struct Crossed { int bin; uint32_t count_above, count_at; unsigned long long mas
 
 template <typename T>
 __global__ void __launch_bounds__(kFT)
-sample_filtered_kernel(const T* logits, int64_t* tokens, float* logprobs, int32_t* kept_count, const int64_t* seeds,
+sample_filtered_kernel(const T* logits, int64_t* tokens, float* logprobs, float* sampling_logprobs, int32_t* kept_count, const int64_t* seeds,
                        const int64_t* steps, const float* temperatures, const int32_t* top_ks, const float* top_ps, int64_t seed,
                        int64_t step, float temperature, int top_k, float top_p, int64_t V) {
   if (temperatures) {   // per-row parameters: rows that ask for no filter (or are greedy) keep what the outputs hold
@@ -533,7 +544,7 @@ sample_filtered_kernel(const T* logits, int64_t* tokens, float* logprobs, int32_
   __shared__ unsigned long long h_mass[kBins];
   __shared__ uint32_t w_cnt[WAVES];
   __shared__ unsigned long long w_mass[WAVES];
-  __shared__ float s_f[WAVES];
+  __shared__ float s_f[WAVES], s_kept[WAVES];
   __shared__ int s_i[WAVES];
   __shared__ int s_best;
   __shared__ Crossed s_crossed;
@@ -790,9 +801,10 @@ sample_filtered_kernel(const T* logits, int64_t* tokens, float* logprobs, int32_
   }
 
   // ---- Gumbel-max over the survivors
-  float best = -INFINITY;
+  float best = -INFINITY, kept_mass = 0.f;
   int best_i = kNoIndex;
   auto consider = [&](float x, int i) {
+    kept_mass += exp2f((x - xmax) * LFM2_LOG2E);
     uint32_t rnd[4];
     // per-row streams depend on the row's own (seed, step) only; a shared seed also counts the row
     philox((uint32_t)(i >> 2), seeds ? 0u : (uint32_t)row, 0x5eed5eedu, seeds ? 0u : (uint32_t)((uint64_t)row >> 32),
@@ -829,7 +841,8 @@ sample_filtered_kernel(const T* logits, int64_t* tokens, float* logprobs, int32_
     if (oi != kNoIndex && (best_i == kNoIndex || ob > best || (ob == best && oi < best_i))) { best = ob; best_i = oi; }
   }
   __syncthreads();
-  if (lane == 0) { s_f[wave] = best; s_i[wave] = best_i; }
+  kept_mass = wave_sum(kept_mass);
+  if (lane == 0) { s_f[wave] = best; s_i[wave] = best_i; s_kept[wave] = kept_mass; }
   __syncthreads();
   if (tid == 0) {
     float b = s_f[0];
@@ -838,7 +851,13 @@ sample_filtered_kernel(const T* logits, int64_t* tokens, float* logprobs, int32_
       if (s_i[w] != kNoIndex && (bi == kNoIndex || s_f[w] > b || (s_f[w] == b && s_i[w] < bi))) { b = s_f[w]; bi = s_i[w]; }
     if (bi == kNoIndex) bi = 0;
     tokens[row] = bi;
-    if (logprobs) logprobs[row] = Elem<T>::load(src[bi]) - (mx + logf(raw_sum));
+    const float chosen = Elem<T>::load(src[bi]);
+    if (logprobs) logprobs[row] = chosen - (mx + logf(raw_sum));
+    if (sampling_logprobs) {   // under the tempered, filtered distribution (lfm25_engine.py:1605-1608)
+      float kept = 0.f;
+      for (int w = 0; w < WAVES; ++w) kept += s_kept[w];
+      sampling_logprobs[row] = (chosen / temperature - xmax) - logf(kept);
+    }
   }
 }
 
@@ -954,9 +973,9 @@ __global__ void advance_positions_kernel(int32_t* lengths, const int32_t* positi
 
 }  // namespace
 
-extern "C" int lfm2_sample(int64_t* tokens, float* logprobs, const void* logits, float* scratch, const int64_t* seeds,
-                           const int64_t* steps, const float* temperatures, int64_t seed, int64_t step, float temperature,
-                           int64_t B, int64_t V, int dtype, void* stream) {
+extern "C" int lfm2_sample(int64_t* tokens, float* logprobs, float* sampling_logprobs, const void* logits, float* scratch,
+                           const int64_t* seeds, const int64_t* steps, const float* temperatures, int64_t seed, int64_t step,
+                           float temperature, int64_t B, int64_t V, int dtype, void* stream) {
   LFM2_REQUIRE(B > 0 && V > 0, "sample: empty logits");
   LFM2_REQUIRE(B <= 65535, "sample: more than 65535 rows");
   LFM2_REQUIRE(temperature >= 0.f, "sample: negative temperature");
@@ -969,7 +988,8 @@ extern "C" int lfm2_sample(int64_t* tokens, float* logprobs, const void* logits,
                  hipLaunchKernelGGL(sample_partial_kernel<T>, dim3(parts, B), dim3(256), 0, s, (const T*)logits, scratch,
                                     temperatures, temperature, V, parts);
                  hipLaunchKernelGGL(sample_finish_kernel<T>, dim3(B), dim3(256), 0, s, (const T*)logits, scratch, tokens,
-                                    logprobs, seeds, steps, temperatures, seed, step, temperature, V, parts, RecordArgs{}));
+                                    logprobs, sampling_logprobs, seeds, steps, temperatures, seed, step, temperature, V, parts,
+                                    RecordArgs{}));
   LFM2_LAUNCH_CHECK();
 }
 
@@ -993,7 +1013,7 @@ extern "C" int lfm2_sample_record(int64_t* sampled, float* logp, const void* log
                  hipLaunchKernelGGL(sample_partial_kernel<T>, dim3(parts, B), dim3(256), 0, s, (const T*)logits, scratch,
                                     temperatures, 0.f, V, parts);
                  hipLaunchKernelGGL(sample_finish_kernel<T>, dim3(B), dim3(256), 0, s, (const T*)logits, scratch, sampled, logp,
-                                    seeds, steps, temperatures, 0, 0, 0.f, V, parts, record));
+                                    (float*)nullptr, seeds, steps, temperatures, 0, 0, 0.f, V, parts, record));
   LFM2_LAUNCH_CHECK();
 }
 
@@ -1040,10 +1060,10 @@ extern "C" int lfm2_sample_static(int64_t* tokens, float* logprobs, const void* 
   float* ptr = static_scratch();
   if (ptr == nullptr) return LFM2_ERR_LAUNCH;
   // pass 1 writes every record pass 2 reads, so nothing of the previous call's contents needs clearing
-  return lfm2_sample(tokens, logprobs, logits, ptr, seeds, steps, temperatures, seed, step, temperature, B, V, dtype, stream);
+  return lfm2_sample(tokens, logprobs, nullptr, logits, ptr, seeds, steps, temperatures, seed, step, temperature, B, V, dtype, stream);
 }
 
-extern "C" int lfm2_sample_filtered(int64_t* tokens, float* logprobs, int32_t* kept_count, const void* logits,
+extern "C" int lfm2_sample_filtered(int64_t* tokens, float* logprobs, float* sampling_logprobs, int32_t* kept_count, const void* logits,
                                     const int64_t* seeds, const int64_t* steps, const float* temperatures,
                                     const int32_t* top_ks, const float* top_ps, int64_t seed, int64_t step,
                                     float temperature, int top_k, float top_p, int64_t B, int64_t V, int dtype,
@@ -1060,12 +1080,12 @@ extern "C" int lfm2_sample_filtered(int64_t* tokens, float* logprobs, int32_t* k
   DISPATCH_DTYPE(dtype, "sample_filtered",
                  if (V <= (int64_t)kFT * kFV)
                    hipLaunchKernelGGL(sample_filtered_kernel<T>, dim3(B), dim3(kFT), 0, (hipStream_t)stream, (const T*)logits,
-                                      tokens, logprobs, kept_count, seeds, steps, temperatures, top_ks, top_ps, seed, step,
-                                      temperature, top_k, top_p, V);
+                                      tokens, logprobs, sampling_logprobs, kept_count, seeds, steps, temperatures, top_ks, top_ps,
+                                      seed, step, temperature, top_k, top_p, V);
                  else
                    hipLaunchKernelGGL(sample_filtered_stream_kernel<T>, dim3(B), dim3(kFT), 0, (hipStream_t)stream,
-                                      (const T*)logits, tokens, logprobs, kept_count, seeds, steps, temperatures, top_ks, top_ps,
-                                      seed, step, temperature, top_k, top_p, V));
+                                      (const T*)logits, tokens, logprobs, sampling_logprobs, kept_count, seeds, steps, temperatures,
+                                      top_ks, top_ps, seed, step, temperature, top_k, top_p, V));
   LFM2_LAUNCH_CHECK();
 }
 

@@ -265,7 +265,7 @@ class LFM25HIPDecoder:
         interval = self.finish_check_interval if batch >= 16 else 1
 
         for step in range(new_tokens):
-            sampled, raw = engine._sample(logits, sampling, step=step, seen_token_mask=seen)
+            sampled, raw, _ = engine._sample(logits, sampling, step=step, seen_token_mask=seen)
             if k:
                 ids, probs = ops.behavior_topk(logits, sampled, raw, k)
                 ops.record_head(ids, probs, head_ids, head_logprobs, lengths, alive, k, new_tokens)

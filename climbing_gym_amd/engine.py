@@ -534,23 +534,28 @@ class LFM25Engine:
         input_tokens = input_tokens.to(device=self.device, dtype=torch.long).reshape(-1)
         reject(input_tokens.numel() != state.active_slot_ids.numel(), "input_tokens must have one token per active slot")
         logits = self._append_decode_tokens(state.cache, state.active_slot_ids, input_tokens)
-        tokens, raw = self._sample(logits, sampling, step=0)
+        tokens, raw, tempered = self._sample(logits, sampling, step=0, sampling_logprobs=sampling.return_logprobs)
         reasons = self._finish_reasons(tokens, sampling)
         keep = sampling.return_logprobs
-        return LFM25StepOutput(tokens, raw if keep else None, raw if keep else None, reasons != 0, reasons, logits)
+        return LFM25StepOutput(tokens, raw if keep else None, tempered if keep else None, reasons != 0, reasons, logits)
 
     # ------------------------------------------------------------------ sampling helpers
-    def _sample(self, logits, sampling: LFM25SamplingConfig, *, step: int, seen_token_mask=None):
-        """Greedy, a full-support categorical draw, or temperature/top-k/top-p on the device; log-probabilities are the raw
-        log-softmax of the draw (lfm25_engine.py:1574-1609).  A repetition penalty is applied to an fp32 copy first."""
+    def _sample(self, logits, sampling: LFM25SamplingConfig, *, step: int, seen_token_mask=None, sampling_logprobs: bool = False):
+        """Greedy, a full-support categorical draw, or temperature/top-k/top-p on the device (lfm25_engine.py:1574-1609):
+        (tokens, raw log-softmax of the draw, its log-probability under the tempered and filtered distribution that was
+        sampled from — None unless `sampling_logprobs`).  A repetition penalty is applied to an fp32 copy first."""
         if seen_token_mask is not None and sampling.repetition_penalty != 1.0:
             lf = logits.float()
             penalised = torch.where(lf < 0, lf * sampling.repetition_penalty, lf / sampling.repetition_penalty)
             logits = torch.where(seen_token_mask, penalised, lf)
+        tempered = torch.empty(logits.size(0), device=logits.device, dtype=torch.float32) if sampling_logprobs else None
         if sampling.filtered:
-            return ops.sample_filtered(logits, temperature=sampling.temperature, top_k=sampling.top_k, top_p=sampling.top_p,
-                                       seed=sampling.seed, step=step)
-        return ops.sample_logits(logits, temperature=sampling.temperature, seed=sampling.seed, step=step, return_logprobs=True)
+            tokens, raw = ops.sample_filtered(logits, temperature=sampling.temperature, top_k=sampling.top_k, top_p=sampling.top_p,
+                                              seed=sampling.seed, step=step, sampling_logprobs=tempered)
+        else:
+            tokens, raw = ops.sample_logits(logits, temperature=sampling.temperature, seed=sampling.seed, step=step,
+                                            return_logprobs=True, sampling_logprobs=tempered)
+        return tokens, raw, tempered
 
     def _finish_reasons(self, token_ids, sampling: LFM25SamplingConfig):
         reasons = torch.zeros_like(token_ids, dtype=torch.int8)

@@ -544,15 +544,24 @@ def advance_positions(lengths, positions, slots, active):
 
 
 # ----------------------------------------------------------------------------------- sampling
+def _check_row_output(tensor, batch: int, dtype, device, name: str) -> None:
+    """A caller-provided per-row output the kernels write through a raw pointer: right type, size and place, or None."""
+    reject(tensor is not None and (not tensor.is_cuda or tensor.device != device or tensor.dtype != dtype
+                                   or tensor.numel() != batch or not tensor.is_contiguous()),
+           f"{name} must be a contiguous {dtype} tensor with one entry per row on the logits' device")
+
+
 def _sample_scratch(batch: int, vocab: int, device):
     return torch.empty(batch * ((vocab + 4095) // 4096) * 4, device=device, dtype=torch.float32)
 
 
-def sample_logits(logits: torch.Tensor, *, temperature: float, seed: int, step: int, return_logprobs: bool):
+def sample_logits(logits: torch.Tensor, *, temperature: float, seed: int, step: int, return_logprobs: bool,
+                  sampling_logprobs: torch.Tensor | None = None):
     """lfm25_sampling.py:61-92: greedy (first maximum) or a categorical draw from softmax(logits / T) over the
     full support (one uniform number per row through the inverse cumulative distribution: the same law as the
     reference's Gumbel-max); log-probabilities are the raw log-softmax of the chosen token.  Deterministic in
-    (seed, step)."""
+    (seed, step).  `sampling_logprobs` (fp32 [batch], optional) receives the draw's log-probability under
+    softmax(logits / T), the third value of lfm25_engine.py:1574-1609."""
     reject(logits.ndim != 2 or not logits.is_cuda or logits.dtype not in (torch.bfloat16, torch.float16, torch.float32),
            "sampling requires a 2D CUDA BF16/FP16/FP32 logits tensor")
     logits = logits.contiguous()
@@ -560,7 +569,8 @@ def sample_logits(logits: torch.Tensor, *, temperature: float, seed: int, step: 
     reject(batch == 0 or vocab == 0 or temperature < 0, "sampling requires nonempty logits and nonnegative temperature")
     tokens = torch.empty(batch, device=logits.device, dtype=torch.long)
     logprobs = torch.empty(batch, device=logits.device, dtype=torch.float32) if return_logprobs else None
-    call("lfm2_sample", tokens, logprobs, logits, _sample_scratch(batch, vocab, logits.device), None, None, None,
+    _check_row_output(sampling_logprobs, batch, torch.float32, logits.device, "sampling_logprobs")
+    call("lfm2_sample", tokens, logprobs, sampling_logprobs, logits, _sample_scratch(batch, vocab, logits.device), None, None, None,
          int(seed) & 0x7FFFFFFFFFFFFFFF, int(step), float(temperature), batch, vocab, _code(logits.dtype))
     return tokens, logprobs
 
@@ -570,9 +580,14 @@ def sample_logits_static(logits: torch.Tensor, tokens: torch.Tensor, logprobs: t
     """`sample_logits` into caller-provided outputs with no device allocation at all: the sampler's tile statistics
     live in a fixed 256 KiB array inside the library (at most 16384 row-tiles of 4096 logits per call; calls that
     overlap on one GPU race on it).  For callers that must not allocate; no counterpart in the reference."""
-    reject(logits.ndim != 2 or not logits.is_cuda or not logits.is_contiguous(),
-           "sampling requires a contiguous 2D GPU logits tensor")
+    reject(logits.ndim != 2 or not logits.is_cuda or not logits.is_contiguous()
+           or logits.dtype not in (torch.bfloat16, torch.float16, torch.float32),
+           "sampling requires a contiguous 2D GPU BF16/FP16/FP32 logits tensor")
     batch, vocab = logits.shape
+    reject(batch == 0 or vocab == 0 or temperature < 0, "sampling requires nonempty logits and nonnegative temperature")
+    reject(tokens is None, "tokens must be a contiguous torch.int64 tensor with one entry per row on the logits' device")
+    _check_row_output(tokens, batch, torch.long, logits.device, "tokens")
+    _check_row_output(logprobs, batch, torch.float32, logits.device, "logprobs")
     call("lfm2_sample_static", tokens, logprobs, logits, None, None, None, int(seed) & 0x7FFFFFFFFFFFFFFF, int(step),
          float(temperature), batch, vocab, _code(logits.dtype))
     return tokens, logprobs
@@ -589,7 +604,7 @@ class RowSampler:
         self.logprobs = torch.zeros(self.batch, device=logits.device, dtype=torch.float32)
 
     def sample(self, logits, seeds, steps, temperatures):
-        call("lfm2_sample", self.tokens, self.logprobs, logits, self.scratch, seeds, steps, temperatures, 0, 0, 1.0,
+        call("lfm2_sample", self.tokens, self.logprobs, None, logits, self.scratch, seeds, steps, temperatures, 0, 0, 1.0,
              self.batch, self.vocab, _code(logits.dtype))
         return self.tokens, self.logprobs
 
@@ -606,11 +621,13 @@ def sample_and_record(sampler: RowSampler, logits, table, input_tokens, stop_tab
 
 
 def sample_filtered(logits, *, temperature: float = 1.0, top_k: int = 0, top_p: float = 1.0, seed: int = 0, step: int = 0,
-                    seeds=None, steps=None, temperatures=None, top_ks=None, top_ps=None, return_kept: bool = False, out=None):
+                    seeds=None, steps=None, temperatures=None, top_ks=None, top_ps=None, return_kept: bool = False, out=None,
+                    sampling_logprobs: torch.Tensor | None = None):
     """Device form of `_sample` + `_apply_top_k_top_p` (lfm25_engine.py:1574-1609, 1759-1774) for temperature > 0:
     returns (tokens, raw log-probabilities[, survivors per row]).  With per-row `temperatures`, `top_ks` (int32) and
     `top_ps` every row has its own parameters, and rows that ask for no filter or for greedy decoding are left as `out`
-    holds them."""
+    holds them.  `sampling_logprobs` (fp32 [batch], optional) receives the draw's log-probability under the tempered,
+    filtered distribution (lfm25_engine.py:1605-1608)."""
     reject(logits.ndim != 2 or not logits.is_cuda, "sampling requires a 2D GPU logits tensor")
     logits = logits.contiguous()
     batch, vocab = logits.shape
@@ -618,7 +635,10 @@ def sample_filtered(logits, *, temperature: float = 1.0, top_k: int = 0, top_p: 
         torch.empty(batch, device=logits.device, dtype=torch.long),
         torch.empty(batch, device=logits.device, dtype=torch.float32))
     kept = torch.empty(batch, device=logits.device, dtype=torch.int32) if return_kept else None
-    call("lfm2_sample_filtered", tokens, logprobs, kept, logits, seeds, steps, temperatures, top_ks, top_ps,
+    _check_row_output(tokens, batch, torch.long, logits.device, "tokens")
+    _check_row_output(logprobs, batch, torch.float32, logits.device, "logprobs")
+    _check_row_output(sampling_logprobs, batch, torch.float32, logits.device, "sampling_logprobs")
+    call("lfm2_sample_filtered", tokens, logprobs, sampling_logprobs, kept, logits, seeds, steps, temperatures, top_ks, top_ps,
          int(seed) & 0x7FFFFFFFFFFFFFFF, int(step), float(temperature), int(top_k), float(top_p), batch, vocab,
          _code(logits.dtype))
     return (tokens, logprobs, kept) if return_kept else (tokens, logprobs)

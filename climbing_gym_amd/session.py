@@ -59,6 +59,14 @@ _REFUSALS = {
 }
 
 
+def filtered_on_device(sampling: LFM25SamplingConfig) -> bool:
+    """Whether the filtered sampler draws this request's rows.  The kernels decide per row from the float32 columns
+    of the row table, so the host decides from the same float32 values: a top_p such as 1 - 1e-9 is 1.0f there and a
+    temperature below the smallest float32 is 0 (greedy), and such a row belongs to the full-support sampler."""
+    as_f32 = lambda value: struct.unpack("<f", struct.pack("<f", float(value)))[0]
+    return as_f32(sampling.temperature) > 0.0 and (sampling.top_k > 0 or as_f32(sampling.top_p) < 1.0)
+
+
 def _refuse(condition: str):
     kind, text = _REFUSALS[condition]
     raise kind(text)
@@ -148,7 +156,7 @@ class _RowTable:
     def spec(slot: int, sampling: LFM25SamplingConfig, stop_offset: int, rng_position: int, stop_state: int) -> list:
         """The eight words `lfm2_configure_rows` reads for one request."""
         floats = struct.unpack("<q", struct.pack("<ff", float(sampling.temperature), float(sampling.top_p)))[0]
-        flags = int(bool(sampling.ignore_eos)) | (int(sampling.top_k if sampling.filtered else 0) << 8)
+        flags = int(bool(sampling.ignore_eos)) | (int(sampling.top_k if filtered_on_device(sampling) else 0) << 8)
         return [slot, sampling.max_new_tokens, sampling.seed & _SEED_MASK, rng_position, stop_state, stop_offset, flags, floats]
 
     def write(self, specs: list) -> None:
@@ -265,14 +273,16 @@ class LFM25GenerationSession:
         """(broken, message) for every rule a request must meet, in checking order; evaluated lazily, so a later rule
         may rely on the earlier ones."""
         vocab, table = self.engine.config.vocab_size, sampling.stop_table
-        yield not prompt, "Empty prompts are not supported"
+        # the order and the texts of lfm25_session.py:205-225; top-k / top-p requests, which the reference refuses with
+        # the same sentence, are accepted here (an extension: such rows are redrawn by the filtered sampler)
         yield sampling.behavior_topk > self.behavior_topk, "Request behavior head exceeds the session reservation"
+        yield not prompt, "Empty prompts are not supported"
         # three C-level passes over the ids instead of a Python loop
         yield (set(map(type, prompt)) != {int} or min(prompt) < 0 or max(prompt) >= vocab), "Prompt token outside the model vocabulary"
-        yield sampling.max_new_tokens > self.max_new_tokens, "Request exceeds the session generation buffer"
         yield (len(prompt) + sampling.max_new_tokens > self.entry.cache.max_seq_len), "Request exceeds reserved session context capacity"
+        yield sampling.max_new_tokens > self.max_new_tokens, "Request exceeds the session generation buffer"
         yield (sampling.repetition_penalty != 1.0,
-               "Sessions support greedy, full-support and top-k/top-p sampling without repetition penalties")
+               "Sessions support greedy/full-support sampling without repetition penalties")
         yield (bool(sampling.stop_token_sequences),
                "Sessions use stop_token_ids or stop_table; encode string stops with build_stop_table")
         yield any(not 0 <= token < vocab for token in sampling.stop_token_ids), "Stop token outside the model vocabulary"
@@ -302,7 +312,7 @@ class LFM25GenerationSession:
             slot = self.slots[index]
             slot.generation += 1
             slot.prompt, slot.sampling, slot.lease, slot.used_before = tuple(prompt), sampling, None, True
-            (self._filtered_rows.add if sampling.filtered else self._filtered_rows.discard)(index)
+            (self._filtered_rows.add if filtered_on_device(sampling) else self._filtered_rows.discard)(index)
             position, stop_state = (0, 0) if carried is None else carried[index]
             specs.append(_RowTable.spec(index, sampling, self.stops.offset(sampling), position, stop_state))
         self.rows.write(specs)

@@ -277,12 +277,14 @@ int lfm2_advance_positions(int32_t* lengths, const int32_t* positions, const int
 
 /* sample_logits / RowSampler.sample of lfm25_sampling.py:9-123: greedy (temperature 0: first
  * maximum) or a draw from softmax(logits / T) over the full support (inverse CDF, one uniform per row;
- * the same law as the reference's Gumbel-max, V <= 2^20); logprobs are raw log-softmax of the pick.
+ * the same law as the reference's Gumbel-max, V <= 2^20); logprobs are raw log-softmax of the pick,
+ * sampling_logprobs (may be NULL) its log-probability under softmax(logits / T), the distribution drawn from
+ * (greedy rows: the raw one; lfm25_engine.py:1591-1608).
  * Per-row arrays (seeds int64, steps int64, temperatures float) may be NULL, then the scalar
  * seed/step/temperature apply.  scratch: float[B*parts*4] with parts = ceil(V/4096). */
-int lfm2_sample(int64_t* tokens, float* logprobs, const void* logits, float* scratch, const int64_t* seeds,
-                const int64_t* steps, const float* temperatures, int64_t seed, int64_t step, float temperature,
-                int64_t B, int64_t V, int dtype, void* stream);
+int lfm2_sample(int64_t* tokens, float* logprobs, float* sampling_logprobs, const void* logits, float* scratch,
+                const int64_t* seeds, const int64_t* steps, const float* temperatures, int64_t seed, int64_t step,
+                float temperature, int64_t B, int64_t V, int dtype, void* stream);
 
 /* lfm2_sample without the scratch argument, for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc): the tile statistics go to a file-scope device array
@@ -297,11 +299,12 @@ int lfm2_sample_static(int64_t* tokens, float* logprobs, const void* logits, con
 
 /* _sample + _apply_top_k_top_p of lfm25_engine.py:1574-1609,1759-1774 on the device: temperature,
  * top-k (ties with the k-th value kept), nucleus (rank 0 never dropped), then a Gumbel-max draw
- * from what is left.  kept_count int32[B] (may be NULL) reports the survivors.
+ * from what is left.  kept_count int32[B] (may be NULL) reports the survivors; sampling_logprobs float[B] (may be
+ * NULL) the pick's log-probability under the tempered, filtered distribution (lfm25_engine.py:1605-1608).
  * temperatures float[B], top_ks int32[B], top_ps float[B] (all three or none) give every row its own parameters and
  * replace the scalars; a row whose parameters ask for no filter (top_k 0 and top_p 1) or for greedy decoding
  * (temperature 0) is then skipped and its outputs keep their contents (the sampler for those rows is lfm2_sample). */
-int lfm2_sample_filtered(int64_t* tokens, float* logprobs, int32_t* kept_count, const void* logits,
+int lfm2_sample_filtered(int64_t* tokens, float* logprobs, float* sampling_logprobs, int32_t* kept_count, const void* logits,
                          const int64_t* seeds, const int64_t* steps, const float* temperatures, const int32_t* top_ks,
                          const float* top_ps, int64_t seed, int64_t step, float temperature, int top_k, float top_p,
                          int64_t B, int64_t V, int dtype, void* stream);

@@ -112,6 +112,18 @@ def top_k_top_p_filter(logits: torch.Tensor, top_k: int, top_p: float) -> torch.
     return out
 
 
+def sampling_logprobs(logits: torch.Tensor, tokens: torch.Tensor, temperature: float, top_k: int, top_p: float):
+    """Third result of ``_sample`` (``lfm25_engine.py:1591-1608``): log-probability of ``tokens`` under the
+    distribution they were drawn from, softmax of the tempered logits with everything outside the top-k / nucleus
+    support at -inf; at temperature 0 it is the raw log-softmax (``:1594-1596``).  A token outside the support gets
+    -inf."""
+    lf = logits.float()
+    if temperature == 0.0:
+        return lf.gather(1, tokens[:, None])[:, 0] - torch.logsumexp(lf, -1)
+    kept = top_k_top_p_filter(lf / float(temperature), top_k, top_p)
+    return kept.gather(1, tokens[:, None])[:, 0] - torch.logsumexp(kept, -1)
+
+
 def repetition_penalty(logits, seen, penalty):
     """``lfm25_engine.py:1777-1790``."""
     if seen is None or penalty == 1.0:
@@ -390,13 +402,23 @@ class OracleEngine:
 
     # ---- sampling (lfm25_engine.py:1574-1609)
     def sample(self, logits, *, temperature=0.0, top_k=0, top_p=1.0, generator=None, seen=None, penalty=1.0):
+        """``lfm25_engine.py:1574-1609``: (token, raw log-probability)."""
+        tok, raw, _ = OracleEngine.sample_with_sampling_logprobs(self, logits, temperature=temperature, top_k=top_k, top_p=top_p,
+                                                         generator=generator, seen=seen, penalty=penalty)
+        return tok, raw
+
+    def sample_with_sampling_logprobs(self, logits, *, temperature=0.0, top_k=0, top_p=1.0, generator=None, seen=None,
+                                      penalty=1.0):
+        """``lfm25_engine.py:1574-1609`` with all three results: the token, its log-probability under softmax of the
+        (penalised) logits, and under the distribution it was drawn from (``sampling_logprobs`` below)."""
         lf = repetition_penalty(logits.float(), seen, penalty)
         if temperature == 0.0:
             tok = lf.argmax(-1)
         else:
             probs = torch.softmax(top_k_top_p_filter(lf / temperature, top_k, top_p), -1)
             tok = torch.multinomial(probs, 1, generator=generator)[:, 0]
-        return tok, lf.gather(1, tok[:, None])[:, 0] - torch.logsumexp(lf, -1)
+        raw = lf.gather(1, tok[:, None])[:, 0] - torch.logsumexp(lf, -1)
+        return tok, raw, sampling_logprobs(lf, tok, temperature, top_k, top_p)
 
     def generate(self, prompts, max_new_tokens: int, *, temperature=0.0, top_k=0, top_p=1.0, seed=0,
                  max_prefill_tokens=None, return_logits=False):

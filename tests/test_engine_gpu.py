@@ -401,7 +401,7 @@ def test_repetition_penalty_in_sample_and_generate_follows_the_cpu_engine():
     seen[:, logits.float().argmax(-1)] = True            # the unpenalised winners are all penalised
     for penalty in (1.0, 1.4, 0.6):
         sampling = LFM25SamplingConfig(temperature=0.0, repetition_penalty=penalty)
-        tokens, raw = engine._sample(logits.to(DEV), sampling, step=0, seen_token_mask=seen.to(DEV))
+        tokens, raw, _ = engine._sample(logits.to(DEV), sampling, step=0, seen_token_mask=seen.to(DEV))
         want_tokens, want_raw = O.OracleEngine.sample(None, logits.float(), temperature=0.0, seen=seen, penalty=penalty)
         assert torch.equal(tokens.cpu(), want_tokens)
         torch.testing.assert_close(raw.cpu(), want_raw, atol=3e-6, rtol=0)
@@ -424,6 +424,30 @@ def test_repetition_penalty_in_sample_and_generate_follows_the_cpu_engine():
             assert abs(penalised.log_softmax(-1)[token].item() - out.logprobs[row, 0, step].item()) <= 2e-2
             mask[0, token] = True
             row_logits = oracle.append_tokens(cache, torch.arange(1), torch.tensor([token]))
+
+
+@torch.inference_mode()
+def test_decode_step_returns_raw_and_sampling_logprobs_like_the_cpu_engine():
+    """lfm25_engine.py:714-735: `decode_step` returns the draw's raw log-probability and, as `sampling_logprobs`, its
+    log-probability under the tempered, filtered distribution (:1598-1608); both from the step's own logits."""
+    engine, ocfg, state = _engine()
+    prompts = [[1, 5, 9, 5], [3, 4], [7, 7, 7, 2, 250]]
+    for kwargs in (dict(temperature=0.7, top_k=5, top_p=0.9), dict(temperature=1.4), dict(temperature=0.8, top_p=0.6),
+                   dict(temperature=0.0)):
+        sampling = LFM25SamplingConfig(return_logprobs=True, seed=12, **kwargs)
+        prefix = engine.prefill(*_flat(prompts))
+        batch = engine.fork(prefix, 1, max_cache_len=16)
+        step = engine.decode_step(batch, torch.tensor([11, 12, 13]), sampling)
+        logits, tokens = step.logits.float().cpu(), step.token_ids.cpu()
+        want_raw = logits.double().log_softmax(-1).gather(1, tokens[:, None])[:, 0].float()
+        want = O.sampling_logprobs(logits.double(), tokens, sampling.temperature, sampling.top_k, sampling.top_p).float()
+        torch.testing.assert_close(step.raw_logprobs.cpu(), want_raw, atol=5e-6, rtol=2e-6)
+        torch.testing.assert_close(step.sampling_logprobs.cpu(), want, atol=1e-5, rtol=2e-6)
+        if kwargs.get("top_k") or kwargs.get("top_p", 1.0) < 1.0 or kwargs["temperature"] not in (0.0, 1.0):
+            assert not torch.allclose(step.sampling_logprobs, step.raw_logprobs)
+        quiet = engine.decode_step(engine.fork(prefix, 1, max_cache_len=16), torch.tensor([11, 12, 13]),
+                                   replace(sampling, return_logprobs=False))
+        assert quiet.raw_logprobs is None and quiet.sampling_logprobs is None and torch.equal(quiet.token_ids, step.token_ids)
 
 
 def test_graphs_can_be_dropped_and_recaptured_while_garbage_is_collected():
@@ -634,6 +658,54 @@ def test_session_rows_keep_their_own_sampling_whatever_their_neighbours_ask_for(
     assert list(together[(1, 4)][0]) == greedy.token_ids[0, 0].tolist()
     top1 = run([([1, 4], replace(base, top_k=1))])
     assert top1[(1, 4)][0] == together[(1, 4)][0]
+
+
+@torch.inference_mode()
+def test_session_row_whose_filter_vanishes_in_float32_is_still_drawn():
+    """A top_p of 1 - 1e-9 is 1.0 in the float32 column the kernels read, and a temperature below the smallest float32
+    is 0 there: the filtered kernel skips such rows, so the host must hand them to the full-support sampler.  Alone in
+    a session (no other row keeps that sampler running) they must decode like the same request with top_p = 1 /
+    temperature = 0, and record fresh tokens at every step."""
+    from climbing_gym_amd.session import filtered_on_device
+    engine, _, _ = _engine()
+    engine.enable_cuda_graphs(max_graphs=1)
+    base = LFM25SamplingConfig(temperature=1.0, seed=21, max_new_tokens=9, ignore_eos=True)
+    almost_one, tiny_temperature = replace(base, top_p=1.0 - 1e-9), replace(base, temperature=1e-60, top_k=5)
+    assert almost_one.filtered and not filtered_on_device(almost_one)
+    assert tiny_temperature.filtered and not filtered_on_device(tiny_temperature)
+    assert filtered_on_device(replace(base, top_p=0.999)) and filtered_on_device(replace(base, top_k=3))
+
+    def run(sampling):
+        with engine.generation_session(max_batch_size=2, max_new_tokens=9, cache_len=32) as session:
+            session.admit([[1, 2, 3]], [sampling])
+            (result,) = session.poll(steps=10)
+            return result.token_ids, result.logprobs
+
+    assert run(almost_one) == run(base)
+    assert run(tiny_temperature) == run(replace(base, temperature=0.0))
+    assert len(set(run(almost_one)[0])) > 2      # not one stale token repeated
+
+
+@torch.inference_mode()
+def test_session_validation_follows_the_reference_order_and_texts():
+    """lfm25_session.py:205-225: behaviour head before the empty-prompt check, context capacity before the generation
+    buffer, and the reference's sentence for the sampling rule (top-k / top-p themselves are accepted here)."""
+    engine, _, _ = _engine()
+    engine.enable_cuda_graphs(max_graphs=1)
+    ok = LFM25SamplingConfig(temperature=1.0, max_new_tokens=4, ignore_eos=True)
+    with engine.generation_session(max_batch_size=2, max_new_tokens=4, cache_len=16) as session:
+        with pytest.raises(ValueError, match="behavior head exceeds"):
+            session.admit([[]], [replace(ok, behavior_topk=3)])
+        with pytest.raises(ValueError, match="Empty prompts"):
+            session.admit([[]], [ok])
+        with pytest.raises(ValueError, match="reserved session context capacity"):
+            session.admit([[1] * 125], [replace(ok, max_new_tokens=9)])   # the 16-token request rounds up to a 128-token cache
+        with pytest.raises(ValueError, match="session generation buffer"):
+            session.admit([[1]], [replace(ok, max_new_tokens=5)])
+        with pytest.raises(ValueError, match="Sessions support greedy/full-support sampling without repetition penalties"):
+            session.admit([[1]], [replace(ok, repetition_penalty=1.2)])
+        session.admit([[1, 2]], [replace(ok, top_k=3, top_p=0.9)])
+        assert len(session.poll(steps=5)) == 1
 
 
 @torch.inference_mode()

@@ -165,6 +165,45 @@ def test_top_k_top_p_filter_by_brute_force(top_k, top_p):
     assert torch.isfinite(O.top_k_top_p_filter(torch.tensor([[9.0, 0.0, 0.0]]), 0, 0.01)).sum() == 1
 
 
+@pytest.mark.parametrize("temperature,top_k,top_p", [(1.0, 0, 1.0), (0.7, 0, 1.0), (0.7, 3, 1.0), (1.3, 0, 0.6), (0.5, 4, 0.8), (0.0, 0, 1.0)])
+def test_sampling_logprobs_by_brute_force(temperature, top_k, top_p):
+    """The third value of the reference's `_sample`: the pick's probability among the survivors of the tempered
+    logits, worked out term by term in Python floats.  A missing temperature, a normaliser over the whole row instead
+    of the survivors, or the raw logit in the numerator each fail one of the cases."""
+    g = torch.Generator().manual_seed(16)
+    logits = torch.randn(5, 9, generator=g) * 2
+    for r in range(5):
+        row = logits[r].tolist()
+        if temperature == 0.0:
+            kept, scaled = row, row
+        else:
+            scaled = [v / temperature for v in row]
+            kept = _filter_brute(scaled, top_k, top_p)
+        m = max(kept)
+        log_z = m + math.log(sum(math.exp(v - m) for v in kept if not math.isinf(v)))
+        for tok in range(9):
+            got = O.sampling_logprobs(logits[r:r + 1], torch.tensor([tok]), temperature, top_k, top_p).item()
+            if math.isinf(kept[tok]):
+                assert got == -math.inf
+            else:
+                assert abs(got - (scaled[tok] - log_z)) < 2e-6
+        # the survivors' probabilities sum to one
+        alive = [t for t in range(9) if not math.isinf(kept[t])]
+        total = sum(math.exp(O.sampling_logprobs(logits[r:r + 1], torch.tensor([t]), temperature, top_k, top_p).item()) for t in alive)
+        assert abs(total - 1.0) < 1e-5
+
+
+def test_sample_returns_raw_and_sampling_logprobs():
+    logits = torch.randn(6, 40, generator=torch.Generator().manual_seed(17))
+    gen = torch.Generator().manual_seed(0)
+    tok, raw, tempered = O.OracleEngine.sample_with_sampling_logprobs(None, logits, temperature=0.8, top_k=5, top_p=0.9, generator=gen)
+    torch.testing.assert_close(raw, logits.log_softmax(-1).gather(1, tok[:, None])[:, 0])
+    assert torch.isfinite(tempered).all()   # drawn tokens are survivors
+    torch.testing.assert_close(tempered, O.sampling_logprobs(logits, tok, 0.8, 5, 0.9))
+    tok0, raw0, tempered0 = O.OracleEngine.sample_with_sampling_logprobs(None, logits, temperature=0.0)
+    assert torch.equal(tok0, logits.argmax(-1)) and torch.equal(raw0, tempered0)
+
+
 def test_greedy_picks_first_maximum_and_true_log_softmax():
     logits = torch.randn(4, 1000, generator=torch.Generator().manual_seed(7)).bfloat16()
     logits[1, 12] = logits[1, 900] = 20
