@@ -5,8 +5,8 @@ A step is one decode token for every sequence of the batch: HIP-graph replay of 
 (FP8 W8A8 linears, e4m3 KV cache), on-device sampling and the record kernel.  Prompts (uniform lengths in
 [256, 2048], uniform token ids, seed 0) are prefilled before the timed region, so inputs are resident in
 HBM when timing starts.  Prints ONE JSON line with the throughput, the roofline of the dominant kernel
-(ragged GQA decode attention over the e4m3 cache, timed with HIP events on the launch stream) and the CPU
-baseline (the oracle's fp32 restatement of the reference CPU engine on a bounded sample of the same workload).
+(ragged GQA decode attention over the e4m3 cache, timed with device timestamps inside the replayed step) and the CPU
+baseline (the oracle's restatement of the reference CPU engine, bf16, on a bounded sample of the same workload).
 """
 from __future__ import annotations
 
@@ -40,17 +40,23 @@ def parse_args():
     p.add_argument("--max-model-len", type=int, default=8192)
     p.add_argument("--precision", choices=("fp8", "bf16"), default="fp8")
     p.add_argument("--cpu-seqs", type=int, default=4, help="sequences of the workload the CPU baseline runs (0 = skip)")
-    p.add_argument("--cpu-steps", type=int, default=96)
+    p.add_argument("--cpu-steps", type=int, default=16)
     p.add_argument("--attn-samples", type=int, default=20, help="timed launches of the decode-attention kernel per layer")
     p.add_argument("--mid-job-advance", type=int, default=2048,
                    help="second timed point: the same batch with every context this many tokens longer (0 = skip)")
     p.add_argument("--top-k", type=int, default=0, help="top-k filter of the sampler (0: full support)")
     p.add_argument("--top-p", type=float, default=1.0, help="top-p filter of the sampler (1: off)")
-    p.add_argument("--workload", choices=("decode", "attention", "gemm", "prefill", "serve"), default="decode",
+    p.add_argument("--workload", choices=("decode", "attention", "gemm", "prefill", "serve", "hbm-ceiling"), default="decode",
                    help="decode: the model's decode step (the headline metric); attention: the decode-attention call alone "
                         "on 256 sequences of U[128, 8192] history tokens, dense and paged (block 16), e4m3 and bf16; "
                         "gemm: the W8A8 projection shapes at 1..4096 rows; prefill: causal varlen attention over a packed "
-                        "4096-token chunk; serve: --requests requests through one session with continuous admit/retire")
+                        "4096-token chunk; serve: --requests requests through one session with continuous admit/retire; "
+                        "hbm-ceiling: the loads-only streaming read (every CU reading, 8 GiB per launch)")
+    p.add_argument("--rows", type=str, default="1,8,64,256,1024,4096", help="gemm workload: row counts, comma separated")
+    p.add_argument("--shapes", type=str, default="w13,conv_in,qkv,out,w2", help="gemm workload: projection shapes to run")
+    p.add_argument("--plain-launches", action="store_true",
+                   help="gemm workload: launch every product directly instead of replaying a graph, the fused MLP variants "
+                        "left out, and one 256 MiB copy for counter calibration at the end (for `rocprofv3 --pmc` runs)")
     p.add_argument("--requests", type=int, default=1024, help="requests of the serve workload")
     p.add_argument("--output-low", type=int, default=64, help="serve workload: shortest output, tokens")
     p.add_argument("--output-high", type=int, default=256, help="serve workload: longest output, tokens")
@@ -64,7 +70,8 @@ def gemm_workload(args):
     Every product is checked against the fp32 matmul of the dequantised operands (1e-2 relative, Frobenius)."""
     from climbing_gym_amd import ops
     shapes = {"w13": (11264, 2048), "conv_in": (6144, 2048), "qkv": (3072, 2048), "out": (2048, 2048), "w2": (2048, 5632)}
-    rows_list = (1, 8, 64, 256, 1024, 4096)
+    shapes = {name: shapes[name] for name in args.shapes.split(",")}
+    rows_list = tuple(int(r) for r in args.rows.split(","))
     gen = torch.Generator(device="cuda").manual_seed(0)
     begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     stream = torch.cuda.current_stream()
@@ -90,22 +97,30 @@ def gemm_workload(args):
                         p.linear_quantized(xq, xs)
             body()
             torch.cuda.synchronize()
-            side, graph = torch.cuda.Stream(), torch.cuda.CUDAGraph()
-            with torch.cuda.stream(side), torch.cuda.graph(graph, stream=side):
-                body()
-            torch.cuda.synchronize()
-            graph.replay()
-            begin.record(stream)
-            for _ in range(args.steps):
+            if args.plain_launches:
+                begin.record(stream)
+                for _ in range(args.steps):
+                    body()
+                end.record(stream)
+                end.synchronize()
+                graph = None
+            else:
+                side, graph = torch.cuda.Stream(), torch.cuda.CUDAGraph()
+                with torch.cuda.stream(side), torch.cuda.graph(graph, stream=side):
+                    body()
+                torch.cuda.synchronize()
                 graph.replay()
-            end.record(stream)
-            end.synchronize()
+                begin.record(stream)
+                for _ in range(args.steps):
+                    graph.replay()
+                end.record(stream)
+                end.synchronize()
             sec = begin.elapsed_time(end) / 1000 / (args.steps * repeats * copies)
             moved = n * k + 4 * n + m * k + 4 * m + 2 * m * n
             table[f"{name} n{n} k{k} m{m}"] = {"us": round(sec * 1e6, 2), "GBps": round(moved / sec / 1e9, 1),
-                                               "TFLOPs": round(2 * m * n * k / sec / 1e12, 1)}
+                                               "TFLOPs": round(2 * m * n * k / sec / 1e12, 1), "algorithmic_bytes": moved}
             del graph
-            if name == "w13" and m in (256, 4096):
+            if name == "w13" and m in (256, 4096) and not args.plain_launches:
                 # the MLP's first half as the engine runs it: projection, SwiGLU and per-token e4m3 rows for the down
                 # projection; with the SwiGLU in the product's epilogue, and as projection + SwiGLU launch
                 def timed(step):
@@ -135,13 +150,16 @@ def gemm_workload(args):
                                                           "fused_TFLOPs": round(2 * m * n * k / fused / 1e6, 1)}
         del packs
         torch.cuda.empty_cache()
-    big, small = table["w13 n11264 k2048 m4096"], table["w13 n11264 k2048 m256"]
+    if args.plain_launches:
+        calibration_copy()
+    big = table.get("w13 n11264 k2048 m4096") or max(table.values(), key=lambda r: r["TFLOPs"])
+    small = table.get("w13 n11264 k2048 m256") or max(table.values(), key=lambda r: r["GBps"])
     print(json.dumps({
         "metric": "W8A8 FP8 GEMM, gate+up projection (N 11264, K 2048) at 4096 rows", "value": big["TFLOPs"],
         "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": 1, "ms_per_step": round(big["us"] / 1000, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3 (fp32 accumulate, bf16 out)",
         "data": "synthetic",
-        "config": {"workload": "W8A8 products of the LFM2.5-1.2B projection shapes at 1, 8, 64, 256, 1024 and 4096 rows, "
+        "config": {"workload": f"W8A8 products of the LFM2.5-1.2B projection shapes {args.shapes} at {args.rows} rows, "
                                "per-token and per-channel scales, weights streamed from HBM",
                    "worst_relative_error": round(worst, 6), "shapes": table},
         "roofline": {"kernel": "gemm_nt_kernel (128x128 ring tile) at 4096 rows", "bound": "mfma", "achieved": big["TFLOPs"],
@@ -202,7 +220,7 @@ def prefill_workload(args):
 
 
 def attention_workload(args):
-    """One ragged GQA decode-attention call (split kernel + combine) on 256 sequences with U[128, 8192] history tokens,
+    """One ragged GQA decode-attention call (one workgroup per row and KV head, finished rows) on 256 sequences with U[128, 8192] history tokens,
     32 query heads over 8 KV heads of 64 dims: history stored dense (each head's tokens contiguous) and in 16-token
     pages reached through a shuffled block table (pages token-major and head-major), e4m3 with scales and bf16.
     Paged results must equal the dense ones bit for bit."""
@@ -362,9 +380,10 @@ def build_engine(args, state):
 
 
 def time_decode_attention(engine, session, samples):
-    """Average duration (s) of one decode-attention call (the persistent split kernel plus its combine kernel, over the
-    work list the decode step shares between its layers) at the batch's current context lengths, from HIP events
-    recorded on the launch stream around back-to-back launches, and the algorithmic bytes of one call."""
+    """Average duration (s) of one decode-attention call in the decode step's form (the attention kernel, one
+    workgroup per row and KV head over the schedule the step shares between its layers, plus the row quantiser when the
+    out projection is W8A8) at the batch's current context lengths, from HIP events recorded on the launch stream around
+    back-to-back launches, and the algorithmic bytes of one call."""
     from climbing_gym_amd import ops
     cfg, cache = engine.config, session.entry.cache
     rows = session.batch_size
@@ -408,6 +427,99 @@ def time_decode_attention(engine, session, samples):
     kv_token = cfg.num_key_value_heads * cfg.head_dim * 2 * (1 if cache.fp8 else 2) + (cfg.num_key_value_heads * 2 * 4 if cache.fp8 else 0)
     bytes_per_call = tokens * kv_token + 2 * rows * cfg.num_attention_heads * cfg.head_dim * 2
     return total_ms / 1000 / launches, bytes_per_call, tokens
+
+
+def time_attention_in_step(engine, session, replays):
+    """Duration (s) of one decode-attention call (attention kernel + row quantiser) INSIDE the replayed decode step: the
+    step is recorded once more with a timestamp kernel (one lane storing the device's constant-rate wall clock) before
+    and after each attention layer's call, replayed `replays` times, and the stamps are read after each replay.  This
+    is the time the call takes where it runs, after the QKV projection and with the other layers' traffic in the
+    caches.  A pair of adjacent stamps costs one dispatch gap, measured in a graph of adjacent pairs and subtracted, so
+    the figure holds the two kernels and the gaps between and after them like the back-to-back loop's elapsed / calls."""
+    from climbing_gym_amd import ops
+    layers = session.entry.cache.k_cache.size(0)
+    hz = ops.timestamp_rate_hz()
+    stamps = torch.zeros((layers, 2), device="cuda", dtype=torch.int64)
+    empty = torch.zeros((16, 2), device="cuda", dtype=torch.int64)
+    side, bracket = torch.cuda.Stream(), torch.cuda.CUDAGraph()
+    ops.timestamp(empty[0, 0])
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side), torch.cuda.graph(bracket, stream=side):
+        for pair in range(16):
+            ops.timestamp(empty[pair, 0])
+            ops.timestamp(empty[pair, 1])
+    torch.cuda.synchronize()
+    bracket.replay()
+    bracket.replay()
+    torch.cuda.synchronize()
+    gap_ticks = float((empty[:, 1] - empty[:, 0]).double().median())
+    graph = engine._cuda_decoder.capture_probed_step(session.entry, lambda kind, index, phase: ops.timestamp(stamps[index, phase]))
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    per_layer = torch.zeros(layers, dtype=torch.float64)
+    for _ in range(replays):
+        graph.replay()
+        torch.cuda.synchronize()
+        per_layer += (stamps[:, 1] - stamps[:, 0]).double().cpu() - gap_ticks
+    del graph, bracket
+    per_layer_s = per_layer / replays / hz
+    return float(per_layer_s.mean()), {"us_by_layer": [round(v * 1e6, 2) for v in per_layer_s.tolist()],
+                                       "bracket_us": round(gap_ticks / hz * 1e6, 2)}
+
+
+def measure_hbm_ceiling(gib=8, repeats=3):
+    """GB/s of the loads-only streaming read (`lfm2_hbm_stream_read`): `gib` GiB per launch, far beyond the 256 MB
+    memory-side cache, 2048 workgroups (eight per CU) each streaming a private contiguous region, and the same bytes
+    swept by the whole grid together; HIP events around `repeats` launches of each.  Returns (best, {layout: GB/s})."""
+    from climbing_gym_amd import ops
+    buffer = torch.empty(gib << 28, device="cuda", dtype=torch.int32)
+    buffer.zero_()
+    buffer[1] = 5     # read by lane 0 of workgroup 0 in both layouts
+    groups = 2048
+    sink = torch.empty(groups * 256, device="cuda", dtype=torch.int32)
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    stream = torch.cuda.current_stream()
+    rates = {}
+    for layout, name in ((0, "private_regions"), (1, "grid_sweep")):
+        read = ops.hbm_stream_read(buffer, sink, workgroups=groups, layout=layout)
+        torch.cuda.synchronize()
+        begin.record(stream)
+        for _ in range(repeats):
+            ops.hbm_stream_read(buffer, sink, workgroups=groups, layout=layout)
+        end.record(stream)
+        end.synchronize()
+        rates[name] = round(read * repeats / (begin.elapsed_time(end) / 1000) / 1e9, 1)
+    # every lane folds what it read into one word: the single non-zero word of the buffer must come out, once
+    if int(sink[0]) != 5 or int(sink.count_nonzero()) != 1:
+        raise SystemExit("the streaming read did not fold what it read")
+    del buffer
+    torch.cuda.empty_cache()
+    return max(rates.values()), rates
+
+
+def ceiling_workload(args):
+    """The chip's streaming read rate as this library can measure it: every CU issuing 16-byte loads, nothing else."""
+    best, rates = measure_hbm_ceiling(gib=8, repeats=max(args.steps, 3))
+    src = torch.ones(64 << 20, device="cuda", dtype=torch.int32)
+    dst = torch.empty_like(src)
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.mul(src, 1, out=dst)
+    begin.record()
+    for _ in range(10):
+        torch.mul(src, 1, out=dst)
+    end.record()
+    end.synchronize()
+    copy_rate = round(2 * src.numel() * 4 * 10 / (begin.elapsed_time(end) / 1000) / 1e9, 1)
+    print(json.dumps({
+        "metric": "HBM streaming read, loads only, 8 GiB per launch", "value": best, "unit": "GB/s", "n_gpus": 1,
+        "steps": max(args.steps, 3), "warmup": 1, "ms_per_step": round((8 << 30) / best / 1e6, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "u8 (16-byte loads)", "data": "synthetic",
+        "config": {"workload": "hbm_stream_kernel: 2048 workgroups x 256 lanes, eight 16-byte loads in flight per lane, 8 GiB "
+                               "read once per launch", "layouts_GBps": rates, "elementwise_copy_256MiB_read_plus_write_GBps": copy_rate},
+        "roofline": {"kernel": "hbm_stream_kernel", "bound": "hbm", "achieved": best, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(best / HBM_PEAK_GBS, 4), "traffic": None},
+        "cpu_baseline": None}))
 
 
 def time_gemms(engine, rows=256, prefill_rows=4096, repeats=5):
@@ -488,28 +600,41 @@ def measured_traffic(args, attn_bytes):
 
 
 def cpu_baseline(args, state, prompts):
-    """The oracle (fp32 restatement of the reference CPU engine) on the first `cpu_seqs` sequences of the workload:
-    prefill untimed, `cpu_steps` greedy decode steps timed on all host threads."""
+    """The oracle (restatement of the reference CPU engine) on the first `cpu_seqs` sequences of the workload, with
+    bf16 weights and activations as the reference's engine holds a 1.2B model: one untimed warm-up (a short prompt and
+    two steps), then two repeats of prefill + `cpu_steps` greedy decode steps, both phases timed, on all host threads;
+    the medians are reported, `value` being the decode rate (the metric is decode output tok/s)."""
     from climbing_gym_amd.synthetic import LFM2_1P2B
     from oracle.lfm2_oracle import OracleConfig, OracleEngine
     torch.set_num_threads(max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))))
     ocfg = OracleConfig(vocab_size=LFM2_1P2B["vocab"], hidden_size=LFM2_1P2B["hidden"], mlp_hidden_size=LFM2_1P2B["mlp_hidden"],
                         num_hidden_layers=16, num_attention_heads=32, num_key_value_heads=8,
                         layer_types=LFM2_1P2B["layer_types"])
-    oracle = OracleEngine(ocfg, state, torch.float32, max_model_len=args.max_model_len)
+    oracle = OracleEngine(ocfg, state, torch.bfloat16, max_model_len=args.max_model_len)
     sample = prompts[:args.cpu_seqs]
+    slots = torch.arange(len(sample))
+    decode_rates, prefill_rates = [], []
     with torch.inference_mode():
-        cache, logits = oracle.prefill(sample, cap=max(map(len, sample)) + args.cpu_steps + 1)
-        slots = torch.arange(len(sample))
-        tokens = logits.argmax(-1)
-        start = time.perf_counter()
-        for _ in range(args.cpu_steps):
-            logits = oracle.append_tokens(cache, slots, tokens)
+        cache, logits = oracle.prefill([sample[0][:64]], cap=72)
+        for _ in range(2):
+            logits = oracle.append_tokens(cache, torch.arange(1), logits.argmax(-1))
+        for _ in range(2):
+            start = time.perf_counter()
+            cache, logits = oracle.prefill(sample, cap=max(map(len, sample)) + args.cpu_steps + 1)
             tokens = logits.argmax(-1)
-        elapsed = time.perf_counter() - start
-    return {"value": round(len(sample) * args.cpu_steps / elapsed, 3), "unit": "tok/s", "cores": torch.get_num_threads(),
-            "kind": "port", "sample": f"first {len(sample)} of the {args.batch} sequences (fp32 weights), prefill untimed, "
-                                       f"{args.cpu_steps} greedy decode steps timed"}
+            middle = time.perf_counter()
+            for _ in range(args.cpu_steps):
+                logits = oracle.append_tokens(cache, slots, tokens)
+                tokens = logits.argmax(-1)
+            done = time.perf_counter()
+            prefill_rates.append(sum(map(len, sample)) / (middle - start))
+            decode_rates.append(len(sample) * args.cpu_steps / (done - middle))
+    median = lambda xs: sorted(xs)[len(xs) // 2] if len(xs) % 2 else sum(sorted(xs)[len(xs) // 2 - 1:len(xs) // 2 + 1]) / 2
+    return {"value": round(median(decode_rates), 3), "unit": "tok/s", "cores": torch.get_num_threads(), "kind": "port",
+            "prefill_tok_per_s": round(median(prefill_rates), 1),
+            "sample": f"first {len(sample)} of the {args.batch} sequences ({sum(map(len, sample))} prompt tokens), bf16 weights and "
+                      f"activations, one warm-up, then the median of 2 repeats of prefill (timed apart) + {args.cpu_steps} greedy "
+                      "decode steps; a bounded sample because the whole batch would take hours on the host"}
 
 
 def main():
@@ -521,7 +646,7 @@ def main():
     if args.workload != "decode":
         with torch.inference_mode():
             {"attention": attention_workload, "gemm": gemm_workload, "prefill": prefill_workload,
-             "serve": serve_workload}[args.workload](args)
+             "serve": serve_workload, "hbm-ceiling": ceiling_workload}[args.workload](args)
         return
     from climbing_gym_amd.config import LFM25SamplingConfig
     from climbing_gym_amd.synthetic import LFM2_1P2B, random_prompts, random_state_dict
@@ -553,12 +678,21 @@ def main():
         elapsed = time.perf_counter() - t0
         assert not finished, "no sequence may finish inside the timed region"
         attn_s, attn_bytes, ctx_tokens = time_decode_attention(engine, session, args.attn_samples)
+        in_step_s, in_step_layers = time_attention_in_step(engine, session, max(args.attn_samples // 2, 4))
         kv_token = 6 * (attn_bytes - 2 * args.batch * 32 * 64 * 2) // max(ctx_tokens, 1)
         # the same batch later in the job: every row's context longer by `--mid-job-advance` tokens (the cache is
         # written by the steps that follow; what the history holds does not change what the step costs)
         mid = None
-        if args.mid_job_advance > 0:
-            session.entry.cache.seq_lens.add_(args.mid_job_advance)
+        # every position a step of this run will write must lie inside the cache: the steps timed so far, the probed
+        # replays, then 2 + steps more at the advanced lengths, and the probed replays there
+        cache = session.entry.cache
+        headroom = cache.max_seq_len - int(cache.seq_lens.max()) - (2 + args.steps + 2 * args.attn_samples + 16)
+        advance = min(args.mid_job_advance, headroom)
+        if 0 < advance < args.mid_job_advance:
+            print(f"--mid-job-advance {args.mid_job_advance} does not fit the {cache.max_seq_len}-token cache behind the "
+                  f"longest row: advancing by {advance}", file=sys.stderr)
+        if advance > 0:
+            cache.seq_lens.add_(advance)   # the skipped span holds the zeros the cache was allocated with
             session.poll(steps=2)
             torch.cuda.synchronize()
             t0 = time.perf_counter()
@@ -567,26 +701,35 @@ def main():
             mid_elapsed = time.perf_counter() - t0
             assert not finished, "no sequence may finish inside the timed region"
             mid_attn_s, mid_attn_bytes, mid_tokens = time_decode_attention(engine, session, max(args.attn_samples // 2, 2))
-            mid = (mid_elapsed, mid_attn_s, mid_attn_bytes, mid_tokens)
+            mid_in_step_s, _ = time_attention_in_step(engine, session, max(args.attn_samples // 4, 3))
+            mid = (mid_elapsed, mid_attn_s, mid_attn_bytes, mid_tokens, mid_in_step_s, advance)
         calibration_copy()
         gemms = time_gemms(engine) if fp8_requested(args) else None
+        ceiling, ceiling_layouts = measure_hbm_ceiling()
     fp8 = args.precision == "fp8"
     weights = sum(w.numel() for w in set(engine.weights.linear_matrices())) * (1 if fp8 else 2)
     fixed_bytes = weights + args.batch * 122880 * 2 + args.batch * cfg.vocab_size * 2 * 2
     step_bytes = fixed_bytes + ctx_tokens * kv_token
     ms_per_step = elapsed / args.steps * 1000
-    achieved = attn_bytes / attn_s / 1e9
+    # the roofline figure is the call's time INSIDE the replayed step; the back-to-back loop over the layers' caches
+    # (faster: no other kernel's traffic between the calls) is reported next to it
+    loop_achieved = attn_bytes / attn_s / 1e9
+    launch_s = in_step_s if in_step_s is not None else attn_s
+    achieved = attn_bytes / launch_s / 1e9
     mid_job = None
     if mid is not None:
-        mid_elapsed, mid_attn_s, mid_attn_bytes, mid_tokens = mid
+        mid_elapsed, mid_attn_s, mid_attn_bytes, mid_tokens, mid_in_step_s, advance = mid
         mid_ms = mid_elapsed / args.steps * 1000
         mid_bytes = fixed_bytes + mid_tokens * kv_token
-        mid_job = {"context_tokens": mid_tokens, "ms_per_step": round(mid_ms, 4),
+        mid_launch_s = mid_in_step_s if mid_in_step_s is not None else mid_attn_s
+        mid_job = {"advance": advance, "context_tokens": mid_tokens, "ms_per_step": round(mid_ms, 4),
                    "tok_per_s": round(args.batch * args.steps / mid_elapsed, 1), "step_algorithmic_bytes": mid_bytes,
                    "step_hbm_fraction": round(mid_bytes / (mid_ms / 1000) / 1e9 / HBM_PEAK_GBS, 4),
-                   "attention_us_per_call": round(mid_attn_s * 1e6, 2),
-                   "attention_GBps": round(mid_attn_bytes / mid_attn_s / 1e9, 1),
-                   "attention_frac": round(mid_attn_bytes / mid_attn_s / 1e9 / HBM_PEAK_GBS, 4)}
+                   "attention_us_per_call": round(mid_launch_s * 1e6, 2),
+                   "attention_GBps": round(mid_attn_bytes / mid_launch_s / 1e9, 1),
+                   "attention_frac": round(mid_attn_bytes / mid_launch_s / 1e9 / HBM_PEAK_GBS, 4),
+                   "attention_frac_of_measured_ceiling": round(mid_attn_bytes / mid_launch_s / 1e9 / ceiling, 4),
+                   "attention_loop_us_per_call": round(mid_attn_s * 1e6, 2)}
     line = {
         "metric": "decode output tok/s @256 ragged seqs, LFM2.5-1.2B FP8; % HBM roofline",
         "value": round(args.batch * args.steps / elapsed, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
@@ -601,12 +744,20 @@ def main():
                    "prefill_chunks": prefill_plan.get("chunks"), "prefill_chunk_fill": round(prefill_plan.get("fill", 0.0), 4),
                    "gemm": gemms, "step_algorithmic_bytes": step_bytes,
                    "step_hbm_fraction": round(step_bytes / (ms_per_step / 1000) / 1e9 / HBM_PEAK_GBS, 4),
+                   "step_fraction_of_measured_ceiling": round(step_bytes / (ms_per_step / 1000) / 1e9 / ceiling, 4),
                    "mid_job": mid_job},
         "roofline": {"kernel": "decode_attn_mfma_kernel, one workgroup per row and KV head, + quantize_kernel (one ragged GQA decode-attention call, e4m3 KV, rows quantised for the W8A8 out projection as in the decode step)"
                                if fp8 else "decode_attn_mfma_kernel, one workgroup per row and KV head (one ragged GQA decode-attention call, bf16 KV)",
                      "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(args, attn_bytes),
-                     "avg_launch_us": round(attn_s * 1e6, 2), "algorithmic_bytes_per_launch": attn_bytes},
+                     "timed": "device timestamps recorded before and after the call inside the replayed decode step",
+                     "avg_launch_us": round(launch_s * 1e6, 2), "in_step": in_step_layers,
+                     "algorithmic_bytes_per_launch": attn_bytes,
+                     "back_to_back_loop": {"avg_launch_us": round(attn_s * 1e6, 2), "achieved": round(loop_achieved, 1),
+                                           "frac": round(loop_achieved / HBM_PEAK_GBS, 4)},
+                     "measured_ceiling": {"GBps": ceiling, "layouts_GBps": ceiling_layouts,
+                                          "what": "loads-only streaming read of 8 GiB by 2048 workgroups (lfm2_hbm_stream_read)"},
+                     "frac_of_measured_ceiling": round(achieved / ceiling, 4)},
     }
     del session
     engine.disable_cuda_graphs()

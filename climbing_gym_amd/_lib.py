@@ -62,6 +62,8 @@ _SIGNATURES = {
     "lfm2_record_sample": "ppppppppppppppp" "llllp",
     "lfm2_sample_record": "pppppppppppppppppppp" "llllip",
     "lfm2_record_head": "pppppp" "illp",
+    "lfm2_hbm_stream_read": "plpiip",
+    "lfm2_timestamp": "pp",
 }
 _INT64_RESULT = {
     "lfm2_fp8_gemm_workspace": "lll",
@@ -72,6 +74,7 @@ _INT64_RESULT = {
     "lfm2_bf16_gemm_workspace": "lll",
     "lfm2_decode_attention_workspace": "liil",
     "lfm2_decode_schedule_size": "ll",
+    "lfm2_timestamp_rate_khz": "",
 }
 _CTYPE = {"p": ctypes.c_void_p, "l": ctypes.c_int64, "i": ctypes.c_int, "f": ctypes.c_float}
 

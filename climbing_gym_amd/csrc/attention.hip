@@ -387,7 +387,15 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
     if (PAGED) {
       const int64_t koff = token_offset(b, slot, h, tk);
 #pragma unroll
-      for (int c = 0; c < 4; ++c) t.k[c] = *reinterpret_cast<const i32x4*>(kbase + koff * ES + krow_byte + 16 * c);
+      for (int c = 0; c < 4; ++c) {
+        if constexpr (FP8) {   // a quarter row of token 16c + lane / 4: see the dense form below
+          int tc = T + 16 * c + (lane >> 2);
+          tc = tc < wend ? tc : wend - 1;
+          t.k[c] = *reinterpret_cast<const i32x4*>(kbase + token_offset(b, slot, h, tc) + 16 * (lane & 3));
+        } else {
+          t.k[c] = *reinterpret_cast<const i32x4*>(kbase + koff * ES + krow_byte + 16 * c);
+        }
+      }
       if constexpr (FP8) {
         t.sk = a.ks[koff / D];
         t.sv = a.vs[koff / D];
@@ -406,20 +414,32 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
       const uint8_t* vitem = vbase + item_base * ES;
       const uint32_t row_bytes = (uint32_t)a.c1 * ES;
       const uint32_t koff = (uint32_t)tk * row_bytes + krow_byte;
+      // a history is read once per step and is far larger than the caches: non-temporal loads (streaming reads of
+      // this size run at 6.6-6.9 TB/s with the hint against 5.9-6.1 without)
 #pragma unroll
-      for (int c = 0; c < 4; ++c) t.k[c] = *reinterpret_cast<const i32x4*>(kitem + koff + 16 * c);
+      for (int c = 0; c < 4; ++c) {
+        if constexpr (FP8) {
+          // the K tile as 4 x 1 KiB of consecutive bytes: load c brings lane L the quarter row L % 4 of token
+          // 16c + L / 4, so every instruction asks for whole cache lines; the rows are put back together through LDS
+          int tc = T + 16 * c + (lane >> 2);
+          tc = tc < wend ? tc : wend - 1;
+          t.k[c] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(kitem + (uint32_t)tc * row_bytes + 16 * (lane & 3)));
+        } else {
+          t.k[c] = *reinterpret_cast<const i32x4*>(kitem + koff + 16 * c);
+        }
+      }
       if constexpr (FP8) {
         const float* ks_item = a.ks + item_base / D;
         const float* vs_item = a.vs + item_base / D;
         const uint32_t soff = (uint32_t)tk * (uint32_t)(a.c1 / D);
-        t.sk = ks_item[soff];
-        t.sv = vs_item[soff];
+        t.sk = __builtin_nontemporal_load(ks_item + soff);
+        t.sv = __builtin_nontemporal_load(vs_item + soff);
       }
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         int tv = T + vstep * u + vtok;
         tv = tv < wend ? tv : wend - 1;
-        t.v[u] = *reinterpret_cast<const i32x4*>(vitem + (uint32_t)tv * row_bytes + vbyte);
+        t.v[u] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(vitem + (uint32_t)tv * row_bytes + vbyte));
       }
     }
     if constexpr (!FP8) { t.sk = 1.f; t.sv = 1.f; }
@@ -525,15 +545,22 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
 #pragma unroll
       for (int i = 0; i < 4; ++i) s[i] = add_lane_xor32(s[i]);
     } else {
+    // the K quarter rows go to LDS as they arrived and come back as rows: lane L owns token L.  The 16-byte column of
+    // a row is XORed with bits 2..3 of its token, which spreads both the 16 stores and the 16 loads that share a cycle
+    // over all banks.  The buffer is the wave's V buffer: the V rows are stored after these reads.
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      *reinterpret_cast<i32x4*>(&lds_v[wave][16 * c + (lane >> 2)][16 * ((lane & 3) ^ (g16 & 3))]) = cur.k[c];
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
+      const i32x4 kr = *reinterpret_cast<const i32x4*>(&lds_v[wave][lane][16 * (c ^ ((lane >> 2) & 3))]);
       const i32x4 q4 = *reinterpret_cast<const i32x4*>(&lds_q[wave][g][16 * c]);       // dims 16c .. 16c+7
       const i32x4 q5 = *reinterpret_cast<const i32x4*>(&lds_q[wave][g][16 * c + 8]);   // dims 16c+8 .. 16c+15
       const i32x2 qa = {q4[0], q4[1]}, qb = {q4[2], q4[3]}, qc = {q5[0], q5[1]}, qd = {q5[2], q5[3]};
-      s = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, qa), e4m3x4_to_bf16x4(cur.k[c][0]), s, 0, 0, 0);
-      s = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, qb), e4m3x4_to_bf16x4(cur.k[c][1]), s, 0, 0, 0);
-      s = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, qc), e4m3x4_to_bf16x4(cur.k[c][2]), s, 0, 0, 0);
-      s = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, qd), e4m3x4_to_bf16x4(cur.k[c][3]), s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, qa), e4m3x4_to_bf16x4(kr[0]), s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, qb), e4m3x4_to_bf16x4(kr[1]), s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, qc), e4m3x4_to_bf16x4(kr[2]), s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, qd), e4m3x4_to_bf16x4(kr[3]), s, 0, 0, 0);
     }
     }
     // the tile's V rows to LDS, as they arrived (row = token, 16 bytes per lane)

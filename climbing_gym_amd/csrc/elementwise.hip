@@ -913,3 +913,72 @@ extern "C" int lfm2_prepare_qkv_store(void* q, const void* x, const void* q_weig
   else { DISPATCH_DTYPE(dtype, (launch_prepare<T, 1>(a, D, (hipStream_t)stream))); }
   LFM2_LAUNCH_CHECK();
 }
+
+// ------------------------------------------------------------------------------------ HBM streaming read probe
+// What the chip delivers when every CU only reads: the measured ceiling that the bandwidth-bound kernels of this
+// library are held against next to the nominal 8 TB/s.  Each lane keeps UNROLL 16-byte loads in flight, folds what
+// arrives into one word (so the loads cannot be dropped) and stores that word once at the end.
+//   layout 0: every workgroup streams a private contiguous region (how the decode-attention kernel reads a history);
+//   layout 1: the whole grid sweeps the buffer together, workgroup w taking 4 KiB blocks w, w + grid, ...
+namespace {
+template <int UNROLL, bool SWEEP>
+__global__ void __launch_bounds__(256)
+hbm_stream_kernel(const i32x4* __restrict__ src, int64_t vectors, int32_t* __restrict__ sink) {
+  const int64_t grid = gridDim.x, block = blockIdx.x;
+  // a block is 256 lanes x 16 bytes; blocks [first, first + count) with stride `step` belong to this workgroup
+  const int64_t blocks = vectors / 256;
+  const int64_t per = blocks / grid;                      // whole blocks per workgroup; the tail is not read
+  const int64_t first = SWEEP ? block : block * per, step = SWEEP ? grid : 1;
+  i32x4 acc = {0, 0, 0, 0};
+  int64_t b = 0;
+  for (; b + UNROLL <= per; b += UNROLL) {
+    i32x4 v[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+      v[u] = __builtin_nontemporal_load(src + (first + (b + u) * step) * 256 + threadIdx.x);
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) acc ^= v[u];
+  }
+  for (; b < per; ++b) acc ^= __builtin_nontemporal_load(src + (first + b * step) * 256 + threadIdx.x);
+  sink[block * 256 + threadIdx.x] = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
+}
+}  // namespace
+
+extern "C" int lfm2_hbm_stream_read(const void* src, int64_t bytes, int32_t* sink, int workgroups, int layout, void* stream) {
+  LFM2_REQUIRE(src && sink, "hbm_stream_read: null buffer");
+  LFM2_REQUIRE(((uintptr_t)src & 15) == 0, "hbm_stream_read: source not 16-byte aligned");
+  LFM2_REQUIRE(workgroups > 0 && workgroups <= 65536, "hbm_stream_read: workgroups %d not in [1, 65536]", workgroups);
+  LFM2_REQUIRE(bytes >= (int64_t)workgroups * 4096, "hbm_stream_read: fewer than 4096 bytes per workgroup");
+  LFM2_REQUIRE(layout == 0 || layout == 1, "hbm_stream_read: layout %d not 0 (private regions) or 1 (sweep)", layout);
+  const int64_t vectors = bytes / 16;
+  if (layout == 0)
+    hipLaunchKernelGGL((hbm_stream_kernel<8, false>), dim3(workgroups), dim3(256), 0, (hipStream_t)stream,
+                       (const i32x4*)src, vectors, sink);
+  else
+    hipLaunchKernelGGL((hbm_stream_kernel<8, true>), dim3(workgroups), dim3(256), 0, (hipStream_t)stream,
+                       (const i32x4*)src, vectors, sink);
+  LFM2_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------------------ device timestamps
+// A one-lane kernel that stores the device's constant-rate wall clock.  Recorded into a graph in front of and behind
+// a kernel, two of them bracket that kernel's time inside the replayed graph (stream order makes each run when its
+// predecessor has finished); two adjacent ones measure the cost of the bracket itself.
+namespace {
+__global__ void timestamp_kernel(int64_t* out) {
+  if (threadIdx.x == 0) *out = (int64_t)wall_clock64();
+}
+}  // namespace
+
+extern "C" int lfm2_timestamp(int64_t* out, void* stream) {
+  LFM2_REQUIRE(out != nullptr, "timestamp: null output");
+  hipLaunchKernelGGL(timestamp_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, out);
+  LFM2_LAUNCH_CHECK();
+}
+
+extern "C" int64_t lfm2_timestamp_rate_khz(void) {
+  int device = 0, rate = 0;
+  if (hipGetDevice(&device) != hipSuccess) return 0;
+  if (hipDeviceGetAttribute(&rate, hipDeviceAttributeWallClockRate, device) != hipSuccess) return 0;
+  return rate;
+}

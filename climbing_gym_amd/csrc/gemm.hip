@@ -15,6 +15,9 @@
 // Workgroup ids are remapped so that the M-tiles sharing one W tile run back to back on the same
 // XCD (ids are dealt round-robin over the 8 XCDs, each with its own L2): W streams from HBM once.
 #include "lfm2_common.h"
+#ifndef LFM2_W_AUX
+#define LFM2_W_AUX 0
+#endif
 
 namespace {
 
@@ -272,7 +275,7 @@ gemm_nt_body(void* __restrict__ out, float* __restrict__ partial, const uint8_t*
           if (EPI == 2) gr = swiglu_weight_row(gr, N);
           if (EPI == 3) gr = conv_weight_row(gr, N);
           __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(W + (int64_t)gr * Kb + kb + c * 16),
-                                           (__attribute__((address_space(3))) void*)(&lds[buf][A_CHUNKS + i * NT + wave * 64]), 16, 0, 0);
+                                           (__attribute__((address_space(3))) void*)(&lds[buf][A_CHUNKS + i * NT + wave * 64]), 16, 0, LFM2_W_AUX);
         }
       }
     };

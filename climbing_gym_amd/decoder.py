@@ -119,8 +119,9 @@ class LFM25HIPDecoder:
         return self.engine._decode_forward(cache, tokens, active, slot_ids=slot_ids, positions=positions, fp8=self.fp8_weights,
                                            logits_out=logits_out, gather=gather)
 
-    def _capture(self, step, before_warmup=None):
-        """Two warm-up launches, then record `step` into a HIP graph on the decoder's capture stream."""
+    def _capture(self, step, before_warmup=None, probe=None):
+        """Two warm-up launches, then record `step` into a HIP graph on the decoder's capture stream.  `probe` is
+        installed as the engine's step probe for the recorded run only."""
         if not self.capture:
             return _EagerStep(step)
         device = self.engine.device
@@ -144,10 +145,12 @@ class LFM25HIPDecoder:
         # an object (thread-local capture mode confines the check to the capturing thread).
         collector_was_on = gc.isenabled()
         gc.disable()
+        self.engine._step_probe = probe
         try:
             with torch.cuda.graph(graph, stream=stream, capture_error_mode="thread_local"):
                 step()
         finally:
+            self.engine._step_probe = None
             if collector_was_on:
                 gc.enable()
         current.wait_stream(stream)
@@ -184,6 +187,29 @@ class LFM25HIPDecoder:
         if batch_size >= 64:
             torch.cuda.empty_cache()
         return entry
+
+    @torch.inference_mode()
+    def capture_probed_step(self, entry: _DecodeGraph, probe):
+        """`entry`'s decode step recorded once more, over the same cache and buffers, with `probe(kind, index, phase)`
+        called on the capture stream before (phase 0) and after (phase 1) each decode-attention call (`kind` is
+        "attention", `index` the attention layer).  A probe that records events made with `external=True` puts
+        event-record nodes around those kernels, so their time inside a replayed step can be read with
+        `Event.elapsed_time`.  For measurement: the two warm-up runs advance the rolling conv state, which is put back
+        together with the lengths; the rows they append to the KV cache are overwritten by the next real step."""
+        reject(not self.capture, "a probed step needs graph capture", RuntimeError)
+        cache = entry.cache
+        lengths, conv_state = cache.seq_lens.clone(), cache.conv_state.clone()
+        logits = entry.logits
+
+        def restore():
+            cache.seq_lens.copy_(lengths)
+            cache.conv_state.copy_(conv_state)
+
+        def step():
+            self._forward(cache, entry.input_tokens, entry.active, logits_out=logits)
+
+        graph = self._capture(step, before_warmup=restore, probe=probe)
+        return graph
 
     @torch.inference_mode()
     def capture_compact(self, entry: _DecodeGraph, batch_size: int) -> CompactDecodeGraph:

@@ -135,6 +135,7 @@ class LFM25Engine:
                "max_model_len cannot exceed config.max_position_embeddings")
         self._scaling = cfg.head_dim ** -0.5
         self._cuda_decoder = None
+        self._step_probe = None   # measurement hook of the decode step, see LFM25HIPDecoder.capture_probed_step
         self.policy_version = 0
         self.last_prefill: dict = {}   # chunk count, tokens and fill of the latest prefill() call
         # fp32 rotary tables [max_model_len, D/2] (lfm25_engine.py:1004-1012)
@@ -351,6 +352,18 @@ class LFM25Engine:
             schedule = ops.decode_schedule(positions, active, slot_ids, capacity=cache.max_seq_len)
             advance_after = True
 
+        probe = self._step_probe
+
+        def attend(i, q, k_scales, v_scales, quantized):
+            # `probe(kind, index, phase)`, when a measurement asks for it, brackets the call on the launch stream
+            if probe is not None:
+                probe("attention", i, 0)
+            out = ops.attend(q, cache.k_cache[i], cache.v_cache[i], k_scales, v_scales, positions, active=active,
+                             scale=self._scaling, slot_ids=slot_ids, schedule=schedule, quantized=quantized)
+            if probe is not None:
+                probe("attention", i, 1)
+            return out
+
         def attention_op(op, qkv):
             # QK norm + RoPE with the new token's keys and values written straight into the cache, then attention over
             # [0, position]; rows come back already quantised when the out projection is W8A8
@@ -363,8 +376,7 @@ class LFM25Engine:
                                       slot_ids=slot_ids)
             quantized = (id(op.out_weight) in fp8
                          and -(-cfg.num_attention_heads // 16) * -(-cfg.head_dim // 64) <= 4)  # the fused combine's row limit
-            out = ops.attend(q, cache.k_cache[i], cache.v_cache[i], k_scales, v_scales, positions, active=active,
-                             scale=self._scaling, slot_ids=slot_ids, schedule=schedule, quantized=quantized)
+            out = attend(i, q, k_scales, v_scales, quantized)
             return out if quantized else out.view(rows, -1)
 
         def conv_op(op, bcx):
@@ -385,8 +397,7 @@ class LFM25Engine:
                                       active=active, slot_ids=slot_ids)
             quantized = (id(op.out_weight) in fp8
                          and -(-cfg.num_attention_heads // 16) * -(-cfg.head_dim // 64) <= 4)
-            out = ops.attend(q, cache.k_cache[i], cache.v_cache[i], k_scales, v_scales, positions, active=active,
-                             scale=self._scaling, slot_ids=slot_ids, schedule=schedule, quantized=quantized)
+            out = attend(i, q, k_scales, v_scales, quantized)
             return out if quantized else out.view(rows, -1)
 
         def projecting_conv_op(op, normed):

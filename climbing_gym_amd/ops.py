@@ -674,3 +674,26 @@ def record_head(ids, probs, out_ids, out_probs, lengths, alive, k: int, cap: int
     """lfm25_session.py:22-31."""
     call("lfm2_record_head", ids.contiguous(), probs.contiguous(), out_ids, out_probs, lengths, alive, int(k),
          int(cap), lengths.numel())
+
+
+# ----------------------------------------------------------------------------------- measurement
+def hbm_stream_read(buffer: torch.Tensor, sink: torch.Tensor, *, workgroups: int, layout: int = 0) -> int:
+    """Launch the loads-only streaming read of `buffer` (`lfm2_hbm_stream_read`); returns the bytes the launch reads.
+    `sink` is an int32 tensor of at least workgroups * 256 entries."""
+    reject(not buffer.is_cuda or not buffer.is_contiguous() or not sink.is_cuda or sink.dtype != torch.int32
+           or sink.numel() < workgroups * 256, "hbm_stream_read needs a contiguous GPU buffer and an int32 sink of workgroups * 256")
+    size = buffer.numel() * buffer.element_size()
+    call("lfm2_hbm_stream_read", buffer, size, sink, int(workgroups), int(layout))
+    return (size // 4096 // workgroups) * workgroups * 4096
+
+
+def timestamp(out: torch.Tensor) -> None:
+    """Store the device wall clock into the int64 element `out` points at, in stream order (`lfm2_timestamp`)."""
+    reject(not out.is_cuda or out.dtype != torch.int64 or out.numel() < 1, "timestamp needs an int64 GPU element")
+    call("lfm2_timestamp", out)
+
+
+def timestamp_rate_hz() -> float:
+    rate = query("lfm2_timestamp_rate_khz")
+    reject(rate <= 0, "the device's wall-clock rate cannot be read", RuntimeError)
+    return rate * 1000.0

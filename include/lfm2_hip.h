@@ -342,6 +342,24 @@ int lfm2_configure_rows(const int64_t* specs, int64_t count, int64_t rows, int32
 int lfm2_record_head(const int64_t* ids, const float* probs, int32_t* out_ids, float* out_probs,
                      const int32_t* lengths, const uint8_t* alive, int K, int64_t cap, int64_t B, void* stream);
 
+/* ---------------------------------------------------------------- measurement */
+
+/* Loads-only streaming read of `bytes` bytes at src (16-byte aligned) by `workgroups` workgroups of 256 lanes, eight
+ * 16-byte loads in flight per lane: the read rate the chip delivers to CUs that do nothing else, which bench.py
+ * reports as the measured ceiling next to the nominal HBM peak.  No counterpart in the reference (its harness,
+ * inference/benchmark.py:111-139, reports wall-clock phases only).  layout 0: every workgroup reads a private
+ * contiguous region of floor(bytes / 4096 / workgroups) blocks of 4 KiB; layout 1: the grid sweeps the buffer together.
+ * sink: int32[workgroups * 256], receives one folded word per lane.  Bytes read = workgroups * that many blocks * 4096. */
+int lfm2_hbm_stream_read(const void* src, int64_t bytes, int32_t* sink, int workgroups, int layout, void* stream);
+
+/* Stores the device's constant-rate wall clock into out[0] from a one-lane kernel; lfm2_timestamp_rate_khz() is the
+ * clock's rate (0 if it cannot be read).  Recorded into a graph before and after a kernel, two stamps give that
+ * kernel's time inside the replayed graph, which is how bench.py reads the decode-attention call's time inside the
+ * decode step (the reference reads per-phase CUDA events, lfm25_session.py:184-204; event-record nodes are not
+ * available to graphs captured through PyTorch on ROCm). */
+int lfm2_timestamp(int64_t* out, void* stream);
+int64_t lfm2_timestamp_rate_khz(void);
+
 #ifdef __cplusplus
 }
 #endif
