@@ -393,7 +393,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
           tc = tc < wend ? tc : wend - 1;
           t.k[c] = *reinterpret_cast<const i32x4*>(kbase + token_offset(b, slot, h, tc) + 16 * (lane & 3));
         } else {
-          t.k[c] = *reinterpret_cast<const i32x4*>(kbase + koff * ES + krow_byte + 16 * c);
+          int tc = T + 8 * c + (lane >> 3);
+          tc = tc < wend ? tc : wend - 1;
+          t.k[c] = *reinterpret_cast<const i32x4*>(kbase + token_offset(b, slot, h, tc) * ES + 16 * (lane & 7));
         }
       }
       if constexpr (FP8) {
@@ -424,8 +426,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
           int tc = T + 16 * c + (lane >> 2);
           tc = tc < wend ? tc : wend - 1;
           t.k[c] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(kitem + (uint32_t)tc * row_bytes + 16 * (lane & 3)));
-        } else {
-          t.k[c] = *reinterpret_cast<const i32x4*>(kitem + koff + 16 * c);
+        } else {   // 16-bit rows: load c brings lane L the eighth L % 8 of the 128-byte row of token 8c + L / 8
+          int tc = T + 8 * c + (lane >> 3);
+          tc = tc < wend ? tc : wend - 1;
+          t.k[c] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(kitem + (uint32_t)tc * row_bytes + 16 * (lane & 7)));
         }
       }
       if constexpr (FP8) {
@@ -510,7 +514,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
       acc = f32x4{0.f, 0.f, 0.f, 0.f};
     }
     // ---- the next tile of the stream: this item's, or the first of the next item (its record was asked for one
-    // item ago); without a next item, the current tile again (a cache hit)
+    // item ago)
     const bool last = T + kStride >= wend;
     int nb = b, nlen = len, nh = h, nwbeg = wbeg, nwend = wend;
     int64_t nslot = slot;
@@ -521,7 +525,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
       nwend = nwbeg + chunk_tokens;
       nwend = nwend < nlen ? nwend : nlen;
     }
-    const int fT = last ? (have_next ? nwbeg : T) : T + kStride;
+    // (without a next item the fetch still has to be issued: every lane then asks for the item's last token, one
+    // line per operand; the whole last tile again would be fetched from memory a second time, since non-temporal
+    // loads leave nothing behind in the caches)
+    const int fT = last ? (have_next ? nwbeg : nwend - 1) : T + kStride;
     fetch(nb, nslot, nh, fT, nwend, nxt);
 
     const bool valid = T + tl < wend;
@@ -534,11 +541,18 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))
       // 16-bit history: a lane's K registers hold dims 32 (lane / 32) + 8c .. + 7; the two halves of the wave each
       // sum over their 32 dims and exchange the sums
       const __bf16* qrow = &lds_q[wave][g][32 * (lane >> 5)];
+      // the K row eighths go to LDS as they arrived and come back as half rows (the wave's V buffer; the V rows are
+      // stored after these reads).  The 16-byte column of a row is XORed with bits 1..3 of its token: the 16 stores
+      // and the 16 loads that share a cycle then fall on distinct banks.
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        *reinterpret_cast<i32x4*>(&lds_v[wave][8 * c + (lane >> 3)][16 * ((lane & 7) ^ (((8 * c + (lane >> 3)) >> 1) & 7))]) = cur.k[c];
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
+        const i32x4 kr = *reinterpret_cast<const i32x4*>(&lds_v[wave][tl][16 * ((4 * (lane >> 5) + c) ^ ((tl >> 1) & 7))]);
         const i32x4 q8 = *reinterpret_cast<const i32x4*>(qrow + 8 * c);
         const i32x2 qa = {q8[0], q8[1]}, qb = {q8[2], q8[3]};
-        const i32x2 ka = {cur.k[c][0], cur.k[c][1]}, kb = {cur.k[c][2], cur.k[c][3]};
+        const i32x2 ka = {kr[0], kr[1]}, kb = {kr[2], kr[3]};
         s = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, qa), __builtin_bit_cast(s16x4, ka), s, 0, 0, 0);
         s = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, qb), __builtin_bit_cast(s16x4, kb), s, 0, 0, 0);
       }
