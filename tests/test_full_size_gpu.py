@@ -284,6 +284,41 @@ def test_all_bf16_session_at_256_sequences_graph_equals_eager_and_repeats(big_mo
 
 
 @torch.inference_mode()
+def test_all_bf16_session_as_the_workload_is_worded_graph_equals_eager_and_repeats(big_model):
+    """The all-bf16 workload as it is worded: 256 concurrent sequences with prompts uniform in [256, 2048], a context
+    capacity of 8192, max-prefill-tokens 4096, temperature 1, bf16 linears and a bf16 KV cache (25.8 GB of history).
+    A few decode steps: the captured step equals the step launched kernel by kernel, a second run repeats it, and
+    the rows' first tokens are draws from an independent prefill's logits."""
+    engine, ocfg, _ = big_model
+    from climbing_gym_amd.config import LFM25SamplingConfig
+    g = torch.Generator().manual_seed(18)
+    prompts = [torch.randint(0, ocfg.vocab_size, (int(n),), generator=g).tolist() for n in torch.randint(256, 2049, (256,), generator=g)]
+    sampling = [LFM25SamplingConfig(temperature=1.0, seed=800 + i, max_new_tokens=4, ignore_eos=True) for i in range(256)]
+
+    def run(capture):
+        engine.enable_cuda_graphs(max_graphs=1, max_prefill_tokens=4096, capture=capture)
+        with engine.generation_session(max_batch_size=256, max_new_tokens=4, cache_len=8192) as session:
+            assert not session.entry.cache.fp8 and session.entry.cache.max_seq_len == 8192
+            assert session.entry.cache.k_cache.dtype == torch.bfloat16
+            session.admit(prompts, sampling)
+            results = sorted(session.poll(steps=5), key=lambda r: r.handle.slot)
+            stats = dict(session.stats)
+        engine.disable_cuda_graphs()
+        torch.cuda.empty_cache()
+        return results, stats
+
+    graph, stats = run(True)
+    eager, _ = run(False)
+    again, _ = run(True)
+    assert len(graph) == 256 and stats["decode_batches"] == {"256": 5}
+    assert sum(len(r.prompt_token_ids) for r in graph) == sum(map(len, prompts))
+    for a, b, c in zip(graph, eager, again):
+        assert a.token_ids == b.token_ids == c.token_ids and len(a.token_ids) == 4 and a.finish_reason == 3
+        assert a.logprobs == b.logprobs == c.logprobs
+    assert len({r.token_ids for r in graph}) > 200          # rows decode their own histories
+
+
+@torch.inference_mode()
 def test_filtered_sampling_session_at_512_sequences_is_repeatable_and_stays_in_support(big_model):
     """Config 5: FP8 everywhere, 512 concurrent ragged sequences (prompts uniform in [512, 4096]), top-k 50 /
     top-p 0.95 at temperature 1 with fixed seeds, sequences admitted and retired as they finish."""
@@ -325,3 +360,39 @@ def test_filtered_sampling_session_at_512_sequences_is_repeatable_and_stays_in_s
     key = lambda r: (r.prompt_token_ids[:8], r.token_ids)
     assert sorted(map(key, results_a)) == sorted(map(key, results_b))  # same seeds, same tokens
     assert all(0 <= t < ocfg.vocab_size for r in results_a for t in r.token_ids)
+
+
+@torch.inference_mode()
+def test_filtered_draws_at_512_sequences_stay_inside_the_top_k_and_the_nucleus(big_model):
+    """Config 5's sampler inside the session: after each single-step poll the session's logits buffer still holds the
+    logits the step's tokens were drawn from.  Every drawn token must be one of its row's 50 largest logits (by value:
+    bf16 logits tie) and lie inside the 0.95 nucleus of those, the survivors taken from the filter of
+    lfm25_engine.py:1759-1774 evaluated in float64; a row is exempt from the nucleus check only where one rank's
+    cumulative mass lies within 2e-6 of 0.95.  Every eighth row, three steps."""
+    engine, ocfg, _ = big_model
+    from climbing_gym_amd.config import LFM25SamplingConfig
+    g = torch.Generator().manual_seed(17)
+    prompts = [torch.randint(0, ocfg.vocab_size, (int(n),), generator=g).tolist() for n in torch.randint(64, 513, (512,), generator=g)]
+    sampling = [LFM25SamplingConfig(temperature=1.0, top_k=50, top_p=0.95, seed=7000 + i, max_new_tokens=8, ignore_eos=True)
+                for i in range(512)]
+    engine.enable_cuda_graphs(max_graphs=1, max_prefill_tokens=4096, fp8_mlp=True, fp8_kv=True, fp8_lm_head=True, fp8_operators=True)
+    checked = 0
+    with engine.generation_session(max_batch_size=512, max_new_tokens=8, cache_len=1024) as session:
+        session.admit(prompts, sampling)
+        for step in range(3):
+            assert session.poll(steps=1) == []
+            rows = torch.arange(step, 512, 8, device=DEV)
+            logits = session.entry.logits[rows].double().cpu()
+            drawn = session.rows.tokens[rows, step].cpu()
+            value = logits.gather(1, drawn[:, None])[:, 0]
+            ranked = logits.sort(descending=True, dim=-1).values
+            assert (value >= ranked[:, 49]).all(), "a draw fell outside the 50 largest logits"
+            kept = O.top_k_top_p_filter(logits, 50, 0.95)
+            floor = torch.where(torch.isfinite(kept), logits, torch.full_like(logits, float("inf"))).amin(1)
+            head = torch.softmax(O.top_k_top_p_filter(logits, 50, 1.0).sort(descending=True, dim=-1).values[:, :64], -1).cumsum(-1)
+            clear = (head - 0.95).abs().amin(1) > 2e-6
+            assert (value >= floor)[clear].all(), "a draw fell outside the nucleus"
+            assert (torch.isfinite(kept).sum(1) < 50).any()      # the nucleus does cut rows of this model
+            checked += int(clear.sum())
+    engine.disable_cuda_graphs()
+    assert checked >= 180
