@@ -676,8 +676,193 @@ gemm_naive_kernel(void* out, const uint8_t* A, const uint8_t* W, const float* a_
   store_out(out, out_dtype, (int64_t)m_out * N + n, t);
 }
 
+// ------------------------------------------------------------------------------------ few rows: everything in flight at once
+// Up to 64 rows the tiled kernels are a serial chain: a workgroup walks its K loop step by step behind a ring a few
+// steps deep, so a launch lasts several memory latencies whatever the shape (6.5-7.5 us for every K = 2048 projection
+// at 1-16 rows, on 32-176 workgroups of a 256-CU chip).  This kernel has no K loop.  A workgroup owns 16 NI output
+// columns (weight rows) and all rows of the batch; its waves split K among themselves, 128-byte steps dealt round
+// robin, and every wave loads ALL of its operand fragments straight into registers in the MFMA's own layout (lane
+// l: row l % 16, bytes 32 (l / 16) .. + 31 of a step: no staging through LDS, no barrier before the MFMAs), one memory
+// latency deep.  The waves' partial tiles meet in LDS and are summed in wave order.  N / (16 NI) workgroups, times the
+// parts of K when the product is left as partial sums for the norm that follows it.
+//   EPI 0: out[m, n] = (acc * a_scale[m]) * w_scale[n] with optional row placement; EPI 2: SwiGLU over interleaved
+//   gate/up weight rows as in the tiled kernel's epilogue, out [M, N / 2]; EPI 4: fp32 partial sums of this
+//   workgroup's part of K, partial[blockIdx.y][m][n].
+template <int MI, int NI, int WAVES, int MAXS, int EPI>
+__global__ void __launch_bounds__(WAVES * 64)
+gemm_skinny_kernel(void* __restrict__ out, const uint8_t* __restrict__ A, const uint8_t* __restrict__ W,
+                   const float* __restrict__ a_scales, const float* __restrict__ w_scales, int M, int N, int64_t Kb,
+                   int steps_per_part, int out_dtype, RowMap rows) {
+  typedef StepMfma<1>::frag frag;
+  __shared__ f32x4 red[WAVES][MI * NI][64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lrow = lane & 15, lgrp = lane >> 4;
+  const int n_base = blockIdx.x * (16 * NI);
+  const int step0 = blockIdx.y * steps_per_part;
+  int nsteps = (int)(Kb / kStepBytes) - step0;
+  nsteps = nsteps < steps_per_part ? nsteps : steps_per_part;
+  const uint8_t* wp[NI];
+#pragma unroll
+  for (int j = 0; j < NI; ++j) {
+    int n = n_base + 16 * j + lrow;
+    n = n < N ? n : N - 1;
+    wp[j] = W + (int64_t)(EPI == 2 ? swiglu_weight_row(n, N) : n) * Kb + 32 * lgrp;
+  }
+  const uint8_t* ap[MI];
+#pragma unroll
+  for (int i = 0; i < MI; ++i) {
+    int m = i * 16 + lrow;
+    m = m < M ? m : M - 1;
+    ap[i] = A + (int64_t)m * Kb + 32 * lgrp;
+  }
+  // every load of the wave, unconditionally (a step beyond the last is the last one again and is not multiplied)
+  frag fw[MAXS][NI], fa[MAXS][MI];
+#pragma unroll
+  for (int t = 0; t < MAXS; ++t) {
+    int step = wave + t * WAVES;
+    step = step < nsteps ? step : nsteps - 1;
+    const int64_t kb = (int64_t)(step0 + step) * kStepBytes;
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const i32x4 lo = *reinterpret_cast<const i32x4*>(wp[j] + kb), hi = *reinterpret_cast<const i32x4*>(wp[j] + kb + 16);
+      fw[t][j] = frag{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+      const i32x4 lo = *reinterpret_cast<const i32x4*>(ap[i] + kb), hi = *reinterpret_cast<const i32x4*>(ap[i] + kb + 16);
+      fa[t][i] = frag{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
+  }
+  f32x4 acc[MI][NI];
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < NI; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int t = 0; t < MAXS; ++t) {
+    if (wave + t * WAVES < nsteps) {   // the same for the whole wave
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) acc[i][j] = StepMfma<1>::run(fw[t][j], fa[t][i], acc[i][j]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < NI; ++j) red[wave][i * NI + j][lane] = acc[i][j];
+  __syncthreads();
+  // item (i, j, l) finishes out[m = 16 i + l % 16][n = n_base + 16 j + 4 (l / 16) + r]: the waves' partial sums in wave order
+  auto total = [&](int tile, int l) {
+    f32x4 v = red[0][tile][l];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) v += red[w][tile][l];
+    return v;
+  };
+  for (int item = tid; item < MI * NI * 64; item += WAVES * 64) {
+    const int tile = item >> 6, l = item & 63, i = tile / NI, j = tile % NI;
+    const int m = i * 16 + (l & 15), grp = l >> 4;
+    if (m >= M) continue;
+    const int col = n_base + 16 * j + 4 * grp;
+    if (col >= N) continue;
+    if constexpr (EPI == 4) {
+      *reinterpret_cast<f32x4*>((float*)out + ((int64_t)blockIdx.y * M + m) * N + col) = total(tile, l);
+      continue;
+    }
+    const float sa = a_scales[m];
+    if constexpr (EPI == 2) {
+      // lane groups 0, 1 hold gate columns 0-7 of a tile, groups 2, 3 (32 lanes on) the up columns that pair with them
+      if (l >= 32) continue;
+      const f32x4 gate = total(tile, l), up = total(tile, l + 32);
+      auto finish = [&](auto tag) {
+        typedef decltype(tag) T;
+        float h[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float g = round_to<T>((gate[r] * sa) * w_scales[swiglu_weight_row(col + r, N)]);
+          const float u = round_to<T>((up[r] * sa) * w_scales[swiglu_weight_row(col + 8 + r, N)]);
+          h[r] = round_to<T>(round_to<T>(silu_f(g)) * u);
+        }
+        T* dst = (T*)out + (int64_t)m * (N >> 1) + ((n_base + 16 * j) >> 1) + 4 * grp;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) dst[r] = Elem<T>::store(h[r]);
+      };
+      if (out_dtype == LFM2_DTYPE_BF16) finish(__bf16{});
+      else if (out_dtype == LFM2_DTYPE_F16) finish(_Float16{});
+      else finish(float{});
+      continue;
+    }
+    const int m_out = mapped_row(rows, m);
+    if (m_out < 0) continue;
+    f32x4 v = total(tile, l);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) v[r] = (v[r] * sa) * w_scales[col + r];
+    const int64_t idx = (int64_t)m_out * N + col;
+    if (out_dtype == LFM2_DTYPE_BF16) {
+      bf16x4 o = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
+      *reinterpret_cast<bf16x4*>((__bf16*)out + idx) = o;
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) store_out(out, out_dtype, idx + r, v[r]);
+    }
+  }
+}
+
+// Whether the few-row kernel serves an e4m3 product: whole 128-byte steps, whole 16-column tiles, at most 64 rows, and
+// few enough steps per wave that all of a wave's fragments fit in its registers (16 waves share the steps of a long
+// K).  `parts` > 1: the product is left as that many partial sums along K (one workgroup row per part).
+constexpr int kSkinnyTile = 60;
+struct SkinnyShape { int mi, ni, waves, maxs, per_part; };
+bool skinny_shape(int64_t M, int64_t N, int64_t Kb, int parts, SkinnyShape* shape) {
+  if (M <= 0 || M > 64 || N <= 0 || N % 16 != 0 || Kb % kStepBytes != 0 || Kb < kStepBytes || parts < 1) return false;
+  const int steps = (int)(Kb / kStepBytes), mi = (int)((M + 15) / 16);
+  if (steps < parts) return false;
+  const int per_part = (steps + parts - 1) / parts;
+  if ((int64_t)per_part * (parts - 1) >= steps) return false;   // a part without a step
+  const int waves = per_part > 16 ? 16 : 8;
+  const int maxs = (per_part + waves - 1) / waves;
+  if (maxs > 4) return false;
+  // Where it wins (weights streamed from HBM, launches replayed in a graph, us per launch against the tiled plan):
+  // N 2048 and 3072, K 2048: 4.1-4.8 against 6.2-6.4 at 1-16 rows, 5.8 against 7.2 at 32, level at 48-64; N 6144:
+  // 5.6-6.4 against 7.0-7.2 at 1-16 rows, 7.2 against 7.9 at 32, behind from 48 on; N 11264: behind everywhere (the
+  // tiled kernel is already at the 23 MB's streaming time); K 5632 whole: 6.9-7.5 against 8.1-8.3 at 1-8 rows, level at 16.
+  const int64_t row_limit = steps <= 16 ? (N <= 4096 ? 48 : N <= 8192 ? 32 : 0) : (parts > 1 ? 32 : N <= 4096 ? 8 : 0);
+  if (M > row_limit) return false;
+  // wide outputs on few rows: several column tiles per workgroup, while at least 128 workgroups remain (every workgroup
+  // reads all of the activations, so fewer of them re-read less)
+  int ni = 1;
+  if (parts == 1 && waves == 8 && mi <= 2) ni = N % 64 == 0 && N / 64 >= 128 ? 4 : N % 32 == 0 && N / 32 >= 128 ? 2 : 1;
+  // registers a lane holds in flight: 8 per weight fragment and 8 per activation fragment of every step
+  if (maxs * (8 * ni + 8 * mi) + 4 * mi * ni > (waves == 16 ? 104 : 200)) return false;
+  if (shape) *shape = SkinnyShape{mi, ni, waves, maxs, per_part};
+  return true;
+}
+
+template <int EPI>
+bool launch_skinny(void* out, const uint8_t* A, const uint8_t* W, const float* as, const float* ws, int64_t M, int64_t N,
+                   int64_t Kb, int parts, int out_dtype, RowMap rows, hipStream_t s) {
+  SkinnyShape shape;
+  if (!skinny_shape(M, N, Kb, parts, &shape)) return false;
+  const dim3 grid((unsigned)(N / (16 * shape.ni)), (unsigned)parts);
+#define SKINNY_(MI, NI, WAVES, MAXS)                                                                                    \
+  if (shape.mi == MI && shape.ni == NI && shape.waves == WAVES && shape.maxs == MAXS) {                                 \
+    hipLaunchKernelGGL((gemm_skinny_kernel<MI, NI, WAVES, MAXS, EPI>), grid, dim3(WAVES * 64), 0, s, out, A, W, as, ws, \
+                       (int)M, (int)N, Kb, shape.per_part, out_dtype, rows);                                            \
+    return true;                                                                                                        \
+  }
+#define SKINNY_ROWS_(WAVES, MAXS) SKINNY_(1, 1, WAVES, MAXS) SKINNY_(2, 1, WAVES, MAXS) SKINNY_(3, 1, WAVES, MAXS) SKINNY_(4, 1, WAVES, MAXS)
+  SKINNY_ROWS_(8, 1) SKINNY_ROWS_(8, 2) SKINNY_ROWS_(16, 2) SKINNY_ROWS_(16, 3) SKINNY_ROWS_(16, 4)
+  if constexpr (EPI != 4) {
+    SKINNY_(1, 2, 8, 1) SKINNY_(2, 2, 8, 1) SKINNY_(1, 4, 8, 1) SKINNY_(2, 4, 8, 1)
+    SKINNY_(1, 2, 8, 2) SKINNY_(2, 2, 8, 2) SKINNY_(1, 4, 8, 2) SKINNY_(2, 4, 8, 2)
+  }
+#undef SKINNY_ROWS_
+#undef SKINNY_
+  return false;
+}
+
 struct TileInfo { int bm, bn, ks; };
-constexpr int kNumTiles = 60;
+constexpr int kNumTiles = 61;
 constexpr TileInfo kTiles[kNumTiles] = {{16, 64, 128}, {32, 64, 128}, {64, 64, 128}, {128, 64, 128}, {128, 128, 128},
                                         {64, 128, 128}, {128, 128, 128}, {64, 128, 128}, {128, 64, 128},
                                         {16, 64, 256}, {32, 64, 256}, {64, 64, 256},
@@ -693,7 +878,8 @@ constexpr TileInfo kTiles[kNumTiles] = {{16, 64, 128}, {32, 64, 128}, {64, 64, 1
                                         {32, 64, 128}, {32, 64, 256}, {32, 64, 256}, {64, 64, 256},
                                         {256, 48, 128}, {256, 48, 128}, {256, 32, 128}, {256, 64, 128}, {256, 48, 128},
                                         {256, 32, 128},
-                                        {256, 128, 128}, {128, 256, 128}, {256, 256, 128}, {128, 128, 128}};
+                                        {256, 128, 128}, {128, 256, 128}, {256, 256, 128}, {128, 128, 128},
+                                        {64, 16, 128}};   // 60: the few-row kernel (all rows, 16 columns)
 int64_t tile_steps(int tile, int64_t Kb) { return (Kb + kTiles[tile].ks - 1) / kTiles[tile].ks; }
 
 struct Plan { int tile, splits; };
@@ -703,7 +889,13 @@ struct Plan { int tile, splits; };
 // once it alone fills the 256 CUs (1.3-2.0 PFLOP/s at M = 4096; 42 us for the 65536-row head at M = 256), otherwise
 // smaller tiles with deeper rings the fewer workgroups a CU gets (its K loop is then a serial chain that nothing
 // overlaps).  With K bytes not a multiple of the step these indices run their register-staged twins.
-Plan default_plan(int64_t M, int64_t N, int64_t Kb, bool deferred = false) {
+Plan default_plan(int64_t M, int64_t N, int64_t Kb, bool deferred = false, int eb = 2) {
+  if (eb == 1 && skinny_shape(M, N, Kb, 1, nullptr)) {
+    // a long K on a narrow output whose partial sums the next norm adds up anyway (the down projection of a small decode
+    // batch: 44 steps on 128 column tiles): two parts of K, 256 workgroups
+    if (deferred && Kb / kStepBytes >= 32 && N / 16 <= 128 && skinny_shape(M, N, Kb, 2, nullptr)) return {kSkinnyTile, 2};
+    return {kSkinnyTile, 1};
+  }
   auto count = [&](int t) { return ((M + kTiles[t].bm - 1) / kTiles[t].bm) * ((N + kTiles[t].bn - 1) / kTiles[t].bn); };
   const int64_t steps = (Kb + kStepBytes - 1) / kStepBytes;
   // Few output tiles on a K loop of 32 steps or more: split K (2 or 4 ways) while every part keeps 8 steps and the
@@ -813,10 +1005,26 @@ int gemm_entry(const char* name, void* out, const void* a, const float* as, cons
     hipLaunchKernelGGL(gemm_naive_kernel<EB>, dim3(ceil_div(M * N, 256)), dim3(256), 0, s, out, A, W, as, ws, M, N, K, out_dtype, rows);
     LFM2_LAUNCH_CHECK();
   }
-  Plan plan = default_plan(M, N, Kb, !reduce);
+  // the few-row kernel finishes its product itself: it serves the default plan of a product that is neither split on
+  // request nor left as partial sums
+  // the few-row kernel finishes its product itself, or leaves it as the partial sums of its own plan: it serves the
+  // default plan of a product that is not split on request
+  Plan plan = default_plan(M, N, Kb, !reduce, (tile < 0 && (reduce ? split_k <= 1 : true)) ? EB : 2);
+  if (!reduce && tile < 0 && plan.tile == kSkinnyTile && split_k > 0 && split_k != plan.splits)
+    plan = default_plan(M, N, Kb, true, 2);   // another number of parts than the few-row plan's: the tiled kernels
   if (tile >= 0) {
     LFM2_REQUIRE(tile < kNumTiles, "%s: tile index %d out of range", name, tile);
     plan.tile = tile;
+  }
+  if (plan.tile == kSkinnyTile) {
+    LFM2_REQUIRE(EB == 1, "%s: the few-row kernel takes e4m3 operands", name);
+    const int parts = reduce ? 1 : (split_k > 0 ? split_k : plan.splits);
+    LFM2_REQUIRE(!reduce || split_k <= 1, "%s: the few-row kernel splits K only for partial sums", name);
+    const bool ok = reduce ? launch_skinny<0>(out, A, W, as, ws, M, N, Kb, 1, out_dtype, rows, s)
+                           : launch_skinny<4>(workspace, A, W, as, ws, M, N, Kb, parts, LFM2_DTYPE_F32, rows, s);
+    if (ok) LFM2_LAUNCH_CHECK();
+    LFM2_FAIL(LFM2_ERR_UNSUPPORTED, "%s: the few-row kernel does not cover M %ld, N %ld, K bytes %ld in %d parts", name,
+              (long)M, (long)N, (long)Kb, parts);
   }
   if (split_k > 0) plan.splits = split_k;
   else if (rows.slots || rows.active) plan.splits = 1;   // placed rows are written by the product itself
@@ -910,10 +1118,10 @@ extern "C" int lfm2_fp8_gemm(void* out, const uint8_t* a_q, const float* a_scale
 
 namespace {
 // The fused form exists for the tile the default plan takes at large M; other shapes use the two launches.
-bool swiglu_fits(int64_t M, int64_t N, int64_t Kb) {
+bool swiglu_fits(int64_t M, int64_t N, int64_t Kb, int eb) {
   if (M <= 0 || N <= 0 || Kb <= 0 || N % 16 != 0 || Kb % kStepBytes != 0 || M >= (1 << 30) || N >= (1 << 30)) return false;
-  const Plan plan = default_plan(M, N, Kb);
-  return (plan.tile == 14 || plan.tile == 36 || plan.tile == 56) && plan.splits == 1;
+  const Plan plan = default_plan(M, N, Kb, false, eb);
+  return (plan.tile == 14 || plan.tile == 36 || plan.tile == 56 || plan.tile == kSkinnyTile) && plan.splits == 1;
 }
 template <int EB>
 int swiglu_entry(const char* name, void* out, const void* a, const float* as, const void* w, const float* ws, int64_t M,
@@ -921,8 +1129,13 @@ int swiglu_entry(const char* name, void* out, const void* a, const float* as, co
   LFM2_REQUIRE(out && a && w, "%s: a required pointer is null", name);
   LFM2_REQUIRE(out_dtype >= LFM2_DTYPE_BF16 && out_dtype <= LFM2_DTYPE_F32, "%s: bad output dtype", name);
   LFM2_REQUIRE(((uintptr_t)a | (uintptr_t)w | (uintptr_t)out) % 16 == 0, "%s: pointers must be aligned to 16 bytes", name);
-  if (!swiglu_fits(M, N, K * EB)) LFM2_FAIL(LFM2_ERR_UNSUPPORTED, "%s: no fused form for M %ld, N %ld, K %ld", name, (long)M, (long)N, (long)K);
-  const int tile = default_plan(M, N, K * EB).tile;
+  if (!swiglu_fits(M, N, K * EB, EB)) LFM2_FAIL(LFM2_ERR_UNSUPPORTED, "%s: no fused form for M %ld, N %ld, K %ld", name, (long)M, (long)N, (long)K);
+  const int tile = default_plan(M, N, K * EB, false, EB).tile;
+  if (tile == kSkinnyTile) {
+    launch_skinny<2>(out, (const uint8_t*)a, (const uint8_t*)w, as, ws, M, N, K * EB, 1, out_dtype,
+                     RowMap{nullptr, nullptr, 0x7fffffff}, (hipStream_t)stream);
+    LFM2_LAUNCH_CHECK();
+  }
   const int tiles = (int)(((M + kTiles[tile].bm - 1) / kTiles[tile].bm) * ((N + kTiles[tile].bn - 1) / kTiles[tile].bn));
   const dim3 grid((tiles + 7) / 8 * 8);
   if (tile == 14)
@@ -982,7 +1195,7 @@ extern "C" int lfm2_bf16_gemm_conv_update(void* out, const void* x, const void* 
 }
 
 extern "C" int lfm2_gemm_swiglu_fits(int64_t M, int64_t N, int64_t K, int element_bytes) {
-  return (element_bytes == 1 || element_bytes == 2) && swiglu_fits(M, N, K * element_bytes) ? 1 : 0;
+  return (element_bytes == 1 || element_bytes == 2) && swiglu_fits(M, N, K * element_bytes, element_bytes) ? 1 : 0;
 }
 
 extern "C" int lfm2_fp8_gemm_swiglu(void* out, const uint8_t* a_q, const float* a_scales, const uint8_t* w_q,
@@ -1027,7 +1240,7 @@ extern "C" int lfm2_fp8_gemm_partials(float* partials, const uint8_t* a_q, const
                                       int64_t K, int tile, int split_k, void* stream) {
   LFM2_REQUIRE(split_k >= 1 && split_k <= 16, "fp8_gemm_partials: split_k %d not in [1,16]", split_k);
   LFM2_REQUIRE(tile < kNumTiles, "fp8_gemm_partials: tile index %d out of range", tile);
-  const int64_t steps = tile_steps(tile >= 0 ? tile : default_plan(M, N, K, true).tile, K);
+  const int64_t steps = tile_steps(tile >= 0 ? tile : default_plan(M, N, K, true, 1).tile, K);
   LFM2_REQUIRE(split_k <= steps && (steps + split_k - 1) / split_k * (split_k - 1) < steps,
                "fp8_gemm_partials: %d splits leave one without a K step", split_k);
   return gemm_entry<1>("fp8_gemm_partials", nullptr, a_q, nullptr, w_q, nullptr, partials, M, N, K, LFM2_DTYPE_F32, tile,
@@ -1035,11 +1248,11 @@ extern "C" int lfm2_fp8_gemm_partials(float* partials, const uint8_t* a_q, const
 }
 
 extern "C" int64_t lfm2_fp8_gemm_default_splits(int64_t M, int64_t N, int64_t K) {
-  return K % 16 == 0 ? default_plan(M, N, K, true).splits : 1;
+  return K % 16 == 0 ? default_plan(M, N, K, true, 1).splits : 1;
 }
 
 extern "C" int64_t lfm2_fp8_gemm_workspace(int64_t M, int64_t N, int64_t K) {
-  const Plan p = default_plan(M, N, K);
+  const Plan p = default_plan(M, N, K, false, 1);
   return (K % 16 == 0 && p.splits > 1) ? (int64_t)p.splits * M * N : 0;
 }
 

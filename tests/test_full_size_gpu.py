@@ -48,12 +48,18 @@ def test_fp8_projection_at_benchmark_shapes_matches_dequantised_product_on_sampl
 
 @pytest.mark.parametrize("k,n,row_counts", [(2048, 11264, (129, 200, 255, 257, 300, 512, 513)),
                                             (2048, 6144, (129, 200, 255, 257, 300, 512, 513)),
-                                            (2048, 65536, (192, 193, 256, 300, 512, 513))])
+                                            (2048, 65536, (192, 193, 256, 300, 512, 513)),
+                                            (2048, 2048, (1, 15, 16, 17, 31, 33, 48, 49, 64)),
+                                            (2048, 3072, (2, 16, 47, 48, 49)), (2048, 6144, (1, 16, 17, 32, 33)),
+                                            (5632, 2048, (1, 8, 9, 16, 32, 33))])
 @torch.inference_mode()
 def test_fp8_projection_at_row_counts_where_the_tile_plan_changes(ops, k, n, row_counts):
     """Ragged row counts on either side of every rule of the default plan for the wide projections (one tile per CU at
-    129-256 and 257-512 rows, the 256 x 256 tile of the vocabulary projection at 193-512 rows): first, last and sampled
-    rows against the dequantised float64 product, every column of those rows."""
+    129-256 and 257-512 rows, the 256 x 256 tile of the vocabulary projection at 193-512 rows) and of the few-row
+    kernel (up to 48 rows on at most 4096 columns, 32 rows up to 8192 columns, 8 rows of the long K; 16-row MFMA tiles
+    that end inside the batch): first, last and sampled rows against the dequantised float64 product, every column of
+    those rows.  The same product left as partial sums for the norm that follows (the long K in two parts on up to 32
+    rows) must give the same bound."""
     g = torch.Generator().manual_seed(k + n)
     weight = (torch.randn(n, k, generator=g) * 0.02).bfloat16().to(DEV)
     packed = ops.PackedFP8Weight.from_weight(weight)
@@ -66,9 +72,14 @@ def test_fp8_projection_at_row_counts_where_the_tile_plan_changes(ops, k, n, row
         rows = torch.unique(torch.cat((torch.tensor([0, m - 1, m // 2, min(m - 1, 127), min(m - 1, 128), min(m - 1, 255), min(m - 1, 256)]),
                                        torch.randperm(m, generator=g)[:9]))).to(DEV)
         want = (xq[rows].float() * xs[rows, None]).double() @ wq.T
-        error = (out[rows].double() - want).abs()
         bound = 2 ** -8 * want.abs() + 1e-3 * want.abs().max()
-        assert bool((error <= bound).all()), f"M={m}: {int((error > bound).sum())} entries off, worst {float((error - bound).max()):.3e}"
+        deferred = packed.linear_quantized(xq, xs, defer_reduce=True)
+        if isinstance(deferred, ops.SplitProduct):
+            assert deferred.partials.shape[1:] == (m, n)
+            deferred = deferred.materialize()
+        for product in (out, deferred):
+            error = (product[rows].double() - want).abs()
+            assert bool((error <= bound).all()), f"M={m}: {int((error > bound).sum())} entries off, worst {float((error - bound).max()):.3e}"
 
 
 # ------------------------------------------------------------------------------------------------ config 3

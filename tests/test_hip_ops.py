@@ -226,7 +226,7 @@ def test_bf16_linear_matches_fp32_matmul_of_the_same_operands(ops, m, k, n):
 
 
 @pytest.mark.parametrize("fp8", [True, False])
-@pytest.mark.parametrize("m,k,n", [(48, 512, 1000), (200, 2048, 4096), (7, 100, 72)])
+@pytest.mark.parametrize("m,k,n", [(48, 512, 1000), (200, 2048, 4096), (7, 100, 72), (40, 512, 1024), (9, 1024, 2048)])
 @torch.inference_mode()
 def test_placed_rows_equal_the_product_followed_by_scatter_logits(ops, fp8, m, k, n):
     """The placing GEMMs against the plain product + `scatter_logits` (lfm25_batching.py:25-32): bit-identical live
@@ -1158,18 +1158,22 @@ def test_sampler_that_records_its_draw_equals_sample_then_record(ops):
 
 
 @pytest.mark.parametrize("fp8", (True, False))
-@pytest.mark.parametrize("m,k,inner", [(4096, 256, 512), (2689, 2048, 5632), (1000, 384, 5632), (300, 2048, 5632), (256, 2048, 5632), (200, 2048, 5632), (64, 2048, 5632)])
+@pytest.mark.parametrize("m,k,inner", [(4096, 256, 512), (2689, 2048, 5632), (1000, 384, 5632), (300, 2048, 5632), (256, 2048, 5632), (200, 2048, 5632), (64, 2048, 5632),
+                                       (1, 2048, 1024), (13, 2048, 1024), (40, 1024, 2048), (30, 2048, 3072), (33, 2048, 3072), (49, 2048, 1024)])
 @torch.inference_mode()
 def test_gate_up_projection_with_swiglu_epilogue_equals_the_two_launches(ops, fp8, m, k, inner):
     """The fused gate+up projection (SwiGLU in the product's epilogue, [M, I] written) against the projection followed
-    by the SwiGLU launch, bit for bit: both quantised outputs for W8A8, the bf16 rows otherwise.  The last shape has no
-    fused form and must take the two launches by itself; ragged row counts end inside a tile; 256 and 200 rows run
-    the decode batch's 128 x 96 tile (three MFMA tiles per wave: the odd one is finished by half of the lanes)."""
+    by the SwiGLU launch, bit for bit: both quantised outputs for W8A8, the bf16 rows otherwise.  64 rows of the model's
+    width have no fused form and must take the two launches by themselves; ragged row counts end inside a tile; 256 and
+    200 rows run the decode batch's 128 x 96 tile (three MFMA tiles per wave: the odd one is finished by half of the
+    lanes); the W8A8 products of up to 48 rows on at most 4096 columns (32 rows up to 8192) run the few-row kernel,
+    whose SwiGLU form pairs the gate and up columns out of LDS."""
     torch.manual_seed(m + inner)
     weight = (torch.randn(2 * inner, k, device=DEV) * 0.05).bfloat16()
     x = torch.randn(m, k, device=DEV).bfloat16()
     fused_exists = bool(ops.query("lfm2_gemm_swiglu_fits", m, 2 * inner, k, 1 if fp8 else 2))
-    assert fused_exists == (m > 64)
+    few_rows = fp8 and m <= (48 if 2 * inner <= 4096 else 32 if 2 * inner <= 8192 else 0)
+    assert fused_exists == (m > 64 or few_rows)
     if fp8:
         packed = ops.PackedFP8Weight.from_weight(weight)
         xq, xs = ops.quantize_rows(x)
