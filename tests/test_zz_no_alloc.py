@@ -26,9 +26,13 @@ def test_static_scratch_sampler_equals_the_allocating_one_on_two_calls_in_a_row(
         logprobs = torch.full((logits.size(0),), float("nan"), device="cuda", dtype=torch.float32)
         torch.cuda.synchronize()
         before = torch.cuda.memory_stats()["allocation.all.allocated"]
+        free_before = torch.cuda.mem_get_info()[0]
         ops.sample_logits_static(logits, tokens, logprobs, temperature=temperature, seed=11, step=number)
         torch.cuda.synchronize()
         assert torch.cuda.memory_stats()["allocation.all.allocated"] == before    # nothing came from torch's allocator
+        # nor from the driver: a hipMalloc inside the library would lower the device's free bytes (the first call of the
+        # process looks the array's address up, which allocates nothing either: the array is part of the code object)
+        assert torch.cuda.mem_get_info()[0] >= free_before
         assert torch.equal(tokens, want_tokens)
         assert torch.equal(logprobs.view(torch.int32), want_logprobs.view(torch.int32))
 
@@ -43,3 +47,12 @@ def test_static_scratch_sampler_refuses_what_does_not_fit():
     assert status == -1 and b"static scratch holds 16384" in lib.lfm2_last_error()
     with pytest.raises(ValueError, match="static scratch"):
         ops.call("lfm2_sample_static", tokens, None, logits, None, None, None, 0, 0, 1.0, 16385, 8, 0)
+    # the Python mirror checks the caller's outputs before the raw pointers reach the kernels
+    with pytest.raises(ValueError, match="tokens"):
+        ops.sample_logits_static(logits, tokens.int(), None, temperature=1.0, seed=0, step=0)
+    with pytest.raises(ValueError, match="tokens"):
+        ops.sample_logits_static(logits, tokens[:1], None, temperature=1.0, seed=0, step=0)
+    with pytest.raises(ValueError, match="logprobs"):
+        ops.sample_logits_static(logits, tokens, torch.zeros(2, device="cuda", dtype=torch.float64), temperature=1.0, seed=0, step=0)
+    with pytest.raises(ValueError, match="nonnegative temperature"):
+        ops.sample_logits_static(logits, tokens, None, temperature=-1.0, seed=0, step=0)
