@@ -954,6 +954,29 @@ Plan default_plan(int64_t M, int64_t N, int64_t Kb, bool deferred = false, int e
   // halves the activation bytes a CU pulls (M 256: 48.8 us against 60.0; M 512: 79.4 against 103.9; up to 128 rows the
   // 128x128 tile stays ahead, 37.6 against 43.9).
   if (M > 192 && M <= 512 && N >= 32768 && N % 256 == 0 && Kb % kStepBytes == 0 && steps <= 32) return {58, 1};
+  // Prefill-sized e4m3 products (more than 512 rows, at least a round of 128x128 tiles): the 128x128 tile of 8 waves
+  // (two workgroups per CU), the 256x128 tile of 16 waves or the 256x256 tile of 16 waves (one per CU), whichever
+  // finishes its rounds over the 256 CUs first.  A round's time goes with the tile's area (times the workgroups that
+  // share a CU); against the 128x128 tile at equal rounds the 256x128 tile is 7 % faster and the 256x256 tile 27 %
+  // (its waves read a third fewer LDS bytes per MFMA: 64x64 wave tiles instead of 64x32).  Measured, weights streaming,
+  // us at 4096 / 3400 / 2688 rows for the three tiles: N 11264 147 / 137 / 115, 123 / 115 / 108, 103 / 94 / 78; N 6144
+  // 78 / 71 / 75, 67 / 68 / 70, 51 / 64 / 69; N 3072 45 / 45 / 37, 38 / 42 / 36, 26 / 41 / 36; N 2048 K 5632 58 / 49 / 70,
+  // 53 / 48 / 70, 48 / 45 / 70: the model picks the fastest of each triple, and at 640-2304 rows the fastest or one within
+  // 2 % of it (N 11264: 128x128 at 640 rows, 256x256 at 768-1280 and 2304, 256x128 at 1536-2048).
+  if (eb == 1 && M > 512 && Kb % kStepBytes == 0 && count(6) >= 256) {
+    auto cost = [&](int t, int per_cu, double speed) {
+      const int64_t rounds = (count(t) + 256 * per_cu - 1) / (256 * per_cu);
+      return (double)rounds * kTiles[t].bm * kTiles[t].bn * per_cu / speed;
+    };
+    // a last round of 128x128 tiles that leaves every CU at most one workgroup takes three quarters of a full one
+    // (2048 rows, N 2048: 19.7 us for 256 tiles, 26.1 us for the 512 tiles of 4096 rows)
+    const int64_t rest14 = count(14) % 512;
+    const double c14 = cost(14, 2, 1.0) - (rest14 > 0 && rest14 <= 256 ? 0.5 * 128 * 128 : 0.0);
+    const double c56 = cost(56, 1, 1.07), c58 = cost(58, 1, 1.27);
+    if (c58 < c14 && c58 <= c56) return {58, 1};
+    if (c56 < c14) return {56, 1};
+    return {14, 1};
+  }
   if (count(6) >= 256) return {14, 1};                // 128x128, ring of 2
   if (count(2) >= 512) return {13, 1};                // 64x64, ring of 3
   // one round of 64x64 tiles over the 256 CUs beats two rounds of 32x64 (512 rows, N 2048: K 5632 16.8 us against
@@ -1121,7 +1144,7 @@ namespace {
 bool swiglu_fits(int64_t M, int64_t N, int64_t Kb, int eb) {
   if (M <= 0 || N <= 0 || Kb <= 0 || N % 16 != 0 || Kb % kStepBytes != 0 || M >= (1 << 30) || N >= (1 << 30)) return false;
   const Plan plan = default_plan(M, N, Kb, false, eb);
-  return (plan.tile == 14 || plan.tile == 36 || plan.tile == 56 || plan.tile == kSkinnyTile) && plan.splits == 1;
+  return (plan.tile == 14 || plan.tile == 36 || plan.tile == 56 || plan.tile == 58 || plan.tile == kSkinnyTile) && plan.splits == 1;
 }
 template <int EB>
 int swiglu_entry(const char* name, void* out, const void* a, const float* as, const void* w, const float* ws, int64_t M,
@@ -1143,6 +1166,9 @@ int swiglu_entry(const char* name, void* out, const void* a, const float* as, co
                        (const uint8_t*)a, (const uint8_t*)w, as, ws, (int)M, (int)N, K * EB, out_dtype);
   else if (tile == 56)
     hipLaunchKernelGGL((gemm_swiglu_kernel<EB, 256, 128, 4, 4, 3>), grid, dim3(1024), 0, (hipStream_t)stream, out,
+                       (const uint8_t*)a, (const uint8_t*)w, as, ws, (int)M, (int)N, K * EB, out_dtype);
+  else if (tile == 58)
+    hipLaunchKernelGGL((gemm_swiglu_kernel<EB, 256, 256, 4, 4, 2>), grid, dim3(1024), 0, (hipStream_t)stream, out,
                        (const uint8_t*)a, (const uint8_t*)w, as, ws, (int)M, (int)N, K * EB, out_dtype);
   else
     hipLaunchKernelGGL((gemm_swiglu_kernel<EB, 128, 96, 8, 2, 3>), grid, dim3(1024), 0, (hipStream_t)stream, out,

@@ -51,14 +51,18 @@ def test_fp8_projection_at_benchmark_shapes_matches_dequantised_product_on_sampl
                                             (2048, 65536, (192, 193, 256, 300, 512, 513)),
                                             (2048, 2048, (1, 15, 16, 17, 31, 33, 48, 49, 64)),
                                             (2048, 3072, (2, 16, 47, 48, 49)), (2048, 6144, (1, 16, 17, 32, 33)),
-                                            (5632, 2048, (1, 8, 9, 16, 32, 33))])
+                                            (5632, 2048, (1, 8, 9, 16, 32, 33)),
+                                            (2048, 11264, (640, 1000, 2000, 2689)), (2048, 6144, (1000, 2688, 4001)),
+                                            (2048, 3072, (2000, 2688, 3401)), (2048, 2048, (2048, 4096)),
+                                            (5632, 2048, (2048, 2700))])
 @torch.inference_mode()
 def test_fp8_projection_at_row_counts_where_the_tile_plan_changes(ops, k, n, row_counts):
     """Ragged row counts on either side of every rule of the default plan for the wide projections (one tile per CU at
     129-256 and 257-512 rows, the 256 x 256 tile of the vocabulary projection at 193-512 rows) and of the few-row
     kernel (up to 48 rows on at most 4096 columns, 32 rows up to 8192 columns, 8 rows of the long K; 16-row MFMA tiles
-    that end inside the batch): first, last and sampled rows against the dequantised float64 product, every column of
-    those rows.  The same product left as partial sums for the norm that follows (the long K in two parts on up to 32
+    that end inside the batch), and prefill-sized row counts at which the plan takes each of its three big tiles
+    (128 x 128, 256 x 128, 256 x 256: whichever finishes its rounds over the CUs first), with row counts that end inside
+    a tile: first, last and sampled rows against the dequantised float64 product, every column of those rows.  The same product left as partial sums for the norm that follows (the long K in two parts on up to 32
     rows) must give the same bound."""
     g = torch.Generator().manual_seed(k + n)
     weight = (torch.randn(n, k, generator=g) * 0.02).bfloat16().to(DEV)
