@@ -57,6 +57,8 @@ def parse_args():
     p.add_argument("--plain-launches", action="store_true",
                    help="gemm workload: launch every product directly instead of replaying a graph, the fused MLP variants "
                         "left out, and one 256 MiB copy for counter calibration at the end (for `rocprofv3 --pmc` runs)")
+    p.add_argument("--adaptive-batching", action="store_true",
+                   help="compact graphs (16, 32, 64 ... rows) for a batch that has thinned out, as the reference's switch of that name")
     p.add_argument("--requests", type=int, default=1024, help="requests of the serve workload")
     p.add_argument("--output-low", type=int, default=64, help="serve workload: shortest output, tokens")
     p.add_argument("--output-high", type=int, default=256, help="serve workload: longest output, tokens")
@@ -362,7 +364,8 @@ def serve_workload(args):
                    "admissions": admissions, "polls": polls, "decode_steps": steps,
                    "prompt_plus_output_tok_per_s": round((generated + sum(map(len, prompts))) / elapsed, 1),
                    "mean_compute_rows_per_step": round(stats["decode_row_steps"] / max(steps, 1), 1),
-                   "slot_refills": stats["slot_refills"]},
+                   "slot_refills": stats["slot_refills"], "adaptive_batching": bool(args.adaptive_batching),
+                   "steps_by_compute_rows": dict(stats["decode_batches"])},
         "roofline": None, "cpu_baseline": None}))
 
 
@@ -375,7 +378,8 @@ def build_engine(args, state):
                      layer_types=LFM2_1P2B["layer_types"], max_position_embeddings=128000)
     engine = LFM25Engine.from_state_dict(cfg, state, device="cuda", dtype=torch.bfloat16, max_model_len=args.max_model_len)
     fp8 = args.precision == "fp8"
-    engine.enable_cuda_graphs(max_graphs=1, max_prefill_tokens=4096, fp8_mlp=fp8, fp8_kv=fp8, fp8_lm_head=fp8, fp8_operators=fp8)
+    engine.enable_cuda_graphs(max_graphs=1, max_prefill_tokens=4096, fp8_mlp=fp8, fp8_kv=fp8, fp8_lm_head=fp8, fp8_operators=fp8,
+                              adaptive_batching=args.adaptive_batching)
     return engine, cfg
 
 
