@@ -813,7 +813,7 @@ gemm_skinny_kernel(void* __restrict__ out, const uint8_t* __restrict__ A, const 
 // K).  `parts` > 1: the product is left as that many partial sums along K (one workgroup row per part).
 constexpr int kSkinnyTile = 60;
 struct SkinnyShape { int mi, ni, waves, maxs, per_part; };
-bool skinny_shape(int64_t M, int64_t N, int64_t Kb, int parts, SkinnyShape* shape) {
+bool skinny_shape(int64_t M, int64_t N, int64_t Kb, int parts, SkinnyShape* shape, bool wide = true) {
   if (M <= 0 || M > 64 || N <= 0 || N % 16 != 0 || Kb % kStepBytes != 0 || Kb < kStepBytes || parts < 1) return false;
   const int steps = (int)(Kb / kStepBytes), mi = (int)((M + 15) / 16);
   if (steps < parts) return false;
@@ -831,7 +831,7 @@ bool skinny_shape(int64_t M, int64_t N, int64_t Kb, int parts, SkinnyShape* shap
   // wide outputs on few rows: several column tiles per workgroup, while at least 128 workgroups remain (every workgroup
   // reads all of the activations, so fewer of them re-read less)
   int ni = 1;
-  if (parts == 1 && waves == 8 && mi <= 2) ni = N % 64 == 0 && N / 64 >= 128 ? 4 : N % 32 == 0 && N / 32 >= 128 ? 2 : 1;
+  if (wide && parts == 1 && waves == 8 && mi <= 2) ni = N % 64 == 0 && N / 64 >= 128 ? 4 : N % 32 == 0 && N / 32 >= 128 ? 2 : 1;
   // registers a lane holds in flight: 8 per weight fragment and 8 per activation fragment of every step
   if (maxs * (8 * ni + 8 * mi) + 4 * mi * ni > (waves == 16 ? 104 : 200)) return false;
   if (shape) *shape = SkinnyShape{mi, ni, waves, maxs, per_part};
@@ -842,7 +842,7 @@ template <int EPI>
 bool launch_skinny(void* out, const uint8_t* A, const uint8_t* W, const float* as, const float* ws, int64_t M, int64_t N,
                    int64_t Kb, int parts, int out_dtype, RowMap rows, hipStream_t s) {
   SkinnyShape shape;
-  if (!skinny_shape(M, N, Kb, parts, &shape)) return false;
+  if (!skinny_shape(M, N, Kb, parts, &shape, EPI != 4)) return false;   // partial sums: one column tile per workgroup
   const dim3 grid((unsigned)(N / (16 * shape.ni)), (unsigned)parts);
 #define SKINNY_(MI, NI, WAVES, MAXS)                                                                                    \
   if (shape.mi == MI && shape.ni == NI && shape.waves == WAVES && shape.maxs == MAXS) {                                 \

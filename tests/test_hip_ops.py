@@ -225,6 +225,30 @@ def test_bf16_linear_matches_fp32_matmul_of_the_same_operands(ops, m, k, n):
         torch.testing.assert_close(got.float().cpu(), expected, atol=2e-3, rtol=2 ** -7)
 
 
+@pytest.mark.parametrize("m,k,n,parts", [(16, 2048, 8192, 1), (16, 2048, 2048, 1), (24, 5632, 2048, 2), (300, 2048, 2048, 1),
+                                         (300, 5632, 2048, 4)])
+@torch.inference_mode()
+def test_fp8_partial_sums_through_the_c_abi_add_up_to_the_product(ops, m, k, n, parts):
+    """`lfm2_fp8_gemm_partials` asked for a given number of parts of K, one included (a single fp32 plane: on few rows of
+    a wide output the few-row kernel, which then keeps one column tile per workgroup): the planes, summed in order and
+    scaled, round to the product `lfm2_fp8_gemm` stores."""
+    g = torch.Generator().manual_seed(m + n + parts)
+    packed = ops.PackedFP8Weight.from_weight((torch.randn(n, k, generator=g) * 0.03).bfloat16().to(DEV))
+    xq, xs = ops.quantize_rows(torch.randn(m, k, generator=g).bfloat16().to(DEV))
+    partials = torch.full((parts, m, n), float("nan"), device=DEV, dtype=torch.float32)
+    ops.call("lfm2_fp8_gemm_partials", partials, xq, packed.values, m, n, k, -1, parts)
+    total = partials[0].clone()
+    for part in partials[1:]:
+        total += part
+    got = ((total * xs[:, None]) * packed.scales[None, :]).bfloat16()
+    want = packed.linear_quantized(xq, xs)
+    # the product itself may sum its K steps in another order than the parts do (other tile, other split): one bf16 step
+    exact = packed.linear_quantized(xq, xs, config=(-1, parts)) if parts > 1 else want
+    assert bool(torch.isfinite(partials).all())
+    torch.testing.assert_close(got.float(), exact.float(), atol=2e-3, rtol=2 ** -7)
+    torch.testing.assert_close(got.float(), want.float(), atol=2e-3, rtol=2 ** -7)
+
+
 @pytest.mark.parametrize("fp8", [True, False])
 @pytest.mark.parametrize("m,k,n", [(48, 512, 1000), (200, 2048, 4096), (7, 100, 72), (40, 512, 1024), (9, 1024, 2048)])
 @torch.inference_mode()
