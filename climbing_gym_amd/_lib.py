@@ -35,6 +35,7 @@ _SIGNATURES = {
     "lfm2_rms_norm_split": "ppp" "i" "pppp" "llfip",
     "lfm2_prepare_qkv": "ppppppppp" "liiilfip",
     "lfm2_conv_prefill": "ppppppp" "llllip",
+    "lfm2_conv_prefill_fp8": "pppppppp" "llllip",
     "lfm2_fp8_gemm": "pppppp" "llliiip",
     "lfm2_bf16_gemm": "pppp" "llliip",
     "lfm2_fp8_gemm_rows": "ppppppp" "lllliip",

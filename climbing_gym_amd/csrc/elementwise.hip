@@ -578,60 +578,88 @@ conv_prefill_kernel(T* out, T* state, const T* bcx, const T* w, const int32_t* c
 
 // The same for H % 8 == 0 with 16-byte accesses: a thread owns 8 channels of 4 consecutive tokens, so the products
 // B.x of the six tokens its window touches are formed once (the scalar form reads ten 2-byte values per output).
-template <typename T>
+// FP8 (H <= 2048: one workgroup holds whole rows): the rows leave as e4m3 codes with one scale per token, the bits
+// `quantize_rows` makes of the rows the plain form stores, for an out projection that takes quantised activations.
+template <typename T, bool FP8>
 __global__ void __launch_bounds__(256)
-conv_prefill_vec_kernel(T* out, T* state, const T* bcx, const T* w, const int32_t* cu, const int32_t* seq_of_token,
-                        const int32_t* slots, int64_t H, int64_t T_) {
+conv_prefill_vec_kernel(T* out, uint8_t* q, float* scales, T* state, const T* bcx, const T* w, const int32_t* cu,
+                        const int32_t* seq_of_token, const int32_t* slots, int64_t H, int64_t T_) {
   typedef T vec8 __attribute__((ext_vector_type(8)));
   constexpr int TOK = 4;
+  __shared__ float red[4][TOK];
   const int64_t t0 = (int64_t)blockIdx.y * TOK;
   const int64_t col = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
-  if (col >= H) return;
-  float bx[TOK + 2][8];
+  const bool owns = col < H;
+  if (!FP8 && !owns) return;
+  float y[TOK][8], amax[TOK];
 #pragma unroll
-  for (int i = 0; i < TOK + 2; ++i) {
-    const int64_t tok = t0 - 2 + i;
-    if (tok >= 0 && tok < T_) {
-      const T* in = bcx + tok * 3 * H + col;
-      const vec8 bv = *reinterpret_cast<const vec8*>(in), xv = *reinterpret_cast<const vec8*>(in + 2 * H);
+  for (int j = 0; j < TOK; ++j) amax[j] = 0.f;
+  if (owns) {
+    float bx[TOK + 2][8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) bx[i][e] = round_to<T>(Elem<T>::load(bv[e]) * Elem<T>::load(xv[e]));
-    } else {
+    for (int i = 0; i < TOK + 2; ++i) {
+      const int64_t tok = t0 - 2 + i;
+      if (tok >= 0 && tok < T_) {
+        const T* in = bcx + tok * 3 * H + col;
+        const vec8 bv = *reinterpret_cast<const vec8*>(in), xv = *reinterpret_cast<const vec8*>(in + 2 * H);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) bx[i][e] = 0.f;
+        for (int e = 0; e < 8; ++e) bx[i][e] = round_to<T>(Elem<T>::load(bv[e]) * Elem<T>::load(xv[e]));
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) bx[i][e] = 0.f;
+      }
     }
-  }
-  float taps[24];   // w[col .. col+7][0..2]
+    float taps[24];   // w[col .. col+7][0..2]
 #pragma unroll
-  for (int i = 0; i < 3; ++i) {
-    const vec8 wv = *reinterpret_cast<const vec8*>(w + col * 3 + 8 * i);
+    for (int i = 0; i < 3; ++i) {
+      const vec8 wv = *reinterpret_cast<const vec8*>(w + col * 3 + 8 * i);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) taps[8 * i + e] = Elem<T>::load(wv[e]);
-  }
-#pragma unroll
-  for (int j = 0; j < TOK; ++j) {
-    const int64_t t = t0 + j;
-    if (t >= T_) break;
-    const int seq = seq_of_token[t];
-    const int64_t begin = cu[seq], end = cu[seq + 1];
-    const bool has1 = t - 1 >= begin, has2 = t - 2 >= begin;
-    const vec8 cv = *reinterpret_cast<const vec8*>(bcx + t * 3 * H + H + col);
-    vec8 ov;
-    float x0[8], x1[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      x0[e] = has2 ? bx[j][e] : 0.f;
-      x1[e] = has1 ? bx[j + 1][e] : 0.f;
-      const float conv = round_to<T>(fmaf(bx[j + 2][e], taps[3 * e + 2], fmaf(x1[e], taps[3 * e + 1], x0[e] * taps[3 * e])));
-      ov[e] = Elem<T>::store(Elem<T>::load(cv[e]) * conv);
+      for (int e = 0; e < 8; ++e) taps[8 * i + e] = Elem<T>::load(wv[e]);
     }
-    *reinterpret_cast<vec8*>(out + t * H + col) = ov;
-    if (t == end - 1) {
-      T* st = state + ((int64_t)slots[seq] * H + col) * 3;
+#pragma unroll
+    for (int j = 0; j < TOK; ++j) {
+      const int64_t t = t0 + j;
+      if (t >= T_) break;
+      const int seq = seq_of_token[t];
+      const int64_t begin = cu[seq], end = cu[seq + 1];
+      const bool has1 = t - 1 >= begin, has2 = t - 2 >= begin;
+      const vec8 cv = *reinterpret_cast<const vec8*>(bcx + t * 3 * H + H + col);
+      vec8 ov;
+      float x0[8], x1[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        st[3 * e] = Elem<T>::store(x0[e]); st[3 * e + 1] = Elem<T>::store(x1[e]); st[3 * e + 2] = Elem<T>::store(bx[j + 2][e]);
+        x0[e] = has2 ? bx[j][e] : 0.f;
+        x1[e] = has1 ? bx[j + 1][e] : 0.f;
+        const float conv = round_to<T>(fmaf(bx[j + 2][e], taps[3 * e + 2], fmaf(x1[e], taps[3 * e + 1], x0[e] * taps[3 * e])));
+        ov[e] = Elem<T>::store(Elem<T>::load(cv[e]) * conv);
+        if (FP8) { y[j][e] = Elem<T>::load(ov[e]); amax[j] = fmaxf(amax[j], fabsf(y[j][e])); }
       }
+      if (!FP8) *reinterpret_cast<vec8*>(out + t * H + col) = ov;
+      if (t == end - 1) {
+        T* st = state + ((int64_t)slots[seq] * H + col) * 3;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          st[3 * e] = Elem<T>::store(x0[e]); st[3 * e + 1] = Elem<T>::store(x1[e]); st[3 * e + 2] = Elem<T>::store(bx[j + 2][e]);
+        }
+      }
+    }
+  }
+  if constexpr (FP8) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int j = 0; j < TOK; ++j) {
+      const float m = wave_max(amax[j]);
+      if (lane == 0) red[wave][j] = m;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < TOK; ++j) {
+      const int64_t t = t0 + j;
+      if (t >= T_) break;
+      const float m = fmaxf(fmaxf(red[0][j], red[1][j]), fmaxf(red[2][j], red[3][j]));
+      const float scale = fmaxf(m / LFM2_E4M3_MAX, 1.0e-12f);
+      if (threadIdx.x == 0) scales[t] = scale;
+      if (owns) store_e4m3<8>(q + t * H + col, y[j], scale);
     }
   }
 }
@@ -644,16 +672,36 @@ extern "C" int lfm2_conv_prefill(void* out, void* state, const void* bcx, const 
   if (H % 8 == 0 && dtype != LFM2_DTYPE_F32 && (((uintptr_t)out | (uintptr_t)bcx | (uintptr_t)weight) & 15) == 0) {
     const dim3 grid(ceil_div(H, 2048), ceil_div(T_, 4));
     if (dtype == LFM2_DTYPE_BF16)
-      hipLaunchKernelGGL(conv_prefill_vec_kernel<__bf16>, grid, dim3(256), 0, (hipStream_t)stream, (__bf16*)out, (__bf16*)state,
+      hipLaunchKernelGGL((conv_prefill_vec_kernel<__bf16, false>), grid, dim3(256), 0, (hipStream_t)stream, (__bf16*)out, nullptr, nullptr, (__bf16*)state,
                          (const __bf16*)bcx, (const __bf16*)weight, cu_seqlens, seq_of_token, slots, H, T_);
     else
-      hipLaunchKernelGGL(conv_prefill_vec_kernel<_Float16>, grid, dim3(256), 0, (hipStream_t)stream, (_Float16*)out,
-                         (_Float16*)state, (const _Float16*)bcx, (const _Float16*)weight, cu_seqlens, seq_of_token, slots, H, T_);
+      hipLaunchKernelGGL((conv_prefill_vec_kernel<_Float16, false>), grid, dim3(256), 0, (hipStream_t)stream, (_Float16*)out,
+                         nullptr, nullptr, (_Float16*)state, (const _Float16*)bcx, (const _Float16*)weight, cu_seqlens, seq_of_token, slots, H, T_);
     LFM2_LAUNCH_CHECK();
   }
   DISPATCH_DTYPE(dtype, hipLaunchKernelGGL(conv_prefill_kernel<T>, dim3(ceil_div(H, kThreads), T_), dim3(kThreads), 0,
                                            (hipStream_t)stream, (T*)out, (T*)state, (const T*)bcx, (const T*)weight,
                                            cu_seqlens, seq_of_token, slots, H));
+  LFM2_LAUNCH_CHECK();
+}
+
+// The packed-prefill short conv with its rows quantised for a W8A8 out projection: `lfm2_conv_prefill` followed by
+// `lfm2_quantize_rows`, the same bits, in one launch.  A workgroup must hold whole rows: H <= 2048, H % 8 == 0, 16-bit dtype.
+extern "C" int lfm2_conv_prefill_fp8(uint8_t* q, float* scales, void* state, const void* bcx, const void* weight,
+                                     const int32_t* cu_seqlens, const int32_t* seq_of_token, const int32_t* slots, int64_t T_,
+                                     int64_t nseq, int64_t H, int64_t nslots, int dtype, void* stream) {
+  LFM2_REQUIRE(T_ > 0 && nseq > 0 && H > 0 && nslots > 0, "conv_prefill_fp8: empty shape");
+  LFM2_REQUIRE(T_ <= 4 * 65535, "conv_prefill_fp8: more than 262140 packed tokens in one call");
+  LFM2_REQUIRE(H % 8 == 0 && H <= 2048, "conv_prefill_fp8: width %ld is not a multiple of 8 up to 2048", (long)H);
+  LFM2_REQUIRE(dtype == LFM2_DTYPE_BF16 || dtype == LFM2_DTYPE_F16, "conv_prefill_fp8: 16-bit activations only");
+  LFM2_REQUIRE((((uintptr_t)q & 7) | (((uintptr_t)bcx | (uintptr_t)weight) & 15)) == 0, "conv_prefill_fp8: misaligned buffer");
+  const dim3 grid(1, ceil_div(T_, 4));
+  if (dtype == LFM2_DTYPE_BF16)
+    hipLaunchKernelGGL((conv_prefill_vec_kernel<__bf16, true>), grid, dim3(256), 0, (hipStream_t)stream, (__bf16*)nullptr, q, scales,
+                       (__bf16*)state, (const __bf16*)bcx, (const __bf16*)weight, cu_seqlens, seq_of_token, slots, H, T_);
+  else
+    hipLaunchKernelGGL((conv_prefill_vec_kernel<_Float16, true>), grid, dim3(256), 0, (hipStream_t)stream, (_Float16*)nullptr, q,
+                       scales, (_Float16*)state, (const _Float16*)bcx, (const _Float16*)weight, cu_seqlens, seq_of_token, slots, H, T_);
   LFM2_LAUNCH_CHECK();
 }
 

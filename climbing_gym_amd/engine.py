@@ -445,7 +445,9 @@ class LFM25Engine:
             return ops.prefill_attention(q, k, v, cu, longest, self._scaling).view(total, -1)
 
         def conv_op(op, bcx):
-            return ops.conv_prefill(bcx, op.conv_weight, cache.conv_state[op.cache_index], cu, seq_of_token, slots)
+            # a W8A8 out projection takes the rows quantised: the conv launch does that itself
+            form = ops.conv_prefill_fp8 if id(op.out_weight) in fp8 else ops.conv_prefill
+            return form(bcx, op.conv_weight, cache.conv_state[op.cache_index], cu, seq_of_token, slots)
 
         hidden, residual = self._backbone(tokens, attention_op, conv_op, fp8)
         last = (cu[1:] - 1).long()

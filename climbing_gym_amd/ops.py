@@ -251,6 +251,21 @@ def conv_prefill(bcx, weight, state, cu_seqlens, seq_of_token, slots):
     return out
 
 
+def conv_prefill_fp8(bcx, weight, state, cu_seqlens, seq_of_token, slots):
+    """`quantize_rows(conv_prefill(...))` (lfm25_engine.py:1478-1511, then lfm25_fp8.py:108-117): (e4m3 rows, per-token
+    scales), the same bits, in one launch where a workgroup can hold whole rows (16-bit dtype, width a multiple of 8
+    up to 2048) and in the two launches otherwise."""
+    _check(bcx, weight, state, cu_seqlens, seq_of_token, slots)
+    width = weight.size(0)
+    if width % 8 or width > 2048 or bcx.dtype not in (torch.bfloat16, torch.float16):
+        return quantize_rows(conv_prefill(bcx, weight, state, cu_seqlens, seq_of_token, slots))
+    q = torch.empty((bcx.size(0), width), device=bcx.device, dtype=FP8)
+    scales = torch.empty(bcx.size(0), device=bcx.device, dtype=torch.float32)
+    call("lfm2_conv_prefill_fp8", q, scales, state, bcx, weight, cu_seqlens, seq_of_token, slots, bcx.size(0),
+         cu_seqlens.numel() - 1, width, state.size(0), _code(bcx.dtype))
+    return q, scales
+
+
 # ----------------------------------------------------------------------------------- GEMMs
 @dataclass
 class RowPlacement:

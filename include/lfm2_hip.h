@@ -111,6 +111,13 @@ int lfm2_conv_prefill(void* out, void* state, const void* bcx, const void* weigh
                       const int32_t* seq_of_token, const int32_t* slots, int64_t T, int64_t nseq, int64_t H,
                       int64_t nslots, int dtype, void* stream);
 
+/* lfm2_conv_prefill followed by lfm2_quantize_rows (lfm25_fp8.py:108-117) in one launch, the same bits: the rows leave
+ * as e4m3 codes q [T,H] with one fp32 scale per token, for an out projection that takes quantised activations
+ * (PackedFP8Weight.linear_quantized, lfm25_fp8.py:141-168).  H % 8 == 0, H <= 2048, 16-bit dtype. */
+int lfm2_conv_prefill_fp8(uint8_t* q, float* scales, void* state, const void* bcx, const void* weight,
+                          const int32_t* cu_seqlens, const int32_t* seq_of_token, const int32_t* slots, int64_t T,
+                          int64_t nseq, int64_t H, int64_t nslots, int dtype, void* stream);
+
 /* ---------------------------------------------------------------- GEMMs */
 
 /* PackedFP8Weight.linear_quantized of lfm25_fp8.py:77-105,141-168:

@@ -592,6 +592,34 @@ def test_varlen_prefill_attention_matches_causal_sdpa(ops, dim, qh, kh, lengths)
         torch.testing.assert_close(got[a:b], want, atol=0.02, rtol=0.02)
 
 
+@pytest.mark.parametrize("H,dtype", [(2048, torch.bfloat16), (136, torch.bfloat16), (512, torch.float16), (2056, torch.bfloat16),
+                                     (100, torch.bfloat16)])
+@torch.inference_mode()
+def test_packed_prefill_conv_with_quantised_rows_equals_the_two_launches(ops, H, dtype):
+    """`conv_prefill_fp8` against `quantize_rows(conv_prefill(...))`, bit for bit: codes, per-token scales and every
+    slot's conv state, on a ragged packed batch whose token count is not a multiple of the four tokens a workgroup
+    takes, with a width below a workgroup's 2048 channels (threads that own no channel still take part in the row
+    maximum) and widths the one-launch form does not cover (the wrapper then runs the two launches itself)."""
+    torch.manual_seed(H)
+    lengths, slots = [1, 2, 7, 3, 41, 9], [4, 0, 2, 5, 1, 6]
+    total = sum(lengths)
+    cu = torch.tensor([0, *torch.tensor(lengths).cumsum(0).tolist()], dtype=torch.int32, device=DEV)
+    bcx = torch.randn(total, 3 * H, device=DEV).to(dtype)
+    bcx[5] = 0                                         # a row of zeros: its scale is the floor, its codes zero
+    w = torch.randn(H, 3, device=DEV).to(dtype)
+    seq, _ = ops.build_token_map(cu, total)
+    dslots = torch.tensor(slots, dtype=torch.int32, device=DEV)
+    state_a = torch.ones(7, H, 3, device=DEV, dtype=dtype)
+    state_b = state_a.clone()
+    want_q, want_s = ops.quantize_rows(ops.conv_prefill(bcx, w, state_a, cu, seq, dslots))
+    got_q, got_s = ops.conv_prefill_fp8(bcx, w, state_b, cu, seq, dslots)
+    assert got_q.shape == (total, H) and got_s.shape == (total,)
+    assert torch.equal(got_s.view(torch.int32), want_s.view(torch.int32))
+    assert torch.equal(got_q.view(torch.uint8), want_q.view(torch.uint8))
+    assert torch.equal(state_b.view(torch.int16), state_a.view(torch.int16))
+    assert float(got_s[5]) == pytest.approx(1.0e-12) and int((got_q[5].view(torch.uint8) & 0x7F).max()) == 0   # +0 or -0
+
+
 @pytest.mark.parametrize("H", [128, 100])     # 16-byte accesses, 8 channels x 4 tokens per thread; scalar form
 @torch.inference_mode()
 def test_packed_prefill_conv_and_kv_store_match_per_sequence_oracle(ops, H):
