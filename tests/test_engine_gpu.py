@@ -245,6 +245,39 @@ def test_chunked_prefill_preserves_ragged_prompts_and_reuses_cache(budget, fp8_k
     torch.testing.assert_close(unchunked.next_token_logits, buffer, atol=1e-2, rtol=0)
 
 
+@pytest.mark.parametrize("fp8_kv", (False, True))
+@torch.inference_mode()
+def test_prefill_chunks_of_prompts_that_are_not_neighbours_fill_the_same_slots(fp8_kv):
+    """Prompt lengths 4, 3, 4, 3, 2, 2 under a budget of 6 tokens: five contiguous chunks, but three when the chunks are
+    (4, 2), (4, 2), (3, 3).  The engine takes the three; every prompt must still land in its own slot and row of the
+    logits (given slots, not in order), with the lengths and token ids of the returned prefix as the caller gave them."""
+    engine, ocfg, state = _engine()
+    prompts = [[1, 2, 3, 4], [5, 6, 7], [8, 9, 10, 11], [12, 13, 14], [15, 16], [17, 18]]
+    slots = [6, 0, 3, 5, 1, 4]
+    oracle = O.OracleEngine(ocfg, state, torch.float32, 256)
+    ocache, ologits = oracle.prefill(prompts, cap=64)
+    destination = engine._empty_cache(max_slots=7, max_seq_len=64, fp8_kv=fp8_kv)
+    buffer = torch.zeros((7, 257), device=DEV, dtype=torch.bfloat16)
+    flat, cu, longest = _flat(prompts)
+    actual = engine.prefill(flat, cu, longest, cache=destination, max_prefill_tokens=6, logits_buffer=buffer, slots=slots)
+    assert engine.last_prefill["chunks"] == 3
+    assert actual.prompt_lengths.tolist() == [4, 3, 4, 3, 2, 2] and torch.equal(actual.input_ids.cpu(), flat.cpu().long())
+    assert destination.seq_lens.tolist() == [3, 2, 0, 4, 2, 3, 4]
+    torch.testing.assert_close(buffer[slots].float().cpu(), ologits, atol=2e-2, rtol=0)
+    assert not buffer[2].any()                                         # the slot nobody asked for keeps its row
+    torch.testing.assert_close(destination.conv_state[:, slots].float().cpu(), ocache.conv, atol=2e-3, rtol=2e-2)
+    where = torch.tensor(slots, device=DEV)
+    for step in range(2):
+        got = engine._append_decode_tokens(destination, where, where + 40 + step)
+        want = oracle.append_tokens(ocache, torch.arange(6), torch.tensor(slots) + 40 + step)
+        torch.testing.assert_close(got.float().cpu(), want, atol=3e-2 if fp8_kv else 2e-2, rtol=0)
+    # one chunk for all of them gives the same logits up to GEMM tiling
+    whole = torch.zeros_like(buffer)
+    engine.prefill(flat, cu, longest, cache=engine._empty_cache(max_slots=7, max_seq_len=64, fp8_kv=fp8_kv), logits_buffer=whole, slots=slots)
+    assert engine.last_prefill["chunks"] == 1
+    torch.testing.assert_close(whole, buffer, atol=1e-2, rtol=0)
+
+
 @torch.inference_mode()
 def test_prefill_argument_errors_match_the_reference_contract():
     engine, _, _ = _engine()
