@@ -862,7 +862,7 @@ bool launch_skinny(void* out, const uint8_t* A, const uint8_t* W, const float* a
 }
 
 struct TileInfo { int bm, bn, ks; };
-constexpr int kNumTiles = 61;
+constexpr int kNumTiles = 62;
 constexpr TileInfo kTiles[kNumTiles] = {{16, 64, 128}, {32, 64, 128}, {64, 64, 128}, {128, 64, 128}, {128, 128, 128},
                                         {64, 128, 128}, {128, 128, 128}, {64, 128, 128}, {128, 64, 128},
                                         {16, 64, 256}, {32, 64, 256}, {64, 64, 256},
@@ -879,7 +879,8 @@ constexpr TileInfo kTiles[kNumTiles] = {{16, 64, 128}, {32, 64, 128}, {64, 64, 1
                                         {256, 48, 128}, {256, 48, 128}, {256, 32, 128}, {256, 64, 128}, {256, 48, 128},
                                         {256, 32, 128},
                                         {256, 128, 128}, {128, 256, 128}, {256, 256, 128}, {128, 128, 128},
-                                        {64, 16, 128}};   // 60: the few-row kernel (all rows, 16 columns)
+                                        {64, 16, 128},   // 60: the few-row kernel (all rows, 16 columns)
+                                        {256, 192, 128}};
 int64_t tile_steps(int tile, int64_t Kb) { return (Kb + kTiles[tile].ks - 1) / kTiles[tile].ks; }
 
 struct Plan { int tile, splits; };
@@ -889,7 +890,7 @@ struct Plan { int tile, splits; };
 // once it alone fills the 256 CUs (1.3-2.0 PFLOP/s at M = 4096; 42 us for the 65536-row head at M = 256), otherwise
 // smaller tiles with deeper rings the fewer workgroups a CU gets (its K loop is then a serial chain that nothing
 // overlaps).  With K bytes not a multiple of the step these indices run their register-staged twins.
-Plan default_plan(int64_t M, int64_t N, int64_t Kb, bool deferred = false, int eb = 2) {
+Plan default_plan(int64_t M, int64_t N, int64_t Kb, bool deferred = false, int eb = 2, bool fused = false) {
   if (eb == 1 && skinny_shape(M, N, Kb, 1, nullptr)) {
     // a long K on a narrow output whose partial sums the next norm adds up anyway (the down projection of a small decode
     // batch: 44 steps on 128 column tiles): two parts of K, 256 workgroups
@@ -973,6 +974,11 @@ Plan default_plan(int64_t M, int64_t N, int64_t Kb, bool deferred = false, int e
     const int64_t rest14 = count(14) % 512;
     const double c14 = cost(14, 2, 1.0) - (rest14 > 0 && rest14 <= 256 ? 0.5 * 128 * 128 : 0.0);
     const double c56 = cost(56, 1, 1.07), c58 = cost(58, 1, 1.27);
+    // and a 256x192 tile of 16 waves (64x48 wave tiles, speed 1.15) for the widths it cuts into whole rounds: N 3072 at
+    // 4096 rows is one round of 256 tiles (32 us against 37 on 192 tiles of 256x256), N 6144 two rounds (65 against 70
+    // on three rounds of 256x128).  The product alone: the fused SwiGLU form has no such tile.
+    const double c61 = fused ? 1e30 : cost(61, 1, 1.15);
+    if (c61 < c14 && c61 < c56 && c61 < c58) return {61, 1};
     if (c58 < c14 && c58 <= c56) return {58, 1};
     if (c56 < c14) return {56, 1};
     return {14, 1};
@@ -1121,6 +1127,7 @@ int gemm_entry(const char* name, void* out, const void* a, const float* as, cons
     TILE_(57, 128, 256, 2, 4, 128, 3);
     TILE_(58, 256, 256, 4, 4, 128, 2);
     TILE_(59, 128, 128, 2, 4, 128, 3);
+    TILE_(61, 256, 192, 4, 4, 128, 2);
   }
 #undef TILE_
   if (plan.splits > 1 && reduce)
@@ -1143,7 +1150,7 @@ namespace {
 // The fused form exists for the tile the default plan takes at large M; other shapes use the two launches.
 bool swiglu_fits(int64_t M, int64_t N, int64_t Kb, int eb) {
   if (M <= 0 || N <= 0 || Kb <= 0 || N % 16 != 0 || Kb % kStepBytes != 0 || M >= (1 << 30) || N >= (1 << 30)) return false;
-  const Plan plan = default_plan(M, N, Kb, false, eb);
+  const Plan plan = default_plan(M, N, Kb, false, eb, true);
   return (plan.tile == 14 || plan.tile == 36 || plan.tile == 56 || plan.tile == 58 || plan.tile == kSkinnyTile) && plan.splits == 1;
 }
 template <int EB>
@@ -1153,7 +1160,7 @@ int swiglu_entry(const char* name, void* out, const void* a, const float* as, co
   LFM2_REQUIRE(out_dtype >= LFM2_DTYPE_BF16 && out_dtype <= LFM2_DTYPE_F32, "%s: bad output dtype", name);
   LFM2_REQUIRE(((uintptr_t)a | (uintptr_t)w | (uintptr_t)out) % 16 == 0, "%s: pointers must be aligned to 16 bytes", name);
   if (!swiglu_fits(M, N, K * EB, EB)) LFM2_FAIL(LFM2_ERR_UNSUPPORTED, "%s: no fused form for M %ld, N %ld, K %ld", name, (long)M, (long)N, (long)K);
-  const int tile = default_plan(M, N, K * EB, false, EB).tile;
+  const int tile = default_plan(M, N, K * EB, false, EB, true).tile;
   if (tile == kSkinnyTile) {
     launch_skinny<2>(out, (const uint8_t*)a, (const uint8_t*)w, as, ws, M, N, K * EB, 1, out_dtype,
                      RowMap{nullptr, nullptr, 0x7fffffff}, (hipStream_t)stream);
