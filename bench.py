@@ -46,12 +46,13 @@ def parse_args():
                    help="second timed point: the same batch with every context this many tokens longer (0 = skip)")
     p.add_argument("--top-k", type=int, default=0, help="top-k filter of the sampler (0: full support)")
     p.add_argument("--top-p", type=float, default=1.0, help="top-p filter of the sampler (1: off)")
-    p.add_argument("--workload", choices=("decode", "attention", "gemm", "prefill", "serve", "hbm-ceiling"), default="decode",
+    p.add_argument("--workload", choices=("decode", "attention", "gemm", "prefill", "serve", "hbm-ceiling", "mfma-ceiling"), default="decode",
                    help="decode: the model's decode step (the headline metric); attention: the decode-attention call alone "
                         "on 256 sequences of U[128, 8192] history tokens, dense and paged (block 16), e4m3 and bf16; "
                         "gemm: the W8A8 projection shapes at 1..4096 rows; prefill: causal varlen attention over a packed "
                         "4096-token chunk; serve: --requests requests through one session with continuous admit/retire; "
-                        "hbm-ceiling: the loads-only streaming read (every CU reading, 8 GiB per launch)")
+                        "hbm-ceiling: the loads-only streaming read (every CU reading, 8 GiB per launch); mfma-ceiling: the "
+                        "register-operand fp8 MFMA loop (every SIMD multiplying, no memory traffic)")
     p.add_argument("--rows", type=str, default="1,8,64,256,1024,4096", help="gemm workload: row counts, comma separated")
     p.add_argument("--shapes", type=str, default="w13,conv_in,qkv,out,w2", help="gemm workload: projection shapes to run")
     p.add_argument("--plain-launches", action="store_true",
@@ -154,8 +155,10 @@ def gemm_workload(args):
         torch.cuda.empty_cache()
     if args.plain_launches:
         calibration_copy()
-    big = table.get("w13 n11264 k2048 m4096") or max(table.values(), key=lambda r: r["TFLOPs"])
-    small = table.get("w13 n11264 k2048 m256") or max(table.values(), key=lambda r: r["GBps"])
+    products = [r for r in table.values() if "GBps" in r]
+    big = table.get("w13 n11264 k2048 m4096") or max(products, key=lambda r: r["TFLOPs"])
+    small = table.get("w13 n11264 k2048 m256") or max(products, key=lambda r: r["GBps"])
+    mfma_peak, mfma_details = measure_mfma_peak(repeats=2)
     print(json.dumps({
         "metric": "W8A8 FP8 GEMM, gate+up projection (N 11264, K 2048) at 4096 rows", "value": big["TFLOPs"],
         "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": 1, "ms_per_step": round(big["us"] / 1000, 4),
@@ -164,8 +167,12 @@ def gemm_workload(args):
         "config": {"workload": f"W8A8 products of the LFM2.5-1.2B projection shapes {args.shapes} at {args.rows} rows, "
                                "per-token and per-channel scales, weights streamed from HBM",
                    "worst_relative_error": round(worst, 6), "shapes": table},
-        "roofline": {"kernel": "gemm_nt_kernel (128x128 ring tile) at 4096 rows", "bound": "mfma", "achieved": big["TFLOPs"],
+        "roofline": {"kernel": "gemm_nt_kernel on the tile of the default plan (256x256 of sixteen waves for the gate+up product "
+                               "at 4096 rows)", "bound": "mfma", "achieved": big["TFLOPs"],
                      "peak": 5000.0, "unit": "TFLOP/s", "frac": round(big["TFLOPs"] / 5000.0, 4), "traffic": None,
+                     "measured_peak": {"TFLOPs": mfma_peak, "by_occupancy": mfma_details,
+                                       "what": "register-operand loop of v_mfma_f32_16x16x128_f8f6f4 on every SIMD (lfm2_mfma_fp8_peak)"},
+                     "frac_of_measured_peak": round(big["TFLOPs"] / mfma_peak, 4),
                      "decode_rows_256": {"bound": "hbm", "achieved": small["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                          "frac": round(small["GBps"] / HBM_PEAK_GBS, 4)}},
         "cpu_baseline": None}))
@@ -502,6 +509,51 @@ def measure_hbm_ceiling(gib=8, repeats=3):
     return max(rates.values()), rates
 
 
+def measure_mfma_peak(iterations=20000, repeats=3):
+    """TFLOP/s of the register-operand loop of v_mfma_f32_16x16x128_f8f6f4 (`lfm2_mfma_fp8_peak`) with one, two and four
+    waves per SIMD on all 256 CUs, HIP events around `repeats` launches of each, and the core clock the loop ran at (its
+    cycle counter against the constant-rate clock, median over the workgroups).  Returns (best, details)."""
+    from climbing_gym_amd import ops
+    props = torch.cuda.get_device_properties(0)
+    cus = props.multi_processor_count
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    stream = torch.cuda.current_stream()
+    tick_hz = ops.timestamp_rate_hz()
+    details = {}
+    for waves in (4, 8, 16):
+        sink = torch.empty(cus * waves * 64, device="cuda", dtype=torch.float32)
+        clock = torch.zeros(2 * cus, device="cuda", dtype=torch.int64)
+        flops = ops.mfma_fp8_peak(sink, clock, workgroups=cus, waves=waves, iterations=iterations)
+        torch.cuda.synchronize()
+        begin.record(stream)
+        for _ in range(repeats):
+            ops.mfma_fp8_peak(sink, clock, workgroups=cus, waves=waves, iterations=iterations)
+        end.record(stream)
+        end.synchronize()
+        pairs = clock.view(cus, 2).double().cpu()
+        ghz = float((pairs[:, 0] / pairs[:, 1].clamp_min(1)).median()) * tick_hz / 1e9
+        if not bool(torch.isfinite(sink).all()) or float(sink.abs().max()) == 0.0:
+            raise SystemExit("the MFMA loop left no finite result")
+        details[f"{waves // 4}_waves_per_simd"] = {"TFLOPs": round(flops * repeats / (begin.elapsed_time(end) / 1000) / 1e12, 1),
+                                                   "core_clock_GHz": round(ghz, 3)}
+    best = max(v["TFLOPs"] for v in details.values())
+    return best, details
+
+
+def mfma_ceiling_workload(args):
+    """What the matrix units deliver with nothing else in the way: the figure the prefill products are held against."""
+    best, details = measure_mfma_peak(repeats=max(args.steps, 3))
+    print(json.dumps({
+        "metric": "dense fp8 MFMA rate, register operands only", "value": best, "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": max(args.steps, 3), "warmup": 1, "ms_per_step": None, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "fp8_e4m3 (fp32 accumulate)", "data": "synthetic",
+        "config": {"workload": "mfma_fp8_peak_kernel: one workgroup per CU, 20000 rounds of eight independent "
+                               "v_mfma_f32_16x16x128_f8f6f4 per wave, no memory traffic in the loop", "by_occupancy": details},
+        "roofline": {"kernel": "mfma_fp8_peak_kernel", "bound": "mfma", "achieved": best, "peak": 5000.0, "unit": "TFLOP/s",
+                     "frac": round(best / 5000.0, 4), "traffic": None},
+        "cpu_baseline": None}))
+
+
 def ceiling_workload(args):
     """The chip's streaming read rate as this library can measure it: every CU issuing 16-byte loads, nothing else."""
     best, rates = measure_hbm_ceiling(gib=8, repeats=max(args.steps, 3))
@@ -574,8 +626,10 @@ def time_gemms(engine, rows=256, prefill_rows=4096, repeats=5):
         n, k = packs[0].values.shape
         sec = run(packs[:4], prefill_rows)
         tflops = 2 * prefill_rows * n * k / sec / 1e12
+        peak, _ = measure_mfma_peak(repeats=2)
         out["prefill"] = {"name": "w13", "n": n, "k": k, "us": round(sec * 1e6, 1), "TFLOPs": round(tflops, 1),
-                          "mfma_fp8_frac_of_5PF": round(tflops / 5000, 4)}
+                          "mfma_fp8_frac_of_5PF": round(tflops / 5000, 4), "measured_mfma_peak_TFLOPs": peak,
+                          "mfma_fp8_frac_of_measured_peak": round(tflops / peak, 4)}
     return out
 
 
@@ -650,7 +704,7 @@ def main():
     if args.workload != "decode":
         with torch.inference_mode():
             {"attention": attention_workload, "gemm": gemm_workload, "prefill": prefill_workload,
-             "serve": serve_workload, "hbm-ceiling": ceiling_workload}[args.workload](args)
+             "serve": serve_workload, "hbm-ceiling": ceiling_workload, "mfma-ceiling": mfma_ceiling_workload}[args.workload](args)
         return
     from climbing_gym_amd.config import LFM25SamplingConfig
     from climbing_gym_amd.synthetic import LFM2_1P2B, random_prompts, random_state_dict

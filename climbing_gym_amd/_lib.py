@@ -64,6 +64,7 @@ _SIGNATURES = {
     "lfm2_sample_record": "pppppppppppppppppppp" "llllip",
     "lfm2_record_head": "pppppp" "illp",
     "lfm2_hbm_stream_read": "plpiip",
+    "lfm2_mfma_fp8_peak": "ppiiip",
     "lfm2_timestamp": "pp",
 }
 _INT64_RESULT = {

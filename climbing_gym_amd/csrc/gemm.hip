@@ -1334,3 +1334,52 @@ extern "C" int64_t lfm2_bf16_gemm_workspace(int64_t M, int64_t N, int64_t K) {
   const Plan p = default_plan(M, N, K * 2);
   return ((K * 2) % 16 == 0 && p.splits > 1) ? (int64_t)p.splits * M * N : 0;
 }
+
+// ------------------------------------------------------------------------------------ MFMA peak probe
+// What the matrix units deliver when nothing else is in the way: every wave issues `iterations` rounds of eight
+// independent v_mfma_f32_16x16x128_f8f6f4 (e4m3 operands held in registers, eight accumulators, so no instruction
+// waits for the one before it).  No memory traffic inside the loop; the accumulators are folded into one store per
+// lane at the end so the loop cannot be dropped.  The measured peak that the prefill products' MFMA utilisation is
+// held against next to the nominal 5.0 PFLOP/s.  Also stores the core clock cycles and the 100 MHz wall clock ticks
+// the loop took in the first wave of each workgroup (clock[2 * workgroup], clock[2 * workgroup + 1]): the clock the
+// matrix units run at under this load.
+namespace {
+template <int WAVES>
+__global__ void __launch_bounds__(WAVES * 64)
+mfma_fp8_peak_kernel(float* __restrict__ sink, int64_t* __restrict__ clock, int iterations) {
+  typedef StepMfma<1>::frag frag;
+  const int lane = threadIdx.x & 63;
+  frag a, b;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {   // e4m3 codes of small finite values (exponent field 6 or 7): no infinities, no NaNs
+    a[e] = 0x30303030 + 0x01010101 * ((lane + e) & 7);
+    b[e] = 0x38383838 + 0x01010101 * ((lane * 3 + e) & 7);
+  }
+  f32x4 acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int64_t c0 = (int64_t)clock64(), w0 = (int64_t)wall_clock64();
+  for (int it = 0; it < iterations; ++it) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = StepMfma<1>::run(a, b, acc[i]);
+  }
+  const int64_t c1 = (int64_t)clock64(), w1 = (int64_t)wall_clock64();
+  f32x4 total = acc[0];
+#pragma unroll
+  for (int i = 1; i < 8; ++i) total += acc[i];
+  sink[(int64_t)blockIdx.x * (WAVES * 64) + threadIdx.x] = total[0] + total[1] + total[2] + total[3];
+  if (threadIdx.x == 0 && clock) { clock[2 * blockIdx.x] = c1 - c0; clock[2 * blockIdx.x + 1] = w1 - w0; }
+}
+}  // namespace
+
+extern "C" int lfm2_mfma_fp8_peak(float* sink, int64_t* clock, int workgroups, int waves, int iterations, void* stream) {
+  LFM2_REQUIRE(sink != nullptr, "mfma_fp8_peak: null sink");
+  LFM2_REQUIRE(workgroups > 0 && workgroups <= 65536, "mfma_fp8_peak: workgroups %d not in [1, 65536]", workgroups);
+  LFM2_REQUIRE(waves == 4 || waves == 8 || waves == 16, "mfma_fp8_peak: %d waves per workgroup, not 4, 8 or 16", waves);
+  LFM2_REQUIRE(iterations > 0 && iterations <= (1 << 24), "mfma_fp8_peak: iterations %d not in [1, 2^24]", iterations);
+  hipStream_t s = (hipStream_t)stream;
+  if (waves == 4) hipLaunchKernelGGL(mfma_fp8_peak_kernel<4>, dim3(workgroups), dim3(256), 0, s, sink, clock, iterations);
+  else if (waves == 8) hipLaunchKernelGGL(mfma_fp8_peak_kernel<8>, dim3(workgroups), dim3(512), 0, s, sink, clock, iterations);
+  else hipLaunchKernelGGL(mfma_fp8_peak_kernel<16>, dim3(workgroups), dim3(1024), 0, s, sink, clock, iterations);
+  LFM2_LAUNCH_CHECK();
+}

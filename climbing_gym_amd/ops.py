@@ -702,6 +702,17 @@ def hbm_stream_read(buffer: torch.Tensor, sink: torch.Tensor, *, workgroups: int
     return (size // 4096 // workgroups) * workgroups * 4096
 
 
+def mfma_fp8_peak(sink: torch.Tensor, clock, *, workgroups: int, waves: int, iterations: int) -> int:
+    """Launch the register-operand fp8 MFMA loop (`lfm2_mfma_fp8_peak`); returns the flops of the launch.  `sink` is a
+    float32 tensor of at least workgroups * waves * 64 entries, `clock` None or an int64 tensor of 2 * workgroups."""
+    reject(not sink.is_cuda or sink.dtype != torch.float32 or sink.numel() < workgroups * waves * 64,
+           "mfma_fp8_peak needs a float32 GPU sink of workgroups * waves * 64")
+    reject(clock is not None and (not clock.is_cuda or clock.dtype != torch.int64 or clock.numel() < 2 * workgroups),
+           "mfma_fp8_peak's clock output is an int64 GPU tensor of 2 * workgroups")
+    call("lfm2_mfma_fp8_peak", sink, clock, int(workgroups), int(waves), int(iterations))
+    return workgroups * waves * iterations * 8 * (2 * 16 * 16 * 128)
+
+
 def timestamp(out: torch.Tensor) -> None:
     """Store the device wall clock into the int64 element `out` points at, in stream order (`lfm2_timestamp`)."""
     reject(not out.is_cuda or out.dtype != torch.int64 or out.numel() < 1, "timestamp needs an int64 GPU element")

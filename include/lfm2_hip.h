@@ -359,6 +359,14 @@ int lfm2_record_head(const int64_t* ids, const float* probs, int32_t* out_ids, f
  * sink: int32[workgroups * 256], receives one folded word per lane.  Bytes read = workgroups * that many blocks * 4096. */
 int lfm2_hbm_stream_read(const void* src, int64_t bytes, int32_t* sink, int workgroups, int layout, void* stream);
 
+/* Register-operand loop of v_mfma_f32_16x16x128_f8f6f4 (e4m3): every wave of `workgroups` x `waves` (4, 8 or 16) issues
+ * `iterations` rounds of eight independent instructions, 8 x 65536 flop each per round.  The dense fp8 rate the matrix
+ * units deliver with nothing else in the way, which bench.py reports as the measured peak next to the nominal
+ * 5.0 PFLOP/s when it gives the prefill products' MFMA utilisation.  No counterpart in the reference.
+ * sink: float[workgroups * waves * 64]; clock: int64[2 * workgroups] or NULL, receives per workgroup the core clock
+ * cycles and the constant-rate (lfm2_timestamp_rate_khz) ticks its first wave spent in the loop. */
+int lfm2_mfma_fp8_peak(float* sink, int64_t* clock, int workgroups, int waves, int iterations, void* stream);
+
 /* Stores the device's constant-rate wall clock into out[0] from a one-lane kernel; lfm2_timestamp_rate_khz() is the
  * clock's rate (0 if it cannot be read).  Recorded into a graph before and after a kernel, two stamps give that
  * kernel's time inside the replayed graph, which is how bench.py reads the decode-attention call's time inside the

@@ -1275,3 +1275,68 @@ def test_conv_in_projection_with_conv_update_epilogue_equals_the_two_launches(op
     assert torch.equal(got[live].view(torch.int16), want[live].view(torch.int16))
     assert torch.equal(got_state.view(torch.int16), want_state.view(torch.int16))
     assert not torch.equal(got_state, state)
+
+
+# ------------------------------------------------------------------------------------------------ measurement entry points
+@pytest.mark.parametrize("layout", (0, 1))
+@torch.inference_mode()
+def test_streaming_read_folds_every_word_of_its_blocks_exactly_once(ops, layout):
+    """`lfm2_hbm_stream_read` on a small buffer of random words: lane t of workgroup w must end with the XOR of the
+    words of its 16-byte vector in every 4 KiB block the layout gives that workgroup (a private run of blocks, or
+    blocks w, w + grid, ...); the blocks beyond a whole number per workgroup are not read."""
+    groups, blocks = 3, 31                                   # 10 blocks per workgroup, one left over
+    words = torch.randint(-2 ** 31, 2 ** 31 - 1, (blocks * 1024,), dtype=torch.int64).to(torch.int32)
+    sink = torch.full((groups * 256,), 7, device=DEV, dtype=torch.int32)
+    read = ops.hbm_stream_read(words.to(DEV), sink, workgroups=groups, layout=layout)
+    per = blocks // groups
+    assert read == groups * per * 4096
+    grid = words.view(blocks, 256, 4)
+    for w in range(groups):
+        mine = [w + b * groups for b in range(per)] if layout else list(range(w * per, (w + 1) * per))
+        want = torch.zeros(256, dtype=torch.int32)
+        for b in mine:
+            for e in range(4):
+                want ^= grid[b, :, e]
+        assert torch.equal(sink[w * 256:(w + 1) * 256].cpu(), want), (layout, w)
+    with pytest.raises(ValueError, match="fewer than 4096 bytes"):
+        ops.hbm_stream_read(words[:1024].to(DEV), sink, workgroups=groups, layout=layout)
+    with pytest.raises(ValueError, match="int32 sink"):
+        ops.hbm_stream_read(words.to(DEV), sink[:100], workgroups=groups, layout=layout)
+
+
+@torch.inference_mode()
+def test_device_timestamps_follow_stream_order(ops):
+    stamps = torch.zeros(3, device=DEV, dtype=torch.int64)
+    ops.timestamp(stamps[0:1])
+    torch.zeros(1 << 24, device=DEV).add_(1)                 # some work between the stamps
+    ops.timestamp(stamps[1:2])
+    ops.timestamp(stamps[2:3])
+    a, b, c = stamps.cpu().tolist()
+    assert 0 < a < b <= c
+    rate = ops.timestamp_rate_hz()
+    assert 1e6 <= rate <= 1e10 and (b - a) / rate < 1.0      # a plausible clock: the fill took well under a second
+    with pytest.raises(ValueError, match="int64"):
+        ops.timestamp(torch.zeros(1, device=DEV, dtype=torch.int32))
+
+
+@pytest.mark.parametrize("waves", (4, 8, 16))
+@torch.inference_mode()
+def test_mfma_loop_adds_the_same_product_every_round(ops, waves):
+    """`lfm2_mfma_fp8_peak`: the accumulators grow by one fixed e4m3 product per round (small dyadic values: exact in
+    fp32 for a few hundred rounds), so twice the rounds give exactly twice the folded result in every lane, every
+    workgroup computes the same, and the clock output is filled."""
+    groups = 3
+    once = torch.zeros(groups * waves * 64, device=DEV, dtype=torch.float32)
+    twice, clock = torch.zeros_like(once), torch.zeros(2 * groups, device=DEV, dtype=torch.int64)
+    flops = ops.mfma_fp8_peak(once, None, workgroups=groups, waves=waves, iterations=100)
+    assert flops == groups * waves * 100 * 8 * 65536
+    ops.mfma_fp8_peak(twice, clock, workgroups=groups, waves=waves, iterations=200)
+    assert bool((once > 0).all()) and torch.equal(twice, 2 * once)
+    per_group = once.view(groups, -1)
+    assert torch.equal(per_group[0], per_group[1]) and torch.equal(per_group[0], per_group[2])
+    assert torch.equal(per_group[0][:64], per_group[0][64:128])          # every wave holds the same operands
+    assert bool((clock > 0).all())
+    with pytest.raises(ValueError, match="waves per workgroup"):
+        ops.mfma_fp8_peak(once, None, workgroups=groups, waves=2, iterations=10)
+    with pytest.raises(ValueError, match="float32 GPU sink"):
+        ops.mfma_fp8_peak(once[:10], None, workgroups=groups, waves=waves, iterations=10)
