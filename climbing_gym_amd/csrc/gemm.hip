@@ -455,6 +455,20 @@ gemm_nt_body(void* __restrict__ out, float* __restrict__ partial, const uint8_t*
     auto finish_rows = [&](auto tag) {
       typedef decltype(tag) T;
       const int half = lane >> 5, I = N >> 1;
+      // the column scales of this lane's values do not depend on the row: fetched once, before the rows
+      float cs0[(NI + 1) / 2][4], cs1[(NI + 1) / 2][4];
+      if (a_scales) {
+#pragma unroll
+        for (int j = 0; j < NI; j += 2) {
+          const int j1 = j + 1 < NI ? j + 1 : j;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int n0 = n_base + wn * TN + j * 16 + 4 * lgrp + r, n1 = n_base + wn * TN + j1 * 16 + 4 * lgrp + r;
+            cs0[j / 2][r] = w_scales[swiglu_weight_row(n0 < N ? n0 : N - 1, N)];
+            cs1[j / 2][r] = w_scales[swiglu_weight_row(n1 < N ? n1 : N - 1, N)];
+          }
+        }
+      }
 #pragma unroll
       for (int i = 0; i < MI; ++i) {
         const int m = m_base + wm * TM + i * 16 + lrow;
@@ -465,11 +479,10 @@ gemm_nt_body(void* __restrict__ out, float* __restrict__ partial, const uint8_t*
           float first[4], second[4];
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const int n0 = n_base + wn * TN + j * 16 + 4 * lgrp + r, n1 = n_base + wn * TN + j1 * 16 + 4 * lgrp + r;
             float y0 = acc[i][j][r], y1 = acc[i][j1][r];
             if (a_scales) {
-              y0 = (y0 * sa) * w_scales[swiglu_weight_row(n0 < N ? n0 : N - 1, N)];
-              y1 = (y1 * sa) * w_scales[swiglu_weight_row(n1 < N ? n1 : N - 1, N)];
+              y0 = (y0 * sa) * cs0[j / 2][r];
+              y1 = (y1 * sa) * cs1[j / 2][r];
             }
             const unsigned a = __builtin_bit_cast(unsigned, round_to<T>(y0)), b = __builtin_bit_cast(unsigned, round_to<T>(y1));
             const auto swapped = __builtin_amdgcn_permlane32_swap(a, b, false, false);
@@ -563,9 +576,19 @@ gemm_nt_body(void* __restrict__ out, float* __restrict__ partial, const uint8_t*
 
   // Epilogue: lane holds out[m = .. + lrow][n = .. + 4*lgrp + r], r = 0..3.
   const bool split = partial != nullptr;
-  auto finish = [&](f32x4 v, int m_out, int n, float sa) {  // scale (row then column) and store up to 4 columns
+  // the column scales of this lane's values do not depend on the row: fetched once, before the rows
+  float cw[NI][4];
+  if (a_scales && !split) {
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const int n = n_base + wn * TN + j * 16 + 4 * lgrp;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) cw[j][r] = n + r < N ? w_scales[n + r] : 0.f;
+    }
+  }
+  auto finish = [&](f32x4 v, int m_out, int n, float sa, const float* cols) {  // scale (row then column) and store up to 4 columns
     if (a_scales)
-      for (int r = 0; r < 4; ++r) v[r] = (v[r] * sa) * (n + r < N ? w_scales[n + r] : 0.f);
+      for (int r = 0; r < 4; ++r) v[r] = (v[r] * sa) * cols[r];
     const int64_t idx = (int64_t)m_out * N + n;
     if (out_dtype == LFM2_DTYPE_BF16 && n + 3 < N && (N & 3) == 0) {
       bf16x4 o = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
@@ -590,7 +613,7 @@ gemm_nt_body(void* __restrict__ out, float* __restrict__ partial, const uint8_t*
         if (n + 3 < N && (N & 3) == 0) *reinterpret_cast<f32x4*>(dst) = acc[i][j];
         else for (int r = 0; r < 4 && n + r < N; ++r) dst[r] = acc[i][j][r];
       } else {
-        finish(acc[i][j], m_out, n, sa);
+        finish(acc[i][j], m_out, n, sa, cw[j]);
       }
     }
   }

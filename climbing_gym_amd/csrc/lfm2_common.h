@@ -53,8 +53,16 @@ template <> struct Elem<float> {
 template <typename T> __device__ __forceinline__ float round_to(float v) { return Elem<T>::load(Elem<T>::store(v)); }
 
 // SiLU as the SwiGLU kernels compute it (one definition, so that a fused epilogue and the stand-alone kernels give the
-// same bits).
-__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
+// same bits): g / (1 + e^-g) on the hardware's base-2 exponential and reciprocal (v_exp_f32, v_rcp_f32: one unit in
+// the last place each) instead of the library exponential and an IEEE division, which cost a 256x256 tile of the fused
+// gate+up product a tenth of its time.  The relative error is bounded by (3 + max(-g, 0)) 2^-23: the argument g log2(e)
+// is rounded once, which the exponential turns into max(-g, 0) 2^-24 of relative error where e^-g dominates and into
+// nothing where 1 does.  A 16-bit result differs from the exactly rounded one in about one element in ten thousand.
+// Limits: e^-g overflows to infinity for g < -88.7 and the result is -0 (the exact value is below the smallest normal
+// number there); NaN stays NaN.
+__device__ __forceinline__ float silu_f(float g) {
+  return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -LFM2_LOG2E));
+}
 
 // One channel of the gated short conv: taps (state[1], state[2], b*x) with weights w[0..2]; returns c * conv and the
 // new state entry b*x, every product and the tap sum rounded to T as the reference's kernel rounds them.

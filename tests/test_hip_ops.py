@@ -1340,3 +1340,28 @@ def test_mfma_loop_adds_the_same_product_every_round(ops, waves):
         ops.mfma_fp8_peak(once, None, workgroups=groups, waves=2, iterations=10)
     with pytest.raises(ValueError, match="float32 GPU sink"):
         ops.mfma_fp8_peak(once[:10], None, workgroups=groups, waves=waves, iterations=10)
+
+
+@torch.inference_mode()
+def test_silu_of_the_swiglu_kernels_stays_within_its_stated_error(ops):
+    """The SwiGLU kernels compute g / (1 + e^-g) on the hardware's base-2 exponential and reciprocal
+    (lfm25_cuda_kernels.py:58-72 uses the tracing compiler's sigmoid, itself an approximation).  In fp32, against
+    float64: relative error at most (3 + max(-g, 0)) 2^-23 with a factor 1.5 of slack, over gates in [-30, 30]; far
+    below -88 the result is zero, far above it is the gate; in bf16 the rounded result equals the exactly rounded one
+    in all but a few elements in ten thousand."""
+    gen = torch.Generator().manual_seed(3)
+    gate = torch.cat((torch.linspace(-30, 30, 20001), torch.randn(45535, generator=gen) * 4)).float()
+    x = torch.cat((gate, torch.ones_like(gate))).view(1, -1).to(DEV)
+    got = ops.swiglu(x).double().cpu()[0]
+    g = gate.double()
+    want = g / (1 + torch.exp(-g))
+    bound = 1.5 * (3 + (-g).clamp_min(0)) * 2.0 ** -23 * want.abs() + 1e-45
+    assert bool(((got - want).abs() <= bound).all()), float(((got - want).abs() / bound).max())
+    edge = torch.tensor([-200.0, -100.0, 100.0, 0.0, float("nan")])
+    out = ops.swiglu(torch.cat((edge, torch.ones(5))).view(1, -1).to(DEV)).cpu()[0]
+    assert out[:2].abs().max() == 0 and float(out[2]) == 100.0 and float(out[3]) == 0.0 and bool(torch.isnan(out[4]))
+    half = torch.cat((gate, torch.ones_like(gate))).view(1, -1).bfloat16()
+    got16 = ops.swiglu(half.to(DEV)).cpu()[0]
+    g16 = half[0, :gate.numel()].double()
+    exact16 = (g16 / (1 + torch.exp(-g16))).float().bfloat16()
+    assert float((got16 != exact16).float().mean()) < 1e-3
