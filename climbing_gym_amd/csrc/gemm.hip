@@ -913,7 +913,7 @@ struct Plan { int tile, splits; };
 // once it alone fills the 256 CUs (1.3-2.0 PFLOP/s at M = 4096; 42 us for the 65536-row head at M = 256), otherwise
 // smaller tiles with deeper rings the fewer workgroups a CU gets (its K loop is then a serial chain that nothing
 // overlaps).  With K bytes not a multiple of the step these indices run their register-staged twins.
-Plan default_plan(int64_t M, int64_t N, int64_t Kb, bool deferred = false, int eb = 2, bool fused = false) {
+Plan default_plan(int64_t M, int64_t N, int64_t Kb, bool deferred = false, int eb = 2) {
   if (eb == 1 && skinny_shape(M, N, Kb, 1, nullptr)) {
     // a long K on a narrow output whose partial sums the next norm adds up anyway (the down projection of a small decode
     // batch: 44 steps on 128 column tiles): two parts of K, 256 workgroups
@@ -999,8 +999,8 @@ Plan default_plan(int64_t M, int64_t N, int64_t Kb, bool deferred = false, int e
     const double c56 = cost(56, 1, 1.07), c58 = cost(58, 1, 1.27);
     // and a 256x192 tile of 16 waves (64x48 wave tiles, speed 1.15) for the widths it cuts into whole rounds: N 3072 at
     // 4096 rows is one round of 256 tiles (32 us against 37 on 192 tiles of 256x256), N 6144 two rounds (65 against 70
-    // on three rounds of 256x128).  The product alone: the fused SwiGLU form has no such tile.
-    const double c61 = fused ? 1e30 : cost(61, 1, 1.15);
+    // on three rounds of 256x128; N 11264 at 2048 rows two rounds of 472 tiles, 63 us against 71).
+    const double c61 = cost(61, 1, 1.15);
     if (c61 < c14 && c61 < c56 && c61 < c58) return {61, 1};
     if (c58 < c14 && c58 <= c56) return {58, 1};
     if (c56 < c14) return {56, 1};
@@ -1173,8 +1173,9 @@ namespace {
 // The fused form exists for the tile the default plan takes at large M; other shapes use the two launches.
 bool swiglu_fits(int64_t M, int64_t N, int64_t Kb, int eb) {
   if (M <= 0 || N <= 0 || Kb <= 0 || N % 16 != 0 || Kb % kStepBytes != 0 || M >= (1 << 30) || N >= (1 << 30)) return false;
-  const Plan plan = default_plan(M, N, Kb, false, eb, true);
-  return (plan.tile == 14 || plan.tile == 36 || plan.tile == 56 || plan.tile == 58 || plan.tile == kSkinnyTile) && plan.splits == 1;
+  const Plan plan = default_plan(M, N, Kb, false, eb);
+  return (plan.tile == 14 || plan.tile == 36 || plan.tile == 56 || plan.tile == 58 || plan.tile == 61 || plan.tile == kSkinnyTile) &&
+         plan.splits == 1;
 }
 template <int EB>
 int swiglu_entry(const char* name, void* out, const void* a, const float* as, const void* w, const float* ws, int64_t M,
@@ -1183,7 +1184,7 @@ int swiglu_entry(const char* name, void* out, const void* a, const float* as, co
   LFM2_REQUIRE(out_dtype >= LFM2_DTYPE_BF16 && out_dtype <= LFM2_DTYPE_F32, "%s: bad output dtype", name);
   LFM2_REQUIRE(((uintptr_t)a | (uintptr_t)w | (uintptr_t)out) % 16 == 0, "%s: pointers must be aligned to 16 bytes", name);
   if (!swiglu_fits(M, N, K * EB, EB)) LFM2_FAIL(LFM2_ERR_UNSUPPORTED, "%s: no fused form for M %ld, N %ld, K %ld", name, (long)M, (long)N, (long)K);
-  const int tile = default_plan(M, N, K * EB, false, EB, true).tile;
+  const int tile = default_plan(M, N, K * EB, false, EB).tile;
   if (tile == kSkinnyTile) {
     launch_skinny<2>(out, (const uint8_t*)a, (const uint8_t*)w, as, ws, M, N, K * EB, 1, out_dtype,
                      RowMap{nullptr, nullptr, 0x7fffffff}, (hipStream_t)stream);
@@ -1199,6 +1200,9 @@ int swiglu_entry(const char* name, void* out, const void* a, const float* as, co
                        (const uint8_t*)a, (const uint8_t*)w, as, ws, (int)M, (int)N, K * EB, out_dtype);
   else if (tile == 58)
     hipLaunchKernelGGL((gemm_swiglu_kernel<EB, 256, 256, 4, 4, 2>), grid, dim3(1024), 0, (hipStream_t)stream, out,
+                       (const uint8_t*)a, (const uint8_t*)w, as, ws, (int)M, (int)N, K * EB, out_dtype);
+  else if (tile == 61)
+    hipLaunchKernelGGL((gemm_swiglu_kernel<EB, 256, 192, 4, 4, 2>), grid, dim3(1024), 0, (hipStream_t)stream, out,
                        (const uint8_t*)a, (const uint8_t*)w, as, ws, (int)M, (int)N, K * EB, out_dtype);
   else
     hipLaunchKernelGGL((gemm_swiglu_kernel<EB, 128, 96, 8, 2, 3>), grid, dim3(1024), 0, (hipStream_t)stream, out,

@@ -1210,7 +1210,7 @@ def test_sampler_that_records_its_draw_equals_sample_then_record(ops):
 
 
 @pytest.mark.parametrize("fp8", (True, False))
-@pytest.mark.parametrize("m,k,inner", [(4096, 256, 512), (2689, 2048, 5632), (1000, 384, 5632), (300, 2048, 5632), (256, 2048, 5632), (200, 2048, 5632), (64, 2048, 5632),
+@pytest.mark.parametrize("m,k,inner", [(4096, 256, 512), (2689, 2048, 5632), (2000, 2048, 5632), (1030, 512, 5632), (1000, 384, 5632), (300, 2048, 5632), (256, 2048, 5632), (200, 2048, 5632), (64, 2048, 5632),
                                        (1, 2048, 1024), (13, 2048, 1024), (40, 1024, 2048), (30, 2048, 3072), (33, 2048, 3072), (49, 2048, 1024)])
 @torch.inference_mode()
 def test_gate_up_projection_with_swiglu_epilogue_equals_the_two_launches(ops, fp8, m, k, inner):
@@ -1219,7 +1219,8 @@ def test_gate_up_projection_with_swiglu_epilogue_equals_the_two_launches(ops, fp
     width have no fused form and must take the two launches by themselves; ragged row counts end inside a tile; 256 and
     200 rows run the decode batch's 128 x 96 tile (three MFMA tiles per wave: the odd one is finished by half of the
     lanes); the W8A8 products of up to 48 rows on at most 4096 columns (32 rows up to 8192) run the few-row kernel,
-    whose SwiGLU form pairs the gate and up columns out of LDS."""
+    whose SwiGLU form pairs the gate and up columns out of LDS; 2000 and 1030 rows of the model's 11264 columns run the
+    256 x 192 tile (three MFMA tiles per wave again, and a last column tile that ends inside the output)."""
     torch.manual_seed(m + inner)
     weight = (torch.randn(2 * inner, k, device=DEV) * 0.05).bfloat16()
     x = torch.randn(m, k, device=DEV).bfloat16()
