@@ -8,6 +8,8 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <type_traits>
+
 #include "lfm2_common.h"
 
 // ------------------------------------------------------------------------------------ errors
@@ -130,30 +132,58 @@ rms_norm_kernel(T* out, uint8_t* q, float* scales, T* summed, const T* x, const 
   if (FP8) q += row * H; else out += row * H;
 
   if constexpr (NV > 0) {
-    float v[NV][N];
+    float v[NV][N], g[NV][N];
     float ss = 0.f;
+    // Every load of the row is issued before anything waits: the residual, the norm weights, the scales, and the fp32
+    // planes of a product left as partial sums, whose count is spelled out for 1, 2 and 4 planes (a loop with a count
+    // only known at run time waits for each plane before it asks for the next: one more memory round trip per plane,
+    // in a kernel that is little else).  The planes are added in their order either way.
+    const float sa = (split.partial && split.a_scales) ? split.a_scales[row] : 1.0f;   // a bf16 product has no scales
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       const int64_t i = (int64_t)(j * kRowThreads + threadIdx.x) * N;
       if (i < H) {
+        float r[N];
+        if (ADD) load_vec<T>(res + i, r);
+        load_vec<T>(w + i, g[j]);
         if (split.partial) {
-          const float sa = split.a_scales ? split.a_scales[row] : 1.0f;   // a bf16 product has no scales
+          float cs[N];
+          if (split.w_scales) {
 #pragma unroll
-          for (int e = 0; e < N; ++e) v[j][e] = 0.f;
-          for (int sp = 0; sp < split.splits; ++sp) {
-            const float* p = split.partial + sp * split.stride + row * H + i;
+            for (int e = 0; e < N; ++e) cs[e] = split.w_scales[i + e];
+          }
+          const float* p = split.partial + row * H + i;
+          auto planes = [&](auto count) {
+            constexpr int SP = decltype(count)::value;
+            float part[SP][N];
 #pragma unroll
-            for (int e = 0; e < N; ++e) v[j][e] += p[e];
+            for (int sp = 0; sp < SP; ++sp)
+#pragma unroll
+              for (int e = 0; e < N; ++e) part[sp][e] = p[sp * split.stride + e];
+#pragma unroll
+            for (int e = 0; e < N; ++e) v[j][e] = 0.f;
+#pragma unroll
+            for (int sp = 0; sp < SP; ++sp)
+#pragma unroll
+              for (int e = 0; e < N; ++e) v[j][e] += part[sp][e];
+          };
+          if (split.splits == 1) planes(std::integral_constant<int, 1>{});
+          else if (split.splits == 2) planes(std::integral_constant<int, 2>{});
+          else if (split.splits == 4) planes(std::integral_constant<int, 4>{});
+          else {
+#pragma unroll
+            for (int e = 0; e < N; ++e) v[j][e] = 0.f;
+            for (int sp = 0; sp < split.splits; ++sp)
+#pragma unroll
+              for (int e = 0; e < N; ++e) v[j][e] += p[sp * split.stride + e];
           }
 #pragma unroll
-          for (int e = 0; e < N; ++e) v[j][e] = round_to<T>(split.w_scales ? (v[j][e] * sa) * split.w_scales[i + e] : v[j][e]);
+          for (int e = 0; e < N; ++e) v[j][e] = round_to<T>(split.w_scales ? (v[j][e] * sa) * cs[e] : v[j][e]);
         } else {
           load_vec<T>(x + i, v[j]);
           if (gather) store_vec<T>(summed + i, v[j]);
         }
         if (ADD) {
-          float r[N];
-          load_vec<T>(res + i, r);
 #pragma unroll
           for (int e = 0; e < N; ++e) v[j][e] = round_to<T>(v[j][e] + r[e]);
           store_vec<T>(summed + i, v[j]);
@@ -161,13 +191,6 @@ rms_norm_kernel(T* out, uint8_t* q, float* scales, T* summed, const T* x, const 
 #pragma unroll
         for (int e = 0; e < N; ++e) ss += v[j][e] * v[j][e];
       }
-    }
-    // the norm weights do not depend on the reduction: fetch them before it, so the kernel pays one memory round trip
-    float g[NV][N];
-#pragma unroll
-    for (int j = 0; j < NV; ++j) {
-      const int64_t i = (int64_t)(j * kRowThreads + threadIdx.x) * N;
-      if (i < H) load_vec<T>(w + i, g[j]);
     }
     ss = block_sum<kRowWaves>(ss, red);
     const float rstd = 1.0f / sqrtf(ss / (float)H + eps);
