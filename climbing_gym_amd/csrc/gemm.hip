@@ -243,6 +243,40 @@ gemm_nt_body(void* __restrict__ out, float* __restrict__ partial, const uint8_t*
     }
   };
 
+  // Small wave tiles (the decode batch's tiles) fetch the scales their epilogue needs here, before the K loop: asked for
+  // at the end they are a memory round trip (the weight's scales come from HBM) in which the workgroup does nothing.
+  // Large wave tiles have no registers to spare for them across the loop and find theirs in L2 anyway.
+  constexpr bool kEarlyScales = (EPI == 0 || EPI == 2) && MI * NI <= 6;
+  constexpr int kColScales = EPI == 2 ? 8 * ((NI + 1) / 2) : 4 * NI;
+  float early_cols[kEarlyScales ? kColScales : 1], early_rows[kEarlyScales ? MI : 1];
+  if constexpr (kEarlyScales) {
+    if (a_scales && partial == nullptr) {
+#pragma unroll
+      for (int i = 0; i < MI; ++i) {
+        const int m = m_base + wm * TM + i * 16 + lrow;
+        early_rows[i] = a_scales[m < M ? m : M - 1];
+      }
+      if constexpr (EPI == 2) {
+#pragma unroll
+        for (int j = 0; j < NI; j += 2) {
+          const int j1 = j + 1 < NI ? j + 1 : j;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int n0 = n_base + wn * TN + j * 16 + 4 * lgrp + r, n1 = n_base + wn * TN + j1 * 16 + 4 * lgrp + r;
+            early_cols[8 * (j / 2) + r] = w_scales[swiglu_weight_row(n0 < N ? n0 : N - 1, N)];
+            early_cols[8 * (j / 2) + 4 + r] = w_scales[swiglu_weight_row(n1 < N ? n1 : N - 1, N)];
+          }
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+          const int n = n_base + wn * TN + j * 16 + 4 * lgrp;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) early_cols[4 * j + r] = n + r < N ? w_scales[n + r] : 0.f;
+        }
+      }
+    }
+  }
   static_assert((EPI != 2 && EPI != 3) || ST > 0, "the fused SwiGLU and conv epilogues are built on the ring tiles");
   if constexpr (ST > 0) {
     static_assert(!KTAIL, "direct-to-LDS loads cannot zero-fill a partial K step");
@@ -463,16 +497,25 @@ gemm_nt_body(void* __restrict__ out, float* __restrict__ partial, const uint8_t*
           const int j1 = j + 1 < NI ? j + 1 : j;
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const int n0 = n_base + wn * TN + j * 16 + 4 * lgrp + r, n1 = n_base + wn * TN + j1 * 16 + 4 * lgrp + r;
-            cs0[j / 2][r] = w_scales[swiglu_weight_row(n0 < N ? n0 : N - 1, N)];
-            cs1[j / 2][r] = w_scales[swiglu_weight_row(n1 < N ? n1 : N - 1, N)];
+            if constexpr (kEarlyScales) {
+              cs0[j / 2][r] = early_cols[8 * (j / 2) + r];
+              cs1[j / 2][r] = early_cols[8 * (j / 2) + 4 + r];
+            } else {
+              const int n0 = n_base + wn * TN + j * 16 + 4 * lgrp + r, n1 = n_base + wn * TN + j1 * 16 + 4 * lgrp + r;
+              cs0[j / 2][r] = w_scales[swiglu_weight_row(n0 < N ? n0 : N - 1, N)];
+              cs1[j / 2][r] = w_scales[swiglu_weight_row(n1 < N ? n1 : N - 1, N)];
+            }
           }
         }
       }
 #pragma unroll
       for (int i = 0; i < MI; ++i) {
         const int m = m_base + wm * TM + i * 16 + lrow;
-        const float sa = a_scales ? a_scales[m < M ? m : M - 1] : 1.0f;
+        float sa = 1.0f;
+        if (a_scales) {
+          if constexpr (kEarlyScales) sa = early_rows[i];
+          else sa = a_scales[m < M ? m : M - 1];
+        }
 #pragma unroll
         for (int j = 0; j < NI; j += 2) {
           const int j1 = j + 1 < NI ? j + 1 : j;
@@ -583,7 +626,10 @@ gemm_nt_body(void* __restrict__ out, float* __restrict__ partial, const uint8_t*
     for (int j = 0; j < NI; ++j) {
       const int n = n_base + wn * TN + j * 16 + 4 * lgrp;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) cw[j][r] = n + r < N ? w_scales[n + r] : 0.f;
+      for (int r = 0; r < 4; ++r) {
+        if constexpr (kEarlyScales) cw[j][r] = early_cols[4 * j + r];
+        else cw[j][r] = n + r < N ? w_scales[n + r] : 0.f;
+      }
     }
   }
   auto finish = [&](f32x4 v, int m_out, int n, float sa, const float* cols) {  // scale (row then column) and store up to 4 columns
@@ -603,7 +649,11 @@ gemm_nt_body(void* __restrict__ out, float* __restrict__ partial, const uint8_t*
     if (m >= M) continue;
     const int m_out = split ? m : mapped_row(rows, m);
     if (m_out < 0) continue;
-    const float sa = (!split && a_scales) ? a_scales[m] : 1.0f;
+    float sa = 1.0f;
+    if (!split && a_scales) {
+      if constexpr (kEarlyScales) sa = early_rows[i];
+      else sa = a_scales[m];
+    }
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
       const int n = n_base + wn * TN + j * 16 + 4 * lgrp;
@@ -738,6 +788,27 @@ gemm_skinny_kernel(void* __restrict__ out, const uint8_t* __restrict__ A, const 
     m = m < M ? m : M - 1;
     ap[i] = A + (int64_t)m * Kb + 32 * lgrp;
   }
+  // the scales of the output item this thread finishes (at most one when the items fit the workgroup), asked for with
+  // the operands: at the end they would be one more memory round trip
+  constexpr bool kOneItem = MI * NI <= WAVES && EPI != 4;
+  float item_row_scale = 1.0f, item_cols[8];
+  if constexpr (kOneItem) {
+    if (tid < MI * NI * 64) {
+      const int tile = tid >> 6, l = tid & 63, m = (tile / NI) * 16 + (l & 15), col = n_base + 16 * (tile % NI) + 4 * (l >> 4);
+      if (m < M && col < N) {
+        item_row_scale = a_scales[m];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          if constexpr (EPI == 2) {
+            item_cols[r] = w_scales[swiglu_weight_row(col + r, N)];
+            item_cols[4 + r] = l < 32 ? w_scales[swiglu_weight_row(col + 8 + r, N)] : 0.f;
+          } else {
+            item_cols[r] = w_scales[col + r];
+          }
+        }
+      }
+    }
+  }
   // every load of the wave, unconditionally (a step beyond the last is the last one again and is not multiplied)
   frag fw[MAXS][NI], fa[MAXS][MI];
 #pragma unroll
@@ -792,7 +863,7 @@ gemm_skinny_kernel(void* __restrict__ out, const uint8_t* __restrict__ A, const 
       *reinterpret_cast<f32x4*>((float*)out + ((int64_t)blockIdx.y * M + m) * N + col) = total(tile, l);
       continue;
     }
-    const float sa = a_scales[m];
+    const float sa = kOneItem ? item_row_scale : a_scales[m];
     if constexpr (EPI == 2) {
       // lane groups 0, 1 hold gate columns 0-7 of a tile, groups 2, 3 (32 lanes on) the up columns that pair with them
       if (l >= 32) continue;
@@ -802,8 +873,10 @@ gemm_skinny_kernel(void* __restrict__ out, const uint8_t* __restrict__ A, const 
         float h[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const float g = round_to<T>((gate[r] * sa) * w_scales[swiglu_weight_row(col + r, N)]);
-          const float u = round_to<T>((up[r] * sa) * w_scales[swiglu_weight_row(col + 8 + r, N)]);
+          const float gs = kOneItem ? item_cols[r] : w_scales[swiglu_weight_row(col + r, N)];
+          const float us = kOneItem ? item_cols[4 + r] : w_scales[swiglu_weight_row(col + 8 + r, N)];
+          const float g = round_to<T>((gate[r] * sa) * gs);
+          const float u = round_to<T>((up[r] * sa) * us);
           h[r] = round_to<T>(round_to<T>(silu_f(g)) * u);
         }
         T* dst = (T*)out + (int64_t)m * (N >> 1) + ((n_base + 16 * j) >> 1) + 4 * grp;
@@ -819,7 +892,7 @@ gemm_skinny_kernel(void* __restrict__ out, const uint8_t* __restrict__ A, const 
     if (m_out < 0) continue;
     f32x4 v = total(tile, l);
 #pragma unroll
-    for (int r = 0; r < 4; ++r) v[r] = (v[r] * sa) * w_scales[col + r];
+    for (int r = 0; r < 4; ++r) v[r] = (v[r] * sa) * (kOneItem ? item_cols[r] : w_scales[col + r]);
     const int64_t idx = (int64_t)m_out * N + col;
     if (out_dtype == LFM2_DTYPE_BF16) {
       bf16x4 o = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
