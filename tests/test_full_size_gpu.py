@@ -62,8 +62,8 @@ def test_fp8_projection_at_row_counts_where_the_tile_plan_changes(ops, k, n, row
     kernel (up to 48 rows on at most 4096 columns, 32 rows up to 8192 columns, 8 rows of the long K; 16-row MFMA tiles
     that end inside the batch), and prefill-sized row counts at which the plan takes each of its three big tiles
     (128 x 128, 256 x 128, 256 x 256: whichever finishes its rounds over the CUs first), with row counts that end inside
-    a tile: first, last and sampled rows against the dequantised float64 product, every column of those rows.  The same product left as partial sums for the norm that follows (the long K in two parts on up to 32
-    rows) must give the same bound."""
+    a tile: first, last and sampled rows against the dequantised float64 product, every column of those rows.  The same product left as partial sums for the norm that follows (the long K in two parts of the
+    few-row kernel on up to 8 rows, in four parts of the tiled kernel above) must give the same bound."""
     g = torch.Generator().manual_seed(k + n)
     weight = (torch.randn(n, k, generator=g) * 0.02).bfloat16().to(DEV)
     packed = ops.PackedFP8Weight.from_weight(weight)
